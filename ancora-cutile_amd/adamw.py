@@ -1,0 +1,194 @@
+"""AdamW with fp32 master weights, fp32 m/v and a bf16 working copy, on the MI355X.
+
+Mirror of ancora/optim/adamw.py: the same `AdamW` class (constructor, `step`,
+`weights`, `master`, `free`, the per-name state dict `st` and the step counter `t`),
+the same low-level launch tuple `_adamw(g, m, v, p32, p16, OTM, beta1, beta2, eps, lr,
+wd, ibc1, ibc2)` with `_pick_otm` and `C`, and the host RNE helpers. The cuda-tile
+kernel is replaced by `anc_adamw` / `anc_adamw_multi` (one launch for the whole
+parameter group instead of one per tensor).
+
+Arithmetic: by default the class evaluates the *divide* form of the reference's numpy
+test oracle (tests/optim/test_adamw.py:37-41) with every scalar rounded to fp32 once on
+the host, so master weights and moments are bit-identical to that oracle;
+`form="ibc"` selects the reference kernel's multiply-by-reciprocal form
+(ancora/optim/adamw.py:34-37), which is what the low-level `_adamw` tuple carries.
+
+Extensions (all off by default): bf16 gradients (uint16 arrays), gradients already
+resident in DevBufs, stochastic-rounded bf16 downcast (`sr=True`, counter-based hash of
+ancora/kernels/fused.py:154-161), and a StepGuard (global clip + skip on non-finite).
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import api, AdamWHyper, AdamWDesc, F32, BF16, FORM_DIV, FORM_IBC
+from .bf16 import bf16_bits as _bf16_bits, bits_f32 as _bits_f32  # noqa: F401  (re-exported)
+from .devbuf import DevBuf, upload_table
+
+C = 64   # every tensor is a flat (numel // 64, 64) view (ancora/optim/adamw.py:20)
+
+
+def _pick_otm(R):
+    """Rows per tile of the reference's launch (ancora/optim/adamw.py:44-48). Kept for callers
+    that build the launch tuple; the HIP kernel walks fixed 4096-element blocks instead."""
+    for cand in (128, 64, 32, 16, 8, 4, 2):
+        if R % cand == 0:
+            return cand
+    return 1
+
+
+def _g_code(dtype):
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return F32
+    if dtype == np.uint16:
+        return BF16
+    raise TypeError(f"gradient dtype {dtype}: expected float32 or uint16 (bf16 bits)")
+
+
+def sr_seed_base(base_seed, t):
+    """Per-step seed of the stochastic downcast; tensor i of a group uses seed_base + i
+    (uint32 wrap-around)."""
+    return (int(base_seed) + 1000003 * int(t)) & 0xFFFFFFFF
+
+
+def hyper_div(lr, b1, b2, eps, t, sr=False, seed_base=0):
+    """Scalars of the numpy-oracle form, each computed in Python double and rounded to fp32
+    once (what numpy's weak-scalar promotion does in tests/optim/test_adamw.py:38-40)."""
+    return AdamWHyper(beta1=b1, beta2=b2, omb1=1 - b1, omb2=1 - b2, eps=eps, lr=lr,
+                      bc1=1 - b1 ** t, bc2=1 - b2 ** t, form=FORM_DIV, sr=int(bool(sr)),
+                      seed_base=seed_base)
+
+
+def hyper_ibc(lr, b1, b2, eps, ibc1, ibc2, sr=False, seed_base=0):
+    """Scalars of the reference kernel form (ancora/optim/adamw.py:34-37, 90-91)."""
+    return AdamWHyper(beta1=b1, beta2=b2, omb1=0.0, omb2=0.0, eps=eps, lr=lr, bc1=ibc1, bc2=ibc2,
+                      form=FORM_IBC, sr=int(bool(sr)), seed_base=seed_base)
+
+
+def _adamw(stream_int, g, m, v, p32, p16, OTM, beta1, beta2, eps, lr, wd, ibc1, ibc2, ctl=0):
+    """The reference's launch `ct.launch(si, (R//OTM,1,1), _adamw, (g, m, v, p32, p16, OTM, ...))`
+    (ancora/optim/adamw.py:94-97; also resident_train.py:350-353, resident_model.py:162-166,
+    kernels/moe.py:586-588) as one call. g/m/v/p32/p16 are DevBufs over the same element count;
+    OTM is accepted and ignored. g may be float32 or uint16 (bf16 bits)."""
+    n = p32.size
+    if n % C:
+        raise ValueError(f"_adamw: numel {n} is not a multiple of {C}")
+    h = hyper_ibc(lr, beta1, beta2, eps, ibc1, ibc2)
+    api.anc_adamw(g.ptr, m.ptr, v.ptr, p32.ptr, p16.ptr, n, _g_code(g.dtype), ctypes.byref(h),
+                  float(wd), 0, int(ctl), int(stream_int))
+
+
+class AdamW:
+    """fp32-master AdamW. params: {name: fp32 ndarray}. no_decay: names with wd=0 (norm gains /
+    biases). step(grads, stream) updates in place; .weights() returns the bf16-valued fp32
+    weights for the forward (ancora/optim/adamw.py:69-109)."""
+
+    def __init__(self, params, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.01, no_decay=(),
+                 form="div", sr=False, seed=0, grad_dtype=np.float32):
+        _lib.init()
+        self.lr, (self.b1, self.b2), self.eps, self.wd = lr, betas, eps, wd
+        if form not in ("div", "ibc"):
+            raise ValueError("form must be 'div' or 'ibc'")
+        self.form, self.sr, self.seed = form, bool(sr), int(seed)
+        self.t = 0
+        self.st = {}
+        gdt = np.dtype(grad_dtype)
+        _g_code(gdt)
+        for name, p in params.items():
+            if p.size % C:
+                # the reference silently truncates (R = p.size // C, adamw.py:79); refuse instead
+                raise ValueError(f"AdamW: '{name}' has {p.size} elements, not a multiple of {C}")
+            R = p.size // C
+            flat = np.ascontiguousarray(p, dtype=np.float32).reshape(R, C)
+            self.st[name] = dict(
+                shape=p.shape, R=R, otm=_pick_otm(R), wd=0.0 if name in no_decay else wd,
+                g=DevBuf.zeros((R, C), gdt),
+                m=DevBuf.zeros((R, C), np.float32), v=DevBuf.zeros((R, C), np.float32),
+                p32=DevBuf(flat), p16=DevBuf.zeros((R, C), np.uint16))
+        self._table = None
+        self._table_key = None
+        self.last_skipped = False
+
+    # -- descriptor table: one row per tensor, rebuilt only when a gradient pointer changes
+    def _build_table(self, gbufs):
+        key = tuple((g.ptr, g.dtype.str) for g in gbufs)
+        if key == self._table_key:
+            return
+        if self._table is not None:
+            self._table.free()
+        descs, blk0 = [], 0
+        for seed, ((name, s), g) in enumerate(zip(self.st.items(), gbufs)):
+            n = s["R"] * C
+            if g.size != n:
+                raise ValueError(f"AdamW: gradient of '{name}' has {g.size} elements, expected {n}")
+            descs.append(AdamWDesc(g.ptr, s["m"].ptr, s["v"].ptr, s["p32"].ptr, s["p16"].ptr, n,
+                                   blk0, s["wd"], seed, _g_code(g.dtype), 0))
+            blk0 += api.anc_adamw_num_blocks(n)
+        self._total_blocks = blk0
+        self._table = upload_table(descs)
+        self._table_key = key
+
+    def _hyper(self):
+        sb = sr_seed_base(self.seed, self.t) if self.sr else 0
+        if self.form == "div":
+            return hyper_div(self.lr, self.b1, self.b2, self.eps, self.t, self.sr, sb)
+        ibc1 = 1.0 / (1.0 - self.b1 ** self.t)
+        ibc2 = 1.0 / (1.0 - self.b2 ** self.t)
+        return hyper_ibc(self.lr, self.b1, self.b2, self.eps, ibc1, ibc2, self.sr, sb)
+
+    def launch(self, grads, stream_int, guard=None):
+        """Asynchronous part of the step: upload host gradients (DevBuf gradients are used in
+        place) and launch the fused kernel once over all tensors. `t` is advanced first, as in
+        ancora/optim/adamw.py:89-91; a caller that later finds the step skipped calls `unstep()`."""
+        self.t += 1
+        gbufs = []
+        for name, s in self.st.items():
+            g = grads[name]
+            if isinstance(g, DevBuf):
+                gbufs.append(g)
+            else:
+                g = np.asarray(g)
+                if g.dtype != s["g"].dtype:
+                    g = g.astype(np.float32) if s["g"].dtype == np.float32 else g
+                    if g.dtype != s["g"].dtype:
+                        raise TypeError(f"AdamW: gradient of '{name}' is {g.dtype}, the optimizer "
+                                        f"was built for {s['g'].dtype}")
+                s["g"].upload(g.reshape(s["R"], C), stream_int)
+                gbufs.append(s["g"])
+        self._build_table(gbufs)
+        h = self._hyper()
+        api.anc_adamw_multi(self._table.ptr, len(self.st), self._total_blocks, ctypes.byref(h),
+                            0 if guard is None else guard.ptr, int(stream_int))
+
+    def unstep(self):
+        """Undo the counter advance of a step the guard skipped (state was left untouched)."""
+        self.t -= 1
+
+    def step(self, grads, stream_int, guard=None):
+        self.launch(grads, stream_int, guard)
+        _lib.stream_sync(stream_int)                       # ancora/optim/adamw.py:98
+        self.last_skipped = False
+        if guard is not None and guard.read(stream_int)["skip"]:
+            self.unstep()
+            self.last_skipped = True
+
+    def weights(self):
+        """bf16-valued fp32 weights (what the forward consumes), per name."""
+        return {n: _bits_f32(s["p16"].numpy()).reshape(s["shape"]) for n, s in self.st.items()}
+
+    def master(self):
+        return {n: s["p32"].numpy().reshape(s["shape"]) for n, s in self.st.items()}
+
+    def moments(self):
+        return {n: (s["m"].numpy().reshape(s["shape"]), s["v"].numpy().reshape(s["shape"]))
+                for n, s in self.st.items()}
+
+    def free(self):
+        for s in self.st.values():
+            for k in ("g", "m", "v", "p32", "p16"):
+                s[k].free()
+        if self._table is not None:
+            self._table.free()
+            self._table = None

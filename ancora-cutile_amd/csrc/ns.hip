@@ -1,0 +1,584 @@
+// Batched Newton-Schulz / Polar-Express chain for gfx950.
+// Replaces `newton_schulz_resident[_e]` and the kernels they launch
+// (ancora/kernels/muon_ns.py:68-174, 245-283, 293-406, 430-468); numpy form
+// ancora/optim/muon.py:67-80 and tests/kernels/_probe_polar_express_device.py:27-34.
+//
+// Per matrix X (M,N), M <= N:  X /= ||X||_F + eps;  steps x { A = X X^T;
+//   B = b A + c A A;  X = a X + B X }.
+//
+// Precision design (bf16 modes). The reference stores X, A and B as bf16 between the
+// GEMMs, which leaves it about 6e-3 (relative Frobenius) from the fp32 numpy result.
+// Here the iterate stays in fp32 in HBM and is rounded to bf16 only as a matrix-core
+// operand, and the diagonals of A and B -- the entries that approach 1 and b+c while the
+// off-diagonal part goes to zero -- never pass through bf16:
+//   A = dA + F    dA = diag(A) kept as an fp32 vector, F = off-diagonal part
+//   A A = dA^2 + dA F + F dA + F F       only F F is a matrix-core product (bf16 F)
+//   B = dB + Boff                        likewise
+//   B X = dB (.) X + Boff X              dB (.) X is an fp32 row scaling in the epilogue
+// In the last two iterations the X operand additionally carries its bf16 residual
+// (X = Xh + Xl): A gets Xh Xl^T + Xl Xh^T and B X gets Boff Xl as extra accumulation
+// terms. All products are "NT" (both operands K-contiguous): X is kept both as (M,N) and
+// transposed (N,M) bf16 copies, written by the epilogue that produces it.
+//
+// Determinism: one workgroup owns one 128x128 output tile and its whole K loop, terms in
+// a fixed order, K tiles in ascending order; no split-K, no atomics. A matrix's result
+// does not depend on the batch size E or on its position in the batch. Symmetric outputs
+// (A, B) compute the tiles on or below the diagonal and mirror them, which is bit-identical
+// to computing both halves (same products, same order).
+//
+// GEMM tile: 128x128x64, 256 lanes = 4 wavefronts in 2x2, each 64x64 as 2x2
+// v_mfma_f32_32x32x16_bf16 blocks (fp32 accumulate). Operand tiles are staged through LDS
+// with a 144-byte row pitch (16-byte fragment reads of 16 consecutive rows hit 64 distinct
+// banks); the next K tile is fetched into registers while the current one is multiplied.
+// Workgroup ids are remapped so that consecutive tiles -- the tiles of one matrix -- run on
+// the same XCD and share its L2.
+#include "reduce.h"
+
+namespace {
+
+using namespace anc_reduce;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int PITCH = BK + 8;            // bf16 elements per LDS row: 144 bytes
+constexpr int kGemmThreads = 256;
+constexpr int kXcds = 8;
+
+enum { EPI_GRAM = 0, EPI_BMAT = 1, EPI_BX = 2 };
+
+// Workgroup id -> logical tile id such that logical ids [start(x), start(x+1)) run on XCD x
+// (hardware deals consecutive workgroup ids round-robin over the 8 XCDs).
+__device__ __forceinline__ int xcd_remap(int bid, int grid) {
+  const int x = bid % kXcds, q = bid / kXcds;
+  const int base = grid / kXcds, rem = grid % kXcds;
+  return x * base + (x < rem ? x : rem) + q;
+}
+
+struct NsGemm {
+  const uint16_t *A[3];      // term t: rows of the output  (tiles_m*128 rows, ld = K)
+  const uint16_t *B[3];      // term t: columns of the output (tiles_n*128 rows, ld = K)
+  int nterms;
+  int K;
+  int64_t strideA, strideB;  // elements between consecutive matrices
+  int tiles_m, tiles_n;
+  int lower;                 // symmetric output: tiles with tn <= tm only, mirrored
+  int M, N;                  // matrix dims of the chain (A, B are MxM; X is MxN)
+  float ca, cb, cc;
+  float *A32;                // (E,M,M) fp32 A            GRAM out, BMAT in
+  uint16_t *Fh;              // (E,M,M) bf16 off-diag A   GRAM out
+  float *dA;                 // (E,M)   diag A            GRAM out, BMAT in
+  uint16_t *Bh;              // (E,M,M) bf16 off-diag B   BMAT out
+  float *dB;                 // (E,M)   diag B            BMAT out, BX in
+  float *X32;                // (E,M,N) fp32 iterate      BX in/out
+  uint16_t *Yh, *YhT;        // next iterate bf16 (M,N) and (N,M); null on the last step
+  uint16_t *Yl, *YlT;        // bf16 residual copies; null unless the next step splits
+};
+
+template <int EPI>
+__global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
+  __shared__ __attribute__((aligned(16))) uint16_t sA[BM * PITCH];
+  __shared__ __attribute__((aligned(16))) uint16_t sB[BN * PITCH];
+
+  const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
+  const int tiles_per = p.lower ? p.tiles_m * (p.tiles_m + 1) / 2 : p.tiles_m * p.tiles_n;
+  const int e = L / tiles_per;
+  const int t = L % tiles_per;
+  int tm, tn;
+  if (p.lower) {
+    tm = 0;
+    while ((tm + 1) * (tm + 2) / 2 <= t) ++tm;
+    tn = t - tm * (tm + 1) / 2;
+  } else {
+    tm = t / p.tiles_n;
+    tn = t % p.tiles_n;
+  }
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lrow = tid >> 3, lk = (tid & 7) * 8;     // loader: 8 lanes per 128-byte row
+  const int K = p.K;
+  const int nk = K / BK;
+  const int total = p.nterms * nk;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[bi][bj][r] = 0.0f;
+
+  anc_u32x4 ra[4], rb[4];
+  auto gload = [&](int step) {
+    const int term = step / nk, kt = step - term * nk;
+    const uint16_t *Ap = p.A[term] + (int64_t)e * p.strideA + (int64_t)(tm * BM + lrow) * K + kt * BK + lk;
+    const uint16_t *Bp = p.B[term] + (int64_t)e * p.strideB + (int64_t)(tn * BN + lrow) * K + kt * BK + lk;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ra[i] = *(const anc_u32x4 *)(Ap + (int64_t)(32 * i) * K);
+      rb[i] = *(const anc_u32x4 *)(Bp + (int64_t)(32 * i) * K);
+    }
+  };
+  auto lstore = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *(anc_u32x4 *)&sA[(lrow + 32 * i) * PITCH + lk] = ra[i];
+      *(anc_u32x4 *)&sB[(lrow + 32 * i) * PITCH + lk] = rb[i];
+    }
+  };
+
+  gload(0);
+  lstore();
+  __syncthreads();
+  const int arow = (wm * 64 + (lane & 31)) * PITCH + (lane >> 5) * 8;
+  const int brow = (wn * 64 + (lane & 31)) * PITCH + (lane >> 5) * 8;
+  for (int step = 0; step < total; ++step) {
+    const bool more = step + 1 < total;
+    if (more) gload(step + 1);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      bf16x8 a[2], b[2];
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi) a[bi] = *(const bf16x8 *)&sA[arow + bi * 32 * PITCH + kk * 16];
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj) b[bj] = *(const bf16x8 *)&sB[brow + bj * 32 * PITCH + kk * 16];
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+          acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[bi], b[bj], acc[bi][bj], 0, 0, 0);
+    }
+    __syncthreads();
+    if (more) {
+      lstore();
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue. Accumulator element r of block (bi,bj) in lane l is
+  //      row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 block.
+  const int M = p.M, N = p.N;
+  const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi) {
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gi = tm * BM + wm * 64 + bi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int gj = tn * BN + wn * 64 + bj * 32 + (lane & 31);
+        const float v = acc[bi][bj][r];
+        if (EPI == EPI_GRAM) {
+          const bool diag = gi == gj;
+          const uint16_t fh = diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v);
+          p.A32[mm + (int64_t)gi * M + gj] = v;
+          p.Fh[mm + (int64_t)gi * M + gj] = fh;
+          if (tm != tn) {
+            p.A32[mm + (int64_t)gj * M + gi] = v;
+            p.Fh[mm + (int64_t)gj * M + gi] = fh;
+          }
+          if (diag) p.dA[mv + gi] = v;
+        } else if (EPI == EPI_BMAT) {
+          const float a = p.A32[mm + (int64_t)gi * M + gj];
+          const float di = p.dA[mv + gi], dj = p.dA[mv + gj];
+          uint16_t bh;
+          if (gi != gj) {
+            const float a2 = (v + di * a) + a * dj;
+            const float bv = p.cb * a + p.cc * a2;
+            bh = (uint16_t)anc_bf16_rne_bits(bv);
+          } else {
+            const float a2 = v + di * di;
+            p.dB[mv + gi] = p.cb * di + p.cc * a2;
+            bh = 0;
+          }
+          p.Bh[mm + (int64_t)gi * M + gj] = bh;
+          if (tm != tn) p.Bh[mm + (int64_t)gj * M + gi] = bh;
+        } else {
+          const int64_t o = mn + (int64_t)gi * N + gj;
+          const float x = p.X32[o];
+          const float y = (p.ca + p.dB[mv + gi]) * x + v;
+          p.X32[o] = y;
+          if (p.Yh != nullptr) {
+            const uint32_t yh = anc_bf16_rne_bits(y);
+            const int64_t ot = mn + (int64_t)gj * M + gi;
+            p.Yh[o] = (uint16_t)yh;
+            p.YhT[ot] = (uint16_t)yh;
+            if (p.Yl != nullptr) {
+              const uint16_t yl = (uint16_t)anc_bf16_rne_bits(y - anc_bf16_bits_to_f32(yh));
+              p.Yl[o] = yl;
+              p.YlT[ot] = yl;
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- fp32 validation GEMM
+// 128x128x16 tiles, v_mfma_f32_32x32x2_f32: every product and every sum in fp32.
+constexpr int FK = 16, FPITCH = 20, FNPITCH = 132;
+
+struct NsGemmF32 {
+  const float *A;          // (E, Mo, K) rows of the output
+  const float *B;          // NT: (E, No, K);  NN: (E, K, No)
+  int K, nn;
+  int64_t strideA, strideB;
+  int Mo, No;              // output dims per matrix
+  float ca, cb, cc;
+  const float *D;          // epilogue operand, same shape as the output (may be null)
+  float *out;
+  int epi;
+};
+
+__global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm_f32(NsGemmF32 p) {
+  __shared__ __attribute__((aligned(16))) float sA[BM * FPITCH];
+  __shared__ __attribute__((aligned(16))) float sB[BM * FPITCH > FK * FNPITCH ? BM * FPITCH : FK * FNPITCH];
+  const int tiles_m = p.Mo / BM, tiles_n = p.No / BN;
+  const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
+  const int e = L / (tiles_m * tiles_n), t = L % (tiles_m * tiles_n);
+  const int tm = t / tiles_n, tn = t % tiles_n;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int K = p.K;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[bi][bj][r] = 0.0f;
+
+  const float *Ae = p.A + (int64_t)e * p.strideA + (int64_t)(tm * BM) * K;
+  const float *Be = p.B + (int64_t)e * p.strideB;
+  for (int k0 = 0; k0 < K; k0 += FK) {
+    // A tile: 128 rows x 16 k, 4 lanes per row
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = (tid >> 2) + 64 * i, kq = (tid & 3) * 4;
+      *(anc_f32x4 *)&sA[row * FPITCH + kq] = *(const anc_f32x4 *)(Ae + (int64_t)row * K + k0 + kq);
+    }
+    if (!p.nn) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row = (tid >> 2) + 64 * i, kq = (tid & 3) * 4;
+        *(anc_f32x4 *)&sB[row * FPITCH + kq] =
+            *(const anc_f32x4 *)(Be + (int64_t)(tn * BN + row) * K + k0 + kq);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int kr = (tid >> 5) + 8 * i, c4 = (tid & 31) * 4;
+        *(anc_f32x4 *)&sB[kr * FNPITCH + c4] =
+            *(const anc_f32x4 *)(Be + (int64_t)(k0 + kr) * p.No + tn * BN + c4);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < FK / 2; ++kk) {
+      float a[2], b[2];
+      const int kx = kk * 2 + (lane >> 5);
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi) a[bi] = sA[(wm * 64 + bi * 32 + (lane & 31)) * FPITCH + kx];
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+        b[bj] = p.nn ? sB[kx * FNPITCH + wn * 64 + bj * 32 + (lane & 31)]
+                     : sB[(wn * 64 + bj * 32 + (lane & 31)) * FPITCH + kx];
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+          acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[bi], b[bj], acc[bi][bj], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  const int64_t base = (int64_t)e * p.Mo * p.No;
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gi = tm * BM + wm * 64 + bi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int gj = tn * BN + wn * 64 + bj * 32 + (lane & 31);
+        const int64_t o = base + (int64_t)gi * p.No + gj;
+        const float v = acc[bi][bj][r];
+        float y;
+        if (p.epi == EPI_GRAM)      y = v;
+        else if (p.epi == EPI_BMAT) y = p.cb * p.D[o] + p.cc * v;
+        else                        y = p.ca * p.D[o] + v;
+        p.out[o] = y;
+      }
+}
+
+// ------------------------------------------------------------------ Frobenius prologue
+__global__ void __launch_bounds__(kThreads)
+k_fro_partials(const float *__restrict__ X, int64_t mn, int nchunks, double *__restrict__ partials) {
+  const int64_t e = (int64_t)blockIdx.x / nchunks, c = (int64_t)blockIdx.x % nchunks;
+  chunk_partial<ANC_F32>((const void *)(X + e * mn), mn, c, partials + blockIdx.x);
+}
+
+// One block per matrix: lane t adds partials t, t+256, ... in order; butterfly; 4 wavefronts in order.
+__global__ void __launch_bounds__(kThreads)
+k_fro_finalize(const double *__restrict__ partials, int nchunks, float eps, float *__restrict__ recip) {
+  __shared__ double wave_sum[kThreads / 64];
+  const double *p = partials + (int64_t)blockIdx.x * nchunks;
+  double acc = 0.0;
+  for (int i = threadIdx.x; i < nchunks; i += kThreads) acc = acc + p[i];
+  acc = anc_wave_sum_f64(acc);
+  if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double t = wave_sum[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) t = t + wave_sum[w];
+    recip[blockIdx.x] = 1.0f / ((float)sqrt(t) + eps);
+  }
+}
+
+// X *= recip[e] in place; optional bf16 copies: Xh (M,N), XhT (N,M) and the residuals Xl, XlT.
+__global__ void __launch_bounds__(kThreads)
+k_ns_prep(float *__restrict__ X, const float *__restrict__ recip, int M, int N,
+          uint16_t *__restrict__ Xh, uint16_t *__restrict__ XhT,
+          uint16_t *__restrict__ Xl, uint16_t *__restrict__ XlT) {
+  __shared__ uint16_t th[64][66], tl[64][66];
+  const int tiles_n = N / 64, tiles_m = M / 64;
+  const int64_t per = (int64_t)tiles_m * tiles_n;
+  const int64_t e = (int64_t)blockIdx.x / per, tile = (int64_t)blockIdx.x % per;
+  const int tr = (int)(tile / tiles_n), tc = (int)(tile % tiles_n);
+  const float rc = recip[e];
+  const int64_t mn = e * (int64_t)M * N;
+  const int c4 = (threadIdx.x & 15) * 4, r0 = threadIdx.x >> 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + 16 * i;
+    const int64_t o = mn + (int64_t)(tr * 64 + r) * N + tc * 64 + c4;
+    anc_f32x4 x = *(const anc_f32x4 *)(X + o);
+    float xs[4] = {x.x * rc, x.y * rc, x.z * rc, x.w * rc};
+    anc_f32x4 xo = {xs[0], xs[1], xs[2], xs[3]};
+    *(anc_f32x4 *)(X + o) = xo;
+    if (Xh != nullptr) {
+      uint32_t h[4], l[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        h[k] = anc_bf16_rne_bits(xs[k]);
+        l[k] = anc_bf16_rne_bits(xs[k] - anc_bf16_bits_to_f32(h[k]));
+        th[r][c4 + k] = (uint16_t)h[k];
+        tl[r][c4 + k] = (uint16_t)l[k];
+      }
+      anc_u32x2 ho = {(h[0] & 0xFFFFu) | (h[1] << 16), (h[2] & 0xFFFFu) | (h[3] << 16)};
+      *(anc_u32x2 *)(Xh + o) = ho;
+      if (Xl != nullptr) {
+        anc_u32x2 lo = {(l[0] & 0xFFFFu) | (l[1] << 16), (l[2] & 0xFFFFu) | (l[3] << 16)};
+        *(anc_u32x2 *)(Xl + o) = lo;
+      }
+    }
+  }
+  if (Xh == nullptr) return;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + 16 * i;
+    const int64_t ot = mn + (int64_t)(tc * 64 + r) * M + tr * 64 + c4;
+    const uint32_t a0 = th[c4][r], a1 = th[c4 + 1][r], a2 = th[c4 + 2][r], a3 = th[c4 + 3][r];
+    anc_u32x2 ho = {a0 | (a1 << 16), a2 | (a3 << 16)};
+    *(anc_u32x2 *)(XhT + ot) = ho;
+    if (XlT != nullptr) {
+      const uint32_t b0 = tl[c4][r], b1 = tl[c4 + 1][r], b2 = tl[c4 + 2][r], b3 = tl[c4 + 3][r];
+      anc_u32x2 lo = {b0 | (b1 << 16), b2 | (b3 << 16)};
+      *(anc_u32x2 *)(XlT + ot) = lo;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------- workspace
+struct Carve {
+  uint64_t base;
+  int64_t off = 0;
+  explicit Carve(uint64_t b) : base(b) {}
+  template <typename T> T *take(int64_t count) {
+    T *p = (T *)(base + (uint64_t)off);
+    off += (count * (int64_t)sizeof(T) + 255) / 256 * 256;
+    return p;
+  }
+};
+
+struct Plan {
+  int nchunks;
+  bool split;
+  double *partials;
+  float *recip;
+  // bf16 modes
+  uint16_t *Xh[2], *XhT[2], *Xl[2], *XlT[2];
+  float *A32, *dA, *dB;
+  uint16_t *Fh, *Bh;
+  // fp32 mode
+  float *Af, *Bf, *Yf;
+  int64_t bytes;
+};
+
+Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int steps) {
+  Plan pl{};
+  Carve c(base);
+  pl.nchunks = (int)((M * N + ANC_GN_CHUNK - 1) / ANC_GN_CHUNK);
+  pl.split = (mode == ANC_NS_BF16);
+  pl.partials = c.take<double>(E * pl.nchunks);
+  pl.recip = c.take<float>(E);
+  if (mode == ANC_NS_FP32) {
+    pl.Af = c.take<float>(E * M * M);
+    pl.Bf = c.take<float>(E * M * M);
+    pl.Yf = c.take<float>(E * M * N);
+  } else {
+    for (int i = 0; i < 2; ++i) {
+      pl.Xh[i] = c.take<uint16_t>(E * M * N);
+      pl.XhT[i] = c.take<uint16_t>(E * M * N);
+    }
+    if (pl.split)
+      for (int i = 0; i < 2; ++i) {
+        pl.Xl[i] = c.take<uint16_t>(E * M * N);
+        pl.XlT[i] = c.take<uint16_t>(E * M * N);
+      }
+    pl.A32 = c.take<float>(E * M * M);
+    pl.Fh = c.take<uint16_t>(E * M * M);
+    pl.Bh = c.take<uint16_t>(E * M * M);
+    pl.dA = c.take<float>(E * M);
+    pl.dB = c.take<float>(E * M);
+  }
+  (void)steps;
+  pl.bytes = c.off;
+  return pl;
+}
+
+int check_shape(int64_t E, int64_t M, int64_t N, int mode, const char *who) {
+  ANC_REQUIRE(E > 0 && M > 0 && N > 0, "%s: E, M, N must be positive", who);
+  ANC_REQUIRE(M % 128 == 0 && N % 128 == 0, "%s: (M,N)=(%lld,%lld) must be multiples of 128", who,
+              (long long)M, (long long)N);
+  ANC_REQUIRE(M <= N, "%s: M=%lld > N=%lld; pass tall matrices transposed", who, (long long)M,
+              (long long)N);
+  ANC_REQUIRE(mode == ANC_NS_BF16 || mode == ANC_NS_FP32 || mode == ANC_NS_BF16_FAST,
+              "%s: unknown mode %d", who, mode);
+  ANC_REQUIRE(E * (M / 128) * (N / 128) < (1ll << 30) && E * M * N < (1ll << 40),
+              "%s: batch too large", who);
+  return ANC_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode) {
+  if (check_shape(E, M, N, mode, "anc_ns_workspace_bytes")) return -1;
+  return make_plan(0, E, M, N, mode, 0).bytes;
+}
+
+extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int steps,
+                              const float *coef, float eps, int mode, uint64_t workspace,
+                              int64_t workspace_bytes, uint64_t stream) {
+  if (int rc = check_shape(E, M, N, mode, "anc_ns_batched")) return rc;
+  ANC_REQUIRE(X != 0 && (X & 15) == 0, "anc_ns_batched: X must be a 16-byte aligned device pointer");
+  ANC_REQUIRE(steps >= 0 && steps <= 64 && (steps == 0 || coef != nullptr),
+              "anc_ns_batched: steps=%d out of range or null coefficients", steps);
+  ANC_REQUIRE(workspace != 0 && (workspace & 255) == 0, "anc_ns_batched: workspace must be 256-byte aligned");
+  const Plan pl = make_plan(workspace, E, M, N, mode, steps);
+  ANC_REQUIRE(workspace_bytes >= pl.bytes, "anc_ns_batched: workspace holds %lld bytes, %lld needed",
+              (long long)workspace_bytes, (long long)pl.bytes);
+  hipStream_t s = anc_stream(stream);
+  float *X32 = (float *)X;
+  const int64_t mn = M * N;
+
+  // ---- X /= ||X||_F + eps
+  hipLaunchKernelGGL(k_fro_partials, dim3((unsigned)(E * pl.nchunks)), dim3(kThreads), 0, s, X32, mn,
+                     pl.nchunks, pl.partials);
+  ANC_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s, pl.partials, pl.nchunks,
+                     eps, pl.recip);
+  ANC_LAUNCH_CHECK();
+  const unsigned prep_grid = (unsigned)(E * (M / 64) * (N / 64));
+  const int split_from = pl.split ? (steps >= 2 ? steps - 2 : 0) : steps;   // first split iteration
+
+  if (mode == ANC_NS_FP32) {
+    hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
+                       (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr);
+    ANC_LAUNCH_CHECK();
+    float *cur = X32, *nxt = pl.Yf;
+    const unsigned g_mm = (unsigned)(E * (M / BM) * (M / BN)), g_mn = (unsigned)(E * (M / BM) * (N / BN));
+    for (int k = 0; k < steps; ++k) {
+      const float a = coef[3 * k], b = coef[3 * k + 1], c = coef[3 * k + 2];
+      NsGemmF32 g{};
+      g.A = cur; g.B = cur; g.K = (int)N; g.nn = 0; g.strideA = mn; g.strideB = mn;
+      g.Mo = (int)M; g.No = (int)M; g.out = pl.Af; g.epi = EPI_GRAM;
+      hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mm), dim3(kGemmThreads), 0, s, g);
+      ANC_LAUNCH_CHECK();
+      NsGemmF32 h{};
+      h.A = pl.Af; h.B = pl.Af; h.K = (int)M; h.nn = 0; h.strideA = M * M; h.strideB = M * M;
+      h.Mo = (int)M; h.No = (int)M; h.cb = b; h.cc = c; h.D = pl.Af; h.out = pl.Bf; h.epi = EPI_BMAT;
+      hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mm), dim3(kGemmThreads), 0, s, h);
+      ANC_LAUNCH_CHECK();
+      NsGemmF32 y{};
+      y.A = pl.Bf; y.B = cur; y.K = (int)M; y.nn = 1; y.strideA = M * M; y.strideB = mn;
+      y.Mo = (int)M; y.No = (int)N; y.ca = a; y.D = cur; y.out = nxt; y.epi = EPI_BX;
+      hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mn), dim3(kGemmThreads), 0, s, y);
+      ANC_LAUNCH_CHECK();
+      float *tmp = cur; cur = nxt; nxt = tmp;
+    }
+    if (cur != X32)
+      ANC_HIP(hipMemcpyAsync(X32, cur, (size_t)(E * mn) * sizeof(float), hipMemcpyDeviceToDevice, s));
+    return ANC_OK;
+  }
+
+  // ---- bf16 matrix-core chain
+  if (steps == 0) {
+    hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
+                       (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr);
+    ANC_LAUNCH_CHECK();
+    return ANC_OK;
+  }
+  const bool split0 = split_from <= 0;
+  hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
+                     pl.Xh[0], pl.XhT[0], split0 ? pl.Xl[0] : (uint16_t *)nullptr,
+                     split0 ? pl.XlT[0] : (uint16_t *)nullptr);
+  ANC_LAUNCH_CHECK();
+  const int tM = (int)(M / BM), tN = (int)(N / BN);
+  const unsigned g_sym = (unsigned)(E * tM * (tM + 1) / 2), g_mn = (unsigned)(E * tM * tN);
+  int cur = 0;
+  for (int k = 0; k < steps; ++k) {
+    const bool split = k >= split_from;
+    const bool last = k + 1 == steps;
+    const bool split_next = !last && (k + 1 >= split_from);
+    NsGemm g{};
+    g.M = (int)M; g.N = (int)N;
+    g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB; g.X32 = X32;
+    g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
+    // A = X X^T
+    NsGemm ga = g;
+    ga.A[0] = pl.Xh[cur]; ga.B[0] = pl.Xh[cur]; ga.nterms = 1;
+    if (split) {
+      ga.A[1] = pl.Xh[cur]; ga.B[1] = pl.Xl[cur];
+      ga.A[2] = pl.Xl[cur]; ga.B[2] = pl.Xh[cur];
+      ga.nterms = 3;
+    }
+    ga.K = (int)N; ga.strideA = mn; ga.strideB = mn; ga.tiles_m = tM; ga.tiles_n = tM; ga.lower = 1;
+    hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga);
+    ANC_LAUNCH_CHECK();
+    // B = b A + c A A
+    NsGemm gb = g;
+    gb.A[0] = pl.Fh; gb.B[0] = pl.Fh; gb.nterms = 1;
+    gb.K = (int)M; gb.strideA = M * M; gb.strideB = M * M; gb.tiles_m = tM; gb.tiles_n = tM; gb.lower = 1;
+    hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb);
+    ANC_LAUNCH_CHECK();
+    // X = a X + B X
+    NsGemm gx = g;
+    gx.A[0] = pl.Bh; gx.B[0] = pl.XhT[cur]; gx.nterms = 1;
+    if (split) { gx.A[1] = pl.Bh; gx.B[1] = pl.XlT[cur]; gx.nterms = 2; }
+    gx.K = (int)M; gx.strideA = M * M; gx.strideB = mn; gx.tiles_m = tM; gx.tiles_n = tN; gx.lower = 0;
+    gx.Yh = last ? nullptr : pl.Xh[cur ^ 1];
+    gx.YhT = last ? nullptr : pl.XhT[cur ^ 1];
+    gx.Yl = split_next ? pl.Xl[cur ^ 1] : nullptr;
+    gx.YlT = split_next ? pl.XlT[cur ^ 1] : nullptr;
+    hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx);
+    ANC_LAUNCH_CHECK();
+    cur ^= 1;
+  }
+  return ANC_OK;
+}

@@ -1,0 +1,120 @@
+"""Muon + AdamW hybrid optimizer on the MI355X.
+
+Mirror of ancora/optim/hybrid.py: `HybridOptimizer(params, is_muon, no_decay, muon_kw,
+adamw_kw, si, muon_device)` with `.step(grads, stream_int)`, `.weights()`, `.routing()`,
+`.free()` and the attributes `.muon`, `.adamw`, `.muon_names`, `.adamw_names`; the routing
+predicate `default_is_muon`. Muon takes the 2-D hidden matrices, AdamW everything else
+(gains, embedding, head), and `step` runs Muon first, then AdamW (hybrid.py:45-47).
+
+Extensions, all off by default: `max_grad_norm` (one global norm over every gradient of both
+groups, clip scale applied to g before the momentum / moment updates), the non-finite guard
+that comes with it (a step with an Inf/NaN gradient leaves every state tensor untouched and
+does not advance the step counters), stochastic-rounded bf16 weights, bf16 gradients.
+"""
+import numpy as np
+
+from . import _lib
+from .adamw import AdamW
+from .devbuf import DevBuf
+from .gradnorm import StepGuard
+from .muon import Muon
+from .muon_ns import NTM
+
+_ADAMW_TOKENS = ("norm", "ln", "embed", "lm_head", "head", "wte", "wpe")
+
+
+def default_is_muon(name, p):
+    """2-D matrix that is not a norm gain / embedding / lm_head -> Muon (hybrid.py:18-25)."""
+    if p.ndim != 2:
+        return False
+    low = name.lower()
+    if any(t in low for t in _ADAMW_TOKENS):
+        return False
+    return True
+
+
+def resident_is_muon(name, p):
+    """Routing of the device-resident models: like `default_is_muon`, but a stacked [E,K,N]
+    expert tensor is E Muon matrices (ancora/kernels/moe.py:433-435, 536-548) and a matrix
+    that is not 128-aligned -- the (H, E) router -- stays on AdamW (`_ns_ok`,
+    ancora/optim/muon.py:37-41)."""
+    if p.ndim not in (2, 3):
+        return False
+    low = name.lower()
+    if any(t in low for t in _ADAMW_TOKENS) or "router" in low:
+        return False
+    return p.shape[-2] % NTM == 0 and p.shape[-1] % NTM == 0
+
+
+class HybridOptimizer:
+    def __init__(self, params, is_muon=default_is_muon, no_decay=None, muon_kw=None,
+                 adamw_kw=None, si=None, muon_device=False, max_grad_norm=None, guard=False,
+                 grad_dtype=np.float32):
+        muon_kw = dict(lr=0.02, momentum=0.95, ns_steps=5, **(muon_kw or {}))
+        if muon_device:                      # the reference's switch for GPU Newton-Schulz;
+            muon_kw.update(device=True, si=si)   # here the GPU path is the only path
+        adamw_kw = adamw_kw or dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.01)
+        if no_decay is None:
+            no_decay = lambda n, p: (p.ndim == 1)          # noqa: E731  don't decay 1-D gains/biases
+
+        self.muon_names = [n for n, p in params.items() if is_muon(n, p)]
+        self.adamw_names = [n for n in params if n not in self.muon_names]
+        self.muon = Muon({n: params[n] for n in self.muon_names}, grad_dtype=grad_dtype, **muon_kw)
+        self.adamw = AdamW({n: params[n] for n in self.adamw_names},
+                           no_decay=tuple(n for n in self.adamw_names if no_decay(n, params[n])),
+                           grad_dtype=grad_dtype, **adamw_kw)
+        self.guard = StepGuard(max_grad_norm) if (max_grad_norm is not None or guard) else None
+        self.last_skipped = False
+
+    def _grad_bufs(self, grads):
+        """Gradient DevBufs in the fixed order of the global norm: Muon names, then AdamW names."""
+        out = []
+        for n in self.muon_names:
+            g = grads[n]
+            out.append(g if isinstance(g, DevBuf) else self.muon.st[n]["g"])
+        for n in self.adamw_names:
+            g = grads[n]
+            out.append(g if isinstance(g, DevBuf) else self.adamw.st[n]["g"])
+        return out
+
+    def step(self, grads, stream_int):
+        if self.guard is None:
+            self.muon.step({n: grads[n] for n in self.muon_names}, stream_int)
+            self.adamw.step({n: grads[n] for n in self.adamw_names}, stream_int)
+            return
+        # guarded step: every gradient must be resident before the norm, so upload first
+        for opt, names in ((self.muon, self.muon_names), (self.adamw, self.adamw_names)):
+            for n in names:
+                g = grads[n]
+                if not isinstance(g, DevBuf):
+                    s = opt.st[n]
+                    g = np.asarray(g)
+                    if g.dtype != s["g"].dtype and s["g"].dtype == np.float32:
+                        g = g.astype(np.float32)
+                    s["g"].upload(g.reshape(s["g"].shape), stream_int)
+        resident = {}
+        for opt, names in ((self.muon, self.muon_names), (self.adamw, self.adamw_names)):
+            for n in names:
+                g = grads[n]
+                resident[n] = g if isinstance(g, DevBuf) else opt.st[n]["g"]
+        self.guard.compute(self._grad_bufs(grads), stream_int)
+        self.muon.launch({n: resident[n] for n in self.muon_names}, stream_int, self.guard)
+        self.adamw.launch({n: resident[n] for n in self.adamw_names}, stream_int, self.guard)
+        _lib.stream_sync(stream_int)
+        self.last_ctl = self.guard.read(stream_int)
+        self.last_skipped = self.last_ctl["skip"]
+        if self.last_skipped:
+            self.muon.unstep()
+            self.adamw.unstep()
+
+    def weights(self):
+        return {**self.muon.weights(), **self.adamw.weights()}
+
+    def routing(self):
+        return {"muon": list(self.muon_names), "adamw": list(self.adamw_names)}
+
+    def free(self):
+        self.muon.free()
+        self.adamw.free()
+        if self.guard is not None:
+            self.guard.free()

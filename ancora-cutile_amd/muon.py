@@ -1,0 +1,370 @@
+"""Muon (momentum orthogonalised by Newton-Schulz) on the MI355X.
+
+Mirror of ancora/optim/muon.py: the host-API class `Muon`, the device-resident classes
+`DeviceMuon`, `MuonScratch`, `ResidentMuon`, `BatchedProjMuon`, and `newton_schulz5`.
+In the reference the host class runs Newton-Schulz in numpy on the CPU and the
+resident classes chain cuda-tile kernels one weight (or one chunk of 8) at a time;
+here every class drives the same engine: all weights of one Newton-Schulz shape
+(M = min(K,N), Nn = max(K,N)) form one packed fp32 batch, and a step is three
+launches per batch -- momentum for every weight, the whole NS chain, update + bf16
+refresh for every weight. Tall weights (K > N) enter and leave the batch transposed
+inside those elementwise kernels (ancora/optim/muon.py:72-74, 264-274).
+
+    buf = mu*buf + g;  u = g + mu*buf (Nesterov);  O = NS(u);  W -= lr*sqrt(max(1,K/N))*O
+
+Batching is bitwise neutral: a weight's result does not depend on which other weights
+share its batch, on `chunk` or on `scope` (tests/training/test_batched_proj_muon.py:74).
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import api, MuonDesc, F32, BF16, MUON_MAX_SCALES
+from .bf16 import bf16_bits, bits_f32, bf16_round as _bf        # noqa: F401
+from .devbuf import DevBuf, upload_table
+from . import muon_ns
+from .muon_ns import NTM, _KELLER, NsWorkspace
+
+
+def _g_code(dtype):
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return F32
+    if dtype == np.uint16:
+        return BF16
+    raise TypeError(f"gradient dtype {dtype}: expected float32 or uint16 (bf16 bits)")
+
+
+def _check_aligned(K, N, what="Muon weight"):
+    # same alignment rule as the reference's asserts (ancora/optim/muon.py:98,172,233)
+    if K % NTM or N % NTM:
+        raise ValueError(f"{what} ({K},{N}) tile-misaligned: both dims must be multiples of {NTM}")
+
+
+def _f32bf_trunc(x):
+    """Truncating fp32 -> bf16 bits: the reference's *initial* p16 (`f32_to_bf16_bits`,
+    ancora/kernels/loss.py:273-274, used at ancora/optim/muon.py:105). After the first step p16
+    is the RNE of p32."""
+    return (np.ascontiguousarray(x, dtype=np.float32).view(np.uint32) >> np.uint32(16)).astype(np.uint16)
+
+
+class _Batch:
+    """One packed Newton-Schulz batch: weights of one (M, Nn) shape, its descriptor table."""
+
+    def __init__(self, M, Nn, weights):
+        self.M, self.Nn, self.weights = M, Nn, weights
+        self.E = len(weights)
+        self.table = None
+        self.key = None
+        self.total_blocks = 0
+
+    def build(self, U, scale_index):
+        key = tuple((w["G"].ptr, w["G"].dtype.str, w["p32"].ptr, w["p16"].ptr if w["p16"] is not None else 0,
+                     w["buf"].ptr) for w in self.weights) + (U.ptr,)
+        if key == self.key:
+            return
+        if self.table is not None:
+            self.table.free()
+        descs, blk0 = [], 0
+        for i, w in enumerate(self.weights):
+            K, N = w["K"], w["N"]
+            descs.append(MuonDesc(w["buf"].ptr, w["G"].ptr, w["p32"].ptr,
+                                  w["p16"].ptr if w["p16"] is not None else 0,
+                                  U.ptr + i * self.M * self.Nn * 4, K, N, int(K > N),
+                                  _g_code(w["G"].dtype), scale_index[w["scale"]], w["seed"], blk0))
+            blk0 += (K * N) // 4096
+        self.total_blocks = blk0
+        self.table = upload_table(descs)
+        self.key = key
+
+    def free(self):
+        if self.table is not None:
+            self.table.free()
+            self.table = None
+
+
+class MuonEngine:
+    """Shape-grouped, batched Muon over device-resident weights.
+
+    weights: list of dicts {buf, p32, p16, G: DevBuf; K, N: int; lid: int (optional)} -- the
+    record of ancora/optim/muon.py:220. `chunk` caps the matrices per batch (None = the whole
+    shape group, which is what 288 GB of HBM is for); `scope=k` sub-groups by lid // k
+    (ancora/optim/muon.py:221-222,235). Neither changes any result bit."""
+
+    def __init__(self, weights, momentum=0.95, ns_steps=5, nesterov=True, chunk=None, scope=None,
+                 mode="bf16", sr=False, seed=0, workspace=None):
+        _lib.init()
+        self.mom, self.ns, self.nesterov = float(momentum), int(ns_steps), bool(nesterov)
+        self.mode, self.sr, self.seed = mode, bool(sr), int(seed)
+        self.t = 0
+        groups = {}
+        scales = []
+        for idx, w in enumerate(weights):
+            K, N = int(w["K"]), int(w["N"])
+            _check_aligned(K, N)
+            w["tr"] = K > N
+            w["M"], w["Nn"] = (N, K) if w["tr"] else (K, N)
+            w["scale"] = max(1.0, K / N) ** 0.5                  # ancora/optim/muon.py:232
+            w.setdefault("seed", idx)
+            if w["scale"] not in scales:
+                scales.append(w["scale"])
+            key = (w["M"], w["Nn"]) if scope is None else (w["M"], w["Nn"], w.get("lid", 0) // scope)
+            groups.setdefault(key, []).append(w)
+        if len(scales) > MUON_MAX_SCALES:
+            raise ValueError(f"more than {MUON_MAX_SCALES} distinct K/N ratios in one Muon group")
+        self.scales = scales
+        self.scale_index = {s: i for i, s in enumerate(scales)}
+        self.batches = []
+        for key, ws in groups.items():
+            c = len(ws) if chunk is None else max(1, min(int(chunk), len(ws)))
+            for i0 in range(0, len(ws), c):
+                self.batches.append(_Batch(key[0], key[1], ws[i0:i0 + c]))
+        self.groups = groups
+        self._own_ws = workspace is None
+        self.ws = NsWorkspace() if workspace is None else workspace
+        self.U = None
+        umax = max(b.E * b.M * b.Nn for b in self.batches) if self.batches else 0
+        wmax = max(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, mode) for b in self.batches) \
+            if self.batches else 0
+        if umax:
+            self.U = DevBuf.empty((umax,), np.float32)
+            self.ws.ensure(wmax)
+
+    def nbytes(self):
+        return (self.U.nbytes if self.U is not None else 0) + self.ws.nbytes()
+
+    def step(self, si, lr=0.02, schedule=_KELLER, guard=None):
+        """One Muon step over every weight. Asynchronous on stream `si`."""
+        self.t += 1
+        schedule = muon_ns._resolve(schedule)
+        ctl = 0 if guard is None else guard.ptr
+        lr_scales = (ctypes.c_float * MUON_MAX_SCALES)(*[lr * s for s in self.scales])
+        seed_base = ((self.seed + 1000003 * self.t) & 0xFFFFFFFF) if self.sr else 0
+        coef = muon_ns.coef_array(schedule, self.ns)
+        for b in self.batches:
+            b.build(self.U, self.scale_index)
+            api.anc_muon_momentum_multi(b.table.ptr, b.E, b.total_blocks, self.mom,
+                                        int(self.nesterov), F32, ctl, int(si))
+            need = muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self.mode)
+            buf = self.ws.ensure(need)
+            api.anc_ns_batched(self.U.ptr, b.E, b.M, b.Nn, self.ns, coef, 1e-7,
+                               muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(si))
+            api.anc_muon_update_multi(b.table.ptr, b.E, b.total_blocks, lr_scales, F32,
+                                      int(self.sr), seed_base, ctl, int(si))
+
+    def unstep(self):
+        self.t -= 1
+
+    def free(self):
+        for b in self.batches:
+            b.free()
+        if self.U is not None:
+            self.U.free()
+            self.U = None
+        if self._own_ws:
+            self.ws.free()
+
+
+def newton_schulz5(G, steps=5, eps=1e-7, schedule=None, mode="bf16", si=0):
+    """Orthogonalise one host matrix on the device (the reference's host function,
+    ancora/optim/muon.py:67-80, runs this in numpy; Keller coefficients by default as there).
+    Returns an fp32 ndarray of the same shape. Both dims must be multiples of 128."""
+    G = np.asarray(G, dtype=np.float32)
+    K, N = G.shape
+    _check_aligned(K, N, "newton_schulz5 input")
+    X = np.ascontiguousarray(G.T) if K > N else G
+    M, Nn = X.shape
+    d = DevBuf(X)
+    try:
+        muon_ns.ns_batched(d, 1, M, Nn, si, steps=steps, eps=eps, schedule=schedule, mode=mode)
+        out = d.to_numpy(si)
+    finally:
+        d.free()
+    return np.ascontiguousarray(out.T) if K > N else out
+
+
+class MuonScratch:
+    """Shared transient Newton-Schulz scratch for per-weight resident Muon
+    (ancora/optim/muon.py:138-159): sized for the largest weight, one for the whole model."""
+
+    def __init__(self, shapes, mode="bf16"):
+        self.mode = mode
+        self.ws = NsWorkspace()
+        kn = max(int(K) * int(N) for K, N in shapes)
+        need = max(muon_ns.ns_workspace_bytes(1, min(K, N), max(K, N), mode) for K, N in shapes)
+        self.ws.ensure(need)
+        self.u = DevBuf.empty((kn,), np.float32)
+
+    def nbytes(self):
+        return self.ws.nbytes() + self.u.nbytes
+
+    def free(self):
+        self.ws.free()
+        self.u.free()
+
+
+class ResidentMuon:
+    """Per-2D-weight Muon over the layer's existing buffers (p32 master + the p16 the GEMM reads)
+    with a shared MuonScratch; the only persistent state is the momentum buffer
+    (ancora/optim/muon.py:162-204)."""
+
+    def __init__(self, p32, p16, K, N, scratch, momentum=0.95, ns_steps=5, mode=None):
+        _check_aligned(K, N)
+        self.p32, self.p16, self.K, self.N, self.sc = p32, p16, K, N, scratch
+        self.tr = K > N
+        self.M, self.Nn = (N, K) if self.tr else (K, N)
+        self.shape_scale = max(1.0, K / N) ** 0.5
+        self.mom, self.ns = momentum, ns_steps
+        self.mode = scratch.mode if mode is None else mode
+        self.buf = DevBuf.zeros((K, N), np.float32)
+
+    def step(self, g_dev, si, lr=0.02, schedule=_KELLER, guard=None):
+        """g_dev: (K,N) device weight-gradient (float32, or uint16 bf16 bits)."""
+        K, N, sc = self.K, self.N, self.sc
+        ctl = 0 if guard is None else guard.ptr
+        api.anc_muon_momentum(self.buf.ptr, g_dev.ptr, sc.u.ptr, K, N, float(self.mom), 1,
+                              int(self.tr), _g_code(g_dev.dtype), F32, ctl, int(si))
+        muon_ns.ns_batched(sc.u, 1, self.M, self.Nn, si, steps=self.ns, schedule=schedule,
+                           mode=self.mode, workspace=sc.ws)
+        api.anc_muon_update(self.p32.ptr, self.p16.ptr, sc.u.ptr, K, N,
+                            float(lr * self.shape_scale), int(self.tr), F32, 0, 0, ctl, int(si))
+
+    def free(self):
+        self.buf.free()
+
+
+class DeviceMuon:
+    """Device-resident Muon over one 2-D weight with its own state and scratch
+    (ancora/optim/muon.py:88-135)."""
+
+    def __init__(self, W, lr=0.02, momentum=0.95, ns_steps=5, mode="bf16"):
+        K, N = W.shape
+        _check_aligned(K, N)
+        self.K, self.N = K, N
+        self.lr = lr
+        self.p32 = DevBuf(np.ascontiguousarray(W, dtype=np.float32))
+        self.p16 = DevBuf(_f32bf_trunc(W))
+        self._scratch = MuonScratch([(K, N)], mode)
+        self._rm = ResidentMuon(self.p32, self.p16, K, N, self._scratch, momentum, ns_steps)
+        self.buf = self._rm.buf
+
+    def step(self, g_dev, si, schedule=_KELLER):
+        self._rm.step(g_dev, si, self.lr, schedule)
+
+    def master(self):
+        return self.p32.to_numpy()
+
+    def free(self):
+        self._rm.free()
+        self._scratch.free()
+        self.p32.free()
+        self.p16.free()
+
+
+class BatchedProjMuon:
+    """Model-level batched Muon over all 2-D projection weights across layers
+    (ancora/optim/muon.py:207-284). weights: list of {buf, p32, p16, G, K, N, lid}."""
+
+    def __init__(self, weights, momentum=0.95, ns_steps=5, chunk=8, scope=None, mode="bf16",
+                 sr=False, seed=0):
+        self.mom, self.ns = momentum, ns_steps
+        self.engine = MuonEngine(weights, momentum, ns_steps, True, chunk, scope, mode, sr, seed)
+        self.groups = self.engine.groups
+
+    def step(self, si, lr=0.02, schedule=_KELLER, guard=None):
+        self.engine.step(si, lr, schedule, guard)
+
+    def free(self):
+        self.engine.free()
+
+
+class Muon:
+    """fp32-master Muon for 2-D matrix params (ancora/optim/muon.py:287-318). params:
+    {name: (R,C) fp32 ndarray}; a 3-D [E,R,C] entry is E independent slices. The reference's host
+    class runs Newton-Schulz on the CPU unless `device=True`; this one always runs on the GPU, so
+    `device` and `si` are accepted and only `si` is used (as the default stream). `schedule`
+    defaults to the process-wide setting of `set_polar_express` (Keller unless switched)."""
+
+    def __init__(self, params, lr=0.02, momentum=0.95, nesterov=True, ns_steps=5, device=False,
+                 si=None, schedule=_KELLER, mode="bf16", chunk=None, sr=False, seed=0,
+                 grad_dtype=np.float32):
+        _lib.init()
+        self.lr, self.mom, self.nesterov, self.ns = lr, momentum, nesterov, ns_steps
+        self.device, self.si, self.schedule = device, si, schedule
+        self.st = {}
+        recs = []
+        gdt = np.dtype(grad_dtype)
+        for n, p in params.items():
+            assert p.ndim in (2, 3), f"Muon is for 2D matrices, {n} is {p.shape}"
+            K, N = p.shape[-2], p.shape[-1]
+            _check_aligned(K, N, f"Muon weight '{n}'")
+            E = 1 if p.ndim == 2 else p.shape[0]
+            s = dict(shape=p.shape, E=E, K=K, N=N,
+                     p32=DevBuf(np.ascontiguousarray(p, dtype=np.float32).reshape(E * K, N)),
+                     p16=DevBuf.zeros((E * K, N), np.uint16),
+                     buf=DevBuf.zeros((E * K, N), np.float32),
+                     g=DevBuf.zeros((E * K, N), gdt))
+            self.st[n] = s
+            for e in range(E):
+                recs.append(dict(buf=s["buf"].at_pos(e * K), p32=s["p32"].at_pos(e * K),
+                                 p16=s["p16"].at_pos(e * K), G=s["g"].at_pos(e * K), K=K, N=N,
+                                 name=n, e=e))
+        self._recs = recs
+        self.engine = MuonEngine(recs, momentum, ns_steps, nesterov, chunk, None, mode, sr, seed) \
+            if recs else None
+        self.last_skipped = False
+
+    def launch(self, grads, stream_int=None, guard=None):
+        si = stream_int if stream_int is not None else (self.si or 0)
+        for n, s in self.st.items():
+            g = grads[n]
+            if isinstance(g, DevBuf):
+                for r in self._recs:
+                    if r["name"] == n:
+                        r["G"] = g.view((s["E"] * s["K"], s["N"])).at_pos(r["e"] * s["K"])
+            else:
+                g = np.asarray(g)
+                if g.dtype != s["g"].dtype:
+                    if s["g"].dtype == np.float32:
+                        g = g.astype(np.float32)
+                    else:
+                        raise TypeError(f"Muon: gradient of '{n}' is {g.dtype}, the optimizer was "
+                                        f"built for {s['g'].dtype}")
+                s["g"].upload(g.reshape(s["E"] * s["K"], s["N"]), si)
+        if self.engine is not None:
+            self.engine.step(si, self.lr, self.schedule, guard)
+        return si
+
+    def unstep(self):
+        if self.engine is not None:
+            self.engine.unstep()
+
+    def step(self, grads, stream_int=None, guard=None):
+        si = self.launch(grads, stream_int, guard)
+        _lib.stream_sync(si)
+        self.last_skipped = False
+        if guard is not None and guard.read(si)["skip"]:
+            self.unstep()
+            self.last_skipped = True
+
+    def weights(self):
+        """bf16-valued fp32 weights for the forward (ancora/optim/muon.py:311-312)."""
+        return {n: _bf(s["p32"].to_numpy()).reshape(s["shape"]) for n, s in self.st.items()}
+
+    def weights16(self):
+        """The device-maintained bf16 copy (RNE or SR of the master), as fp32 values."""
+        return {n: bits_f32(s["p16"].to_numpy()).reshape(s["shape"]) for n, s in self.st.items()}
+
+    def master(self):
+        return {n: s["p32"].to_numpy().reshape(s["shape"]) for n, s in self.st.items()}
+
+    def momentum_buffers(self):
+        return {n: s["buf"].to_numpy().reshape(s["shape"]) for n, s in self.st.items()}
+
+    def free(self):
+        if self.engine is not None:
+            self.engine.free()
+        for s in self.st.values():
+            for k in ("p32", "p16", "buf", "g"):
+                s[k].free()

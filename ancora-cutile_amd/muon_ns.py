@@ -1,0 +1,153 @@
+"""Resident Newton-Schulz / Polar-Express drivers on the MI355X.
+
+Mirror of ancora/kernels/muon_ns.py: `newton_schulz_resident`, `newton_schulz_resident_e`,
+`PE_SCHEDULE`, the Keller coefficients, the process-wide `set_polar_express` toggle with
+its `_KELLER` sentinel, and the tile constants `NTM, NTN, NTK`. The 25 cuda-tile kernels
+and the 28-launch chain behind those drivers are replaced by one C entry point,
+`anc_ns_batched`, which runs the whole chain for a batch of same-shape matrices.
+
+The library carries the iterate in fp32 (operands are rounded to bf16 only at the
+matrix-core input), so its native driver `ns_batched` takes and returns fp32. The two
+reference-shaped drivers keep the reference's bf16 in / bf16 out contract on `gX`: they
+widen into a workspace, run the chain and round the result back (RNE). Their scratch
+arguments (gA, gA2, gB, gBX, grecip) are accepted for call compatibility and not touched.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import api, NS_BF16, NS_FP32, NS_BF16_FAST
+from .devbuf import DevBuf
+
+NTM, NTN, NTK = 128, 128, 64                       # ancora/kernels/muon_ns.py:20
+A_COEF, B_COEF, C_COEF = 3.4445, -4.7750, 2.0315   # ancora/kernels/muon_ns.py:21
+
+# Polar-Express per-iteration coefficients (ancora/kernels/muon_ns.py:30-34)
+PE_SCHEDULE = [(4.0848, -6.8946, 2.9270),
+               (3.9505, -6.3029, 2.6377),
+               (3.7418, -5.5913, 2.3037),
+               (2.8769, -3.1427, 1.2046),
+               (2.8366, -3.0525, 1.2012)]
+
+MODES = {"bf16": NS_BF16, "bf16_fast": NS_BF16_FAST, "fp32": NS_FP32}
+
+
+def _coef_at(schedule, k):
+    """(a,b,c) of iteration k: Keller if schedule is None, else schedule[k] with the last triple
+    repeated once the schedule is exhausted (ancora/kernels/muon_ns.py:37-42)."""
+    if schedule is None:
+        return A_COEF, B_COEF, C_COEF
+    return schedule[k] if k < len(schedule) else schedule[-1]
+
+
+# Process-wide default: None = Keller (ancora/kernels/muon_ns.py:44-65). `schedule=None` passed
+# explicitly still means Keller; the sentinel means "caller said nothing, use the default".
+_KELLER = object()
+_DEFAULT_SCHEDULE = None
+
+
+def set_polar_express(on: bool):
+    """Select Polar Express (on) or Keller (off) for every NS call that does not pass an explicit
+    schedule. Returns the previous setting."""
+    global _DEFAULT_SCHEDULE
+    prev = _DEFAULT_SCHEDULE
+    _DEFAULT_SCHEDULE = PE_SCHEDULE if on else None
+    return prev
+
+
+def _resolve(schedule):
+    return _DEFAULT_SCHEDULE if schedule is _KELLER else schedule
+
+
+def coef_array(schedule, steps):
+    flat = []
+    for k in range(steps):
+        flat.extend(_coef_at(schedule, k))
+    return (ctypes.c_float * max(1, len(flat)))(*flat)
+
+
+class NsWorkspace:
+    """Device scratch of the chain; grows on demand, never shrinks. The chain keeps nothing in it
+    between calls, so one workspace serves every group that runs sequentially on a stream
+    (the role of MuonScratch / ExpertMuonScratch, ancora/optim/muon.py:138-159)."""
+
+    def __init__(self):
+        self.buf = None
+
+    def ensure(self, nbytes):
+        if self.buf is None or self.buf.nbytes < nbytes:
+            if self.buf is not None:
+                _lib.api.anc_device_sync()
+                self.buf.free()
+            self.buf = DevBuf.empty((int(nbytes),), np.uint8)
+        return self.buf
+
+    def nbytes(self):
+        return 0 if self.buf is None else self.buf.nbytes
+
+    def free(self):
+        if self.buf is not None:
+            self.buf.free()
+            self.buf = None
+
+
+_SHARED_WS = NsWorkspace()
+
+
+def ns_workspace_bytes(E, M, N, mode="bf16"):
+    _lib.load()
+    n = api.anc_ns_workspace_bytes(E, M, N, MODES[mode])
+    if n < 0:
+        raise _lib.AncoraError(_lib._lib.anc_last_error().decode())
+    return int(n)
+
+
+def ns_batched(X32, E, M, N, si, steps=5, eps=1e-7, schedule=_KELLER, mode="bf16", workspace=None):
+    """Native driver: X32 is a DevBuf of E packed (M,N) fp32 matrices, M <= N, both multiples of
+    128; overwritten with the orthogonalised result."""
+    schedule = _resolve(schedule)
+    if X32.dtype != np.float32 or X32.size < E * M * N:
+        raise ValueError(f"ns_batched: X32 must hold {E}x{M}x{N} float32, has {X32.size} {X32.dtype}")
+    ws = _SHARED_WS if workspace is None else workspace
+    need = ns_workspace_bytes(E, M, N, mode)
+    buf = ws.ensure(need)
+    coef = coef_array(schedule, steps)
+    api.anc_ns_batched(X32.ptr, E, M, N, int(steps), coef, float(eps), MODES[mode], buf.ptr,
+                       buf.nbytes, int(si))
+
+
+ns_fp32_batched = ns_batched
+
+
+def _run_bf16(gX, E, M, N, si, steps, eps, schedule, mode, workspace):
+    if gX.dtype != np.uint16 or gX.size < E * M * N:
+        raise ValueError("newton_schulz_resident: gX must hold the packed bf16 (uint16) batch")
+    if M % NTM or N % NTN or M > N:
+        raise ValueError(f"newton_schulz_resident: (M,N)=({M},{N}) must be 128-aligned with M <= N")
+    ws = _SHARED_WS if workspace is None else workspace
+    n = E * M * N
+    need = ns_workspace_bytes(E, M, N, mode)
+    xbytes = (n * 4 + 255) // 256 * 256
+    buf = ws.ensure(need + xbytes)
+    x32 = DevBuf(shape=(E * M, N), dtype=np.float32, ptr=buf.ptr)
+    api.anc_bf16_to_f32(gX.ptr, x32.ptr, n, int(si))
+    coef = coef_array(schedule, steps)
+    api.anc_ns_batched(x32.ptr, E, M, N, int(steps), coef, float(eps), MODES[mode],
+                       buf.ptr + xbytes, buf.nbytes - xbytes, int(si))
+    api.anc_f32_to_bf16(x32.ptr, gX.ptr, n, int(si))
+
+
+def newton_schulz_resident(gX, gA, gA2, gB, gBX, grecip, M, N, si, steps=5, eps=1e-7,
+                           schedule=_KELLER, fused=True, mode="bf16", workspace=None):
+    """Resident NS on one (M,N) bf16 matrix, overwritten in place
+    (ancora/kernels/muon_ns.py:245-283). `fused` selected between two launch chains of the
+    reference with slightly different rounding; here there is one chain and the flag is ignored."""
+    _run_bf16(gX, 1, M, N, si, steps, eps, _resolve(schedule), mode, workspace)
+
+
+def newton_schulz_resident_e(gX, gA, gA2, gB, gBX, grecip, E, M, N, si, steps=5, eps=1e-7,
+                             schedule=_KELLER, fused=True, mode="bf16", workspace=None):
+    """Batched resident NS over E (M,N) bf16 matrices packed (E*M, N)
+    (ancora/kernels/muon_ns.py:430-468). Each matrix's result is independent of E."""
+    _run_bf16(gX, E, M, N, si, steps, eps, _resolve(schedule), mode, workspace)

@@ -1,0 +1,289 @@
+/*
+ * anc_optim.h — C ABI of libancora_optim.so: the Muon + AdamW optimizer step of
+ * MythosAd/ancora-cutile (ancora/optim + ancora/kernels/muon_ns.py) as hand-written
+ * HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every device pointer crosses the boundary as a raw 64-bit address (uint64_t),
+ *     every size as int64_t, every stream/event as an opaque uint64_t handle
+ *     (0 = the null stream);
+ *   - every entry point returns an int status: 0 = ok, non-zero = error, with a
+ *     human-readable description available from anc_last_error();
+ *   - all launches are asynchronous on the given stream; the library owns no hidden
+ *     state: optimizer state, scratch and partial-sum buffers are caller-owned, so
+ *     the aliasing the reference relies on (p16 IS the model's GEMM weight buffer,
+ *     ancora/model/resident_train.py:96-102) keeps working;
+ *   - bf16 travels as uint16 bit patterns, exactly as in the reference
+ *     (ancora/optim/adamw.py:63-66);
+ *   - results are bitwise reproducible run to run and independent of how tensors are
+ *     batched into launches: fixed tiles, no split-K, no atomics, fixed reduction order.
+ *
+ * Each declaration cites the reference interface (path:line under the reference
+ * repository root) that it replaces.
+ */
+#ifndef ANC_OPTIM_H
+#define ANC_OPTIM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ status */
+
+#define ANC_OK               0
+#define ANC_ERR_HIP          1   /* a HIP runtime call failed                         */
+#define ANC_ERR_ARG          2   /* bad argument: null pointer, misaligned shape, ... */
+#define ANC_ERR_UNSUPPORTED  3   /* valid request outside what the kernels implement  */
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *anc_last_error(void);
+
+/* ABI version: bumped whenever a signature or struct layout below changes. */
+int anc_abi_version(void);
+
+/* ----------------------------------------------------- device and memory ---
+ * Replaces the cuda.bindings driver calls the reference makes directly
+ * (cuMemAlloc/cuMemcpyHtoD/cuMemcpyDtoH/cuMemFree: ancora/optim/adamw.py:51-60,
+ *  ancora/kernels/loss.py:277-294, ancora/model/resident.py:52-94) and its stream
+ * bootstrap (tests/optim/test_adamw.py:14-16). */
+
+typedef struct {
+  int32_t cu_count;          /* compute units                                  */
+  int32_t clock_khz;         /* peak engine clock                              */
+  int32_t mem_clock_khz;     /* peak memory clock                              */
+  int32_t mem_bus_bits;      /* memory bus width                               */
+  int32_t wavefront;         /* lanes per wavefront (64 on gfx950)             */
+  int32_t lds_bytes_per_block;
+  int64_t hbm_bytes;         /* total device memory                            */
+  int64_t l2_bytes;
+  char    name[64];
+  char    arch[64];          /* gcnArchName, e.g. "gfx950:sramecc+:xnack-"     */
+} anc_device_info_t;
+
+int anc_init(int device);                        /* hipSetDevice + arch check (gfx950 only) */
+int anc_device_info(anc_device_info_t *out);
+int anc_malloc(uint64_t *dptr, int64_t bytes);
+int anc_free(uint64_t dptr);
+int anc_host_alloc(void **hptr, int64_t bytes);  /* pinned host memory */
+int anc_host_free(void *hptr);
+int anc_mem_info(int64_t *free_bytes, int64_t *total_bytes);
+/* Fill with a 32-bit pattern using a kernel (safe inside graph capture). */
+int anc_fill_u32(uint64_t dptr, uint32_t value, int64_t n_words, uint64_t stream);
+int anc_memcpy_h2d(uint64_t dst, const void *src, int64_t bytes, uint64_t stream);
+int anc_memcpy_d2h(void *dst, uint64_t src, int64_t bytes, uint64_t stream);
+int anc_memcpy_d2d(uint64_t dst, uint64_t src, int64_t bytes, uint64_t stream);
+int anc_stream_create(uint64_t *stream);
+int anc_stream_destroy(uint64_t stream);
+int anc_stream_sync(uint64_t stream);
+int anc_device_sync(void);
+int anc_event_create(uint64_t *event);
+int anc_event_destroy(uint64_t event);
+int anc_event_record(uint64_t event, uint64_t stream);
+int anc_event_sync(uint64_t event);
+int anc_event_elapsed_ms(uint64_t start, uint64_t stop, float *ms);
+/* Plain streaming copy kernel of n_bytes (multiple of 16): the calibration
+ * reference for HBM traffic counters and the measured copy ceiling. */
+int anc_copy_kernel(uint64_t dst, uint64_t src, int64_t n_bytes, uint64_t stream);
+
+/* --------------------------------------------------------- element types --- */
+#define ANC_F32   0
+#define ANC_BF16  1
+
+/* ------------------------------------------------- step control block -------
+ * 32 bytes in device memory, written by anc_gradnorm_finalize and read by every
+ * update kernel, so that clip and skip decisions never need a host round trip.
+ * No reference counterpart: the reference has no grad-norm, clip or non-finite
+ * guard (its closest pattern is the single-block fixed-order reduction of
+ * ancora/kernels/muon_ns.py:156-165). Passing ctl = 0 to an update kernel means
+ * "clip_scale = 1, never skip". */
+typedef struct {
+  double   sumsq;        /* sum of g*g over every gradient element, fp64          */
+  float    norm;         /* (float)sqrt(sumsq)                                    */
+  float    clip_scale;   /* min(1, max_norm / (norm + eps)); 1 if max_norm <= 0   */
+  uint32_t skip;         /* 1 if sumsq is not finite: update kernels write nothing */
+  uint32_t reserved[3];
+} anc_step_ctl_t;
+
+/* ------------------------------------------------------------ grad-norm ----
+ * Deterministic global gradient norm, no atomics. Stage 1 writes one fp64
+ * partial per ANC_GN_CHUNK-element chunk of the tensor (lane-strided exact
+ * products, wavefront shuffle reduction, fixed LDS tree); chunk boundaries are
+ * fixed relative to the tensor start, so the partials do not depend on the grid
+ * or on which tensors share a launch. Stage 2 reduces the whole partial array
+ * in a fixed order and writes the control block. */
+#define ANC_GN_CHUNK 8192
+int64_t anc_gradnorm_num_partials(int64_t n);
+int anc_gradnorm_partials(uint64_t g, int64_t n, int g_dtype,
+                          uint64_t partials /* double[] */, int64_t part_offset,
+                          uint64_t stream);
+typedef struct {
+  uint64_t g;            /* gradient tensor                                    */
+  int64_t  n;            /* elements                                           */
+  int64_t  chunk0;       /* index of this tensor's first chunk in the launch   */
+  int64_t  part0;        /* index of its first partial in the partial array    */
+  int32_t  dtype;        /* ANC_F32 or ANC_BF16                                */
+  int32_t  pad;
+} anc_gn_desc_t;
+/* One launch over n_tensors tensors described by a device-resident table. */
+int anc_gradnorm_partials_multi(uint64_t desc_table, int32_t n_tensors,
+                                int64_t total_chunks, uint64_t partials,
+                                uint64_t stream);
+int anc_gradnorm_finalize(uint64_t partials, int64_t n_partials,
+                          float max_norm, float eps,
+                          uint64_t ctl /* anc_step_ctl_t* */, uint64_t stream);
+
+/* ---------------------------------------------------------------- AdamW ----
+ * Replaces the `_adamw` cuda-tile kernel and its launch tuple
+ * (g, m, v, p32, p16, OTM, beta1, beta2, eps, lr, wd, ibc1, ibc2)
+ * (ancora/optim/adamw.py:23-41, launched at :94-97, also from
+ *  ancora/model/resident_train.py:350-353, resident_model.py:162-166,
+ *  ancora/kernels/moe.py:586-588,603-604).
+ *
+ * One pass per element: read g (fp32 or bf16), m, v, p32; write m, v, p32 and the
+ * bf16 copy p16. All scalars are rounded to fp32 once on the host, so the kernel
+ * reproduces a numpy fp32 evaluation operation by operation (no FMA contraction,
+ * correctly rounded divide and sqrt).
+ *
+ *   form ANC_ADAMW_FORM_DIV  (numpy oracle, tests/optim/test_adamw.py:37-41):
+ *       g' = g * clip_scale
+ *       m  = beta1*m + omb1*g'            v = beta2*v + (omb2*g')*g'
+ *       p  = p - lr * ((m/bc1) / (sqrt(v/bc2) + eps) + wd*p)
+ *   form ANC_ADAMW_FORM_IBC  (the reference kernel, ancora/optim/adamw.py:34-37):
+ *       m  = beta1*m + (1.0f-beta1)*g'    v = beta2*v + ((1.0f-beta2)*g')*g'
+ *       p  = p - lr * ((m*bc1) / (sqrt(v*bc2) + eps) + wd*p)     (bc = 1/(1-beta^t))
+ *
+ * p16 = round-to-nearest-even bf16 of the new p (ancora/optim/adamw.py:41,63-65), or,
+ * with sr != 0, the stochastic rounding (bits(p) + dither) >> 16 with the counter-based
+ * dither of ancora/kernels/fused.py:154-161 keyed on (row = i/64, col = i%64, seed),
+ * non-finite values passed through unchanged. */
+#define ANC_ADAMW_FORM_DIV 0
+#define ANC_ADAMW_FORM_IBC 1
+typedef struct {
+  float   beta1, beta2;
+  float   omb1, omb2;    /* fp32(1-beta1), fp32(1-beta2) — used by FORM_DIV only   */
+  float   eps, lr;
+  float   bc1, bc2;      /* FORM_DIV: fp32(1-beta^t); FORM_IBC: fp32(1/(1-beta^t)) */
+  int32_t form;
+  int32_t sr;            /* 0 = RNE downcast, 1 = stochastic rounding              */
+  uint32_t seed_base;    /* per-step SR seed; a tensor's seed is seed_base + its own */
+  uint32_t reserved;
+} anc_adamw_hyper_t;
+
+int anc_adamw(uint64_t g, uint64_t m, uint64_t v, uint64_t p32, uint64_t p16,
+              int64_t n /* multiple of 64, as ancora/optim/adamw.py:20,79 */,
+              int g_dtype, const anc_adamw_hyper_t *h, float wd, uint32_t seed,
+              uint64_t ctl, uint64_t stream);
+
+typedef struct {
+  uint64_t g, m, v, p32, p16;
+  int64_t  n;            /* elements, multiple of 64                            */
+  int64_t  blk0;         /* index of this tensor's first block in the launch    */
+  float    wd;           /* per-tensor weight decay (0 for no_decay names)      */
+  uint32_t seed;         /* per-tensor SR seed offset (added to seed_base)      */
+  int32_t  g_dtype;
+  int32_t  pad;
+} anc_adamw_desc_t;
+int64_t anc_adamw_num_blocks(int64_t n);   /* blocks one tensor of n elements occupies */
+/* The whole AdamW parameter group in ONE launch (the reference launches once per
+ * tensor, ancora/optim/adamw.py:92-97). Per-element results are identical to anc_adamw. */
+int anc_adamw_multi(uint64_t desc_table, int32_t n_tensors, int64_t total_blocks,
+                    const anc_adamw_hyper_t *h, uint64_t ctl, uint64_t stream);
+
+/* p16 = bf16(p32): replaces `_cast_bf16` (ancora/kernels/fused.py:285-290). */
+int anc_cast_bf16(uint64_t p32, uint64_t p16, int64_t n, int sr, uint32_t seed,
+                  uint64_t stream);
+
+/* ------------------------------------------------------ Muon elementwise ---
+ * Momentum + Nesterov look-ahead, replaces `_muon_mom`, `_muon_mom_t`, `_e_muon_mom`
+ * (ancora/kernels/muon_ns.py:177-186, 206-217, 409-418; numpy form
+ *  ancora/optim/muon.py:303-305):
+ *     g' = g*clip_scale;  buf = mom*buf + g';  u = nesterov ? g' + mom*buf : buf
+ * buf is (K,N) fp32, g is (K,N) fp32 or bf16; u is written as (K,N), or as (N,K) when
+ * transpose_out != 0 (tall weights enter Newton-Schulz transposed,
+ * ancora/optim/muon.py:72-74), with dtype u_dtype: ANC_BF16 (RNE, the reference's
+ * storage) or ANC_F32 (this library's precise chain). K and N multiples of 64. */
+int anc_muon_momentum(uint64_t buf, uint64_t g, uint64_t u, int64_t K, int64_t N,
+                      float mom, int nesterov, int transpose_out,
+                      int g_dtype, int u_dtype, uint64_t ctl, uint64_t stream);
+
+/* Master update + bf16 refresh, replaces `_muon_update`, `_muon_update_cast`,
+ * `_muon_update_cast_t`, `_e_muon_update` (ancora/kernels/muon_ns.py:189-195,
+ * 220-242, 421-427; numpy form ancora/optim/muon.py:308-309):
+ *     p32 = p32 - lr_scale*O;   p16 = bf16(p32)   (RNE, or SR keyed as for AdamW)
+ * O is (K,N), or (N,K) when transpose_in != 0; o_dtype ANC_BF16 or ANC_F32.
+ * p16 = 0 skips the bf16 refresh. */
+int anc_muon_update(uint64_t p32, uint64_t p16, uint64_t O, int64_t K, int64_t N,
+                    float lr_scale, int transpose_in, int o_dtype,
+                    int sr, uint32_t seed, uint64_t ctl, uint64_t stream);
+
+typedef struct {
+  uint64_t buf, g, p32, p16;   /* per-weight state, (K,N) row-major               */
+  uint64_t u;                  /* this weight's slice of the packed NS batch      */
+  int32_t  K, N;
+  int32_t  transpose;          /* 1 for tall weights (K > N)                      */
+  int32_t  g_dtype;
+  int32_t  scale_idx;          /* which of the launch's lr_scale values applies   */
+  uint32_t seed;               /* per-weight SR seed offset (added to seed_base)  */
+  int64_t  tile0;              /* index of this weight's first 4096-element block */
+} anc_muon_desc_t;
+#define ANC_MUON_MAX_SCALES 8
+/* All weights of a packed batch in ONE launch each (the reference launches once per
+ * weight, ancora/optim/muon.py:261-276). Per-element results equal the single calls. */
+int anc_muon_momentum_multi(uint64_t desc_table, int32_t n_weights, int64_t total_tiles,
+                            float mom, int nesterov, int u_dtype,
+                            uint64_t ctl, uint64_t stream);
+/* lr_scales: host array of ANC_MUON_MAX_SCALES values lr * sqrt(max(1, K/N))
+ * (ancora/optim/muon.py:308), one per distinct weight shape class; the table itself
+ * holds nothing that changes from step to step. */
+int anc_muon_update_multi(uint64_t desc_table, int32_t n_weights, int64_t total_tiles,
+                          const float *lr_scales, int o_dtype, int sr, uint32_t seed_base,
+                          uint64_t ctl, uint64_t stream);
+
+/* bf16 transpose XT(N,M) = X(M,N)^T: replaces `_transpose_mat`
+ * (ancora/kernels/muon_ns.py:198-203) and, batched over E, `_transpose_e`
+ * (ancora/kernels/moe.py:370-377). M, N multiples of 64. */
+int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
+                       uint64_t stream);
+
+/* --------------------------------------------------------- Newton-Schulz ---
+ * Replaces the chains `newton_schulz_resident` / `newton_schulz_resident_e`
+ * (ancora/kernels/muon_ns.py:245-283, 430-468) and the kernels they launch
+ * (`_fro_recip`, `_scale`, `_gemm_nt_tril`, `_gemm_axpy_tril`, `_mirror`,
+ *  `_gemm_axpy_bf16` and their `_e_` twins, :68-174, 293-406); numpy form
+ * ancora/optim/muon.py:67-80 and tests/kernels/_probe_polar_express_device.py:27-34.
+ *
+ * X holds E matrices (M,N), M <= N, packed (E*M, N) row-major, fp32; it is
+ * overwritten with the orthogonalised result. Per matrix:
+ *     X = X / (||X||_F + eps)
+ *     for k < steps: (a,b,c) = coef[3k..3k+2];  A = X X^T;  B = b A + c A A;  X = a X + B X
+ *
+ *   ANC_NS_BF16       GEMM operands rounded to bf16 at the matrix-core input, fp32
+ *                     accumulate (MFMA); the iterate and the diagonals of A and B are
+ *                     carried in fp32, and the last two iterations add the bf16
+ *                     residual of X as extra accumulation terms.
+ *   ANC_NS_BF16_FAST  as ANC_NS_BF16 without the residual terms (15 GEMM passes).
+ *   ANC_NS_FP32       every product in fp32 (validation mode).
+ *
+ * M and N must be multiples of 128 (the reference's tile alignment,
+ * ancora/optim/muon.py:98). workspace must hold anc_ns_workspace_bytes(E,M,N,mode)
+ * bytes; the chain keeps nothing in it between calls. */
+#define ANC_NS_BF16 0
+#define ANC_NS_FP32 1
+#define ANC_NS_BF16_FAST 2
+int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode);
+int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N,
+                   int steps, const float *coef /* host, 3*steps */, float eps,
+                   int mode, uint64_t workspace, int64_t workspace_bytes,
+                   uint64_t stream);
+
+/* fp32 <-> bf16 conversion of packed batches (entry/exit of the bf16-typed
+ * reference drivers): dst_f32 = float(src_bf16); dst_bf16 = RNE(src_f32). */
+int anc_bf16_to_f32(uint64_t src, uint64_t dst, int64_t n, uint64_t stream);
+int anc_f32_to_bf16(uint64_t src, uint64_t dst, int64_t n, uint64_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ANC_OPTIM_H */

@@ -1,0 +1,29 @@
+"""CPU restatement (numpy) of the reference's Muon + AdamW optimizer step.
+
+TEST INFRASTRUCTURE ONLY. Nothing in the product package imports this directory; it is
+used by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of bench.py, and
+only as the checker or the timed baseline, never as the thing shipped.
+
+Every function cites the reference lines (path:line under the reference repository
+root) it restates; the reference itself cannot be imported (its modules import
+cuda.tile and a Windows-only ancora.env at module top), so the restatement was written
+from the source text.
+
+How each function is pinned (see tests/test_oracle_*.py):
+  adamw_step_div / adamw_step_ibc   reference-held case of tests/optim/test_adamw.py:19-43
+                                    (seed 0, 5 steps, rel < 1e-5 between the two forms);
+                                    closed forms: t=1 gives dp = -lr*g/(|g|+eps) - lr*wd*p,
+                                    g=0 decays m and v only, an fp64 evaluation agrees to 1e-6
+  bf16_rne_bits                     exhaustive halfway/tie cases and a value-level definition
+                                    (nearest bf16, ties to even) by brute force over candidates
+  sr_dither / bf16_sr_bits          exact-grid invariance and unbiasedness over 400 seeds
+                                    (tests/kernels/_probe_sr_ops.py:41-66), hand-computed hash
+  gradnorm_f64 / gradnorm_fixed     closed forms (constant vectors, 3-4-5), fsum brute force,
+                                    the two agree to 1 ulp
+  newton_schulz5 / host_ns          SVD cross-check U p(S) V^T, transpose equivariance, scale
+                                    invariance, zero input, ortho_err(PE5) < ortho_err(Keller5)
+                                    (tests/kernels/_probe_polar_express_device.py:83)
+  muon_step / hybrid routing        table-driven over the Qwen3 / MoE name lists, shape scale
+                                    sqrt(max(1, rows/cols)) on square, wide and tall weights
+No function here is "parity unpinned".
+"""

@@ -1,0 +1,152 @@
+"""End-to-end GPU parity of the hybrid step (Muon on 2-D matrices, AdamW on the rest)."""
+import numpy as np
+import pytest
+
+from oracle.adamw_ref import AdamWRef
+from oracle.muon_ref import MuonRef, PE_SCHEDULE, default_is_muon as ref_is_muon
+from oracle.bf16_ref import bf16_rne_bits, bits_to_f32
+from util import max_ulp, rel_fro, bits_equal, bf16_grad
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config1_minimal_hybrid_step(gpu):
+    """BASELINE config 1: AdamW on a 1024x1024 weight (routed by name) + a 1024 gain, Muon on a
+    1024x1024 weight; bf16 grads ~N(0,1e-3); 5 Polar-Express iterations; seed 0; step 1."""
+    from ancora_cutile_amd import HybridOptimizer, PE_SCHEDULE as PE
+    rng = np.random.default_rng(0)
+    params = {"embed": (0.02 * rng.standard_normal((1024, 1024))).astype(np.float32),
+              "final_norm": (1 + 0.05 * rng.standard_normal(1024)).astype(np.float32),
+              "layer0.q_proj": (0.02 * rng.standard_normal((1024, 1024))).astype(np.float32)}
+    gb, g = {}, {}
+    for n, p in params.items():
+        gb[n], g[n] = bf16_grad(rng, p.shape, 1e-3)
+    opt = HybridOptimizer(params, muon_kw=dict(schedule=PE),
+                          adamw_kw=dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.1),
+                          grad_dtype=np.uint16)
+    assert opt.routing() == {"muon": ["layer0.q_proj"], "adamw": ["embed", "final_norm"]}
+    opt.step(gb, 0)
+    ar = AdamWRef({n: params[n] for n in ("embed", "final_norm")}, lr=3e-4, betas=(0.9, 0.95),
+                  eps=1e-8, wd=0.1, no_decay=("final_norm",))
+    ar.step(g)
+    mr = MuonRef({"layer0.q_proj": params["layer0.q_proj"]}, lr=0.02, momentum=0.95, sched=PE_SCHEDULE)
+    mr.step(g)
+    am = opt.adamw.master()
+    for n in ("embed", "final_norm"):
+        assert max_ulp(am[n], ar.st[n]["p"]) == 0
+    mm = opt.muon.master()["layer0.q_proj"]
+    # the update direction (W0 - W1)/lr is the orthogonalised momentum: 2e-3 bar
+    upd_got = (params["layer0.q_proj"].astype(np.float64) - mm) / 0.02
+    upd_ref = (params["layer0.q_proj"].astype(np.float64) - mr.w["layer0.q_proj"]) / 0.02
+    assert rel_fro(upd_got, upd_ref) < 2.5e-3       # 2e-3 chain + fp32 rounding of W - lr*O
+    assert bits_equal(opt.muon.momentum_buffers()["layer0.q_proj"], mr.buf["layer0.q_proj"])
+    w = opt.weights()
+    assert np.array_equal(w["embed"], bits_to_f32(bf16_rne_bits(am["embed"])).reshape(1024, 1024))
+    opt.free()
+
+
+def test_guarded_step_clips_and_skips(gpu):
+    from ancora_cutile_amd import HybridOptimizer
+    rng = np.random.default_rng(1)
+    params = {"embed": rng.standard_normal((128, 64)).astype(np.float32),
+              "norm": np.ones(64, np.float32),
+              "l0.up_proj": (0.02 * rng.standard_normal((128, 256))).astype(np.float32),
+              "l0.down_proj": (0.02 * rng.standard_normal((256, 128))).astype(np.float32)}
+    grads = {n: rng.standard_normal(p.shape).astype(np.float32) for n, p in params.items()}
+    opt = HybridOptimizer(params, max_grad_norm=1.0)
+    opt.step(grads, 0)
+    assert not opt.last_skipped and 0 < opt.last_ctl["clip_scale"] < 1
+    want = np.sqrt(sum(float(np.sum(g.astype(np.float64) ** 2)) for g in grads.values()))
+    assert abs(opt.last_ctl["norm"] - want) / want < 1e-6
+    snap = (opt.muon.master(), opt.adamw.master(), opt.muon.momentum_buffers())
+    bad = {n: g.copy() for n, g in grads.items()}
+    bad["l0.up_proj"][5, 5] = np.nan
+    opt.step(bad, 0)
+    assert opt.last_skipped and opt.adamw.t == 1 and opt.muon.engine.t == 1
+    now = (opt.muon.master(), opt.adamw.master(), opt.muon.momentum_buffers())
+    for a, b in zip(snap, now):
+        for n in a:
+            assert bits_equal(a[n], b[n])
+    opt.free()
+
+
+def test_descent_on_quadratic(gpu):
+    """The pattern of tests/kernels/_probe_device_muon.py:72-101: Muon steps on 0.5*||W-T||^2
+    drive the loss below 20% of its start, on square, wide and tall weights."""
+    from ancora_cutile_amd import Muon, PE_SCHEDULE as PE
+    rng = np.random.default_rng(2)
+    shapes = {"a": (128, 128), "b": (128, 256), "c": (256, 128)}
+    W = {n: (0.05 * rng.standard_normal(s)).astype(np.float32) for n, s in shapes.items()}
+    T = {n: (0.05 * rng.standard_normal(s)).astype(np.float32) for n, s in shapes.items()}
+    opt = Muon(W, lr=0.01, schedule=PE)
+    loss0 = {n: 0.5 * float(np.sum((W[n] - T[n]) ** 2)) for n in W}
+    for _ in range(30):
+        cur = opt.master()
+        opt.step({n: cur[n] - T[n] for n in W}, 0)
+    cur = opt.master()
+    for n in W:
+        assert 0.5 * float(np.sum((cur[n] - T[n]) ** 2)) < 0.2 * loss0[n]
+    opt.free()
+
+
+def test_chunk_and_scope_are_bitwise_neutral(gpu):
+    """tests/training/test_batched_proj_muon.py:74: per-layer buckets == global batches, bitwise."""
+    from ancora_cutile_amd import BatchedProjMuon, DevBuf, PE_SCHEDULE as PE
+    rng = np.random.default_rng(3)
+    shapes = [(128, 128), (128, 256), (256, 128), (128, 128), (256, 128), (128, 256), (128, 128)]
+    W0 = [(0.02 * rng.standard_normal(s)).astype(np.float32) for s in shapes]
+    G = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+
+    def run(**kw):
+        ws = [dict(buf=DevBuf.zeros(s, np.float32), p32=DevBuf(w), p16=DevBuf.zeros(s, np.uint16),
+                   G=DevBuf(g), K=s[0], N=s[1], lid=i // 2) for i, (s, w, g) in enumerate(zip(shapes, W0, G))]
+        opt = BatchedProjMuon(ws, **kw)
+        for _ in range(2):
+            opt.step(0, lr=0.02, schedule=PE)
+        out = [(w["p32"].to_numpy(), w["p16"].to_numpy(), w["buf"].to_numpy()) for w in ws]
+        opt.free()
+        for w in ws:
+            for k in ("buf", "p32", "p16", "G"):
+                w[k].free()
+        return out
+
+    base = run(chunk=8)
+    for kw in (dict(chunk=1), dict(chunk=2, scope=1), dict(chunk=None, scope=2)):
+        other = run(**kw)
+        for a, b in zip(base, other):
+            for x, y in zip(a, b):
+                assert bits_equal(x, y)
+
+
+def test_expert_optimizer(gpu):
+    """Stacked [E,K,N] experts: Muon per slice, idle experts (zero grad) leave their weights
+    unchanged at step 1, router on AdamW with wd=0, transposed copies refreshed."""
+    from ancora_cutile_amd import ExpertOptimizer, DevBuf, PE_SCHEDULE as PE
+    from oracle.muon_ref import muon_momentum, host_ns, muon_update
+    rng = np.random.default_rng(4)
+    E, H = 4, 128
+    W = {n: (0.02 * rng.standard_normal((E, H, H))).astype(np.float32)
+         for n in ("gate_proj", "up_proj", "down_proj")}
+    router = (0.02 * rng.standard_normal((H, 16))).astype(np.float32)
+    G = {n: rng.standard_normal((E, H, H)).astype(np.float32) for n in W}
+    for n in G:
+        G[n][2] = 0
+    Gd = {n: DevBuf(g.reshape(E * H, H)) for n, g in G.items()}
+    rg = rng.standard_normal((H, 16)).astype(np.float32)
+    rgd = DevBuf(rg.reshape(-1, 64))
+    opt = ExpertOptimizer(W, router)
+    opt.step(Gd, 0, lr=1e-3, muon_lr=0.02, router_grad=rgd, schedule=PE)
+    m = opt.master()
+    for n in W:
+        assert bits_equal(m[n][2], W[n][2])                       # idle expert untouched
+        _, u = muon_momentum(np.zeros((H, H), np.float32), G[n][0])
+        want = muon_update(W[n][0], host_ns(u, PE_SCHEDULE, 5), 0.02)
+        assert rel_fro((W[n][0] - m[n][0]) / 0.02, (W[n][0] - want) / 0.02) < 2.5e-3
+        s = opt.st[n]
+        p16 = s["p16"].to_numpy().reshape(E, H, H)
+        assert np.array_equal(s["p16T"].to_numpy().reshape(E, H, H), p16.transpose(0, 2, 1))
+        assert bits_equal(p16, bf16_rne_bits(m[n]).reshape(E, H, H))
+    assert not np.array_equal(m["router"], router)
+    for b in list(Gd.values()) + [rgd]:
+        b.free()
+    opt.free()
