@@ -15,10 +15,11 @@
 //   A A = dA^2 + dA F + F dA + F F       only F F is a matrix-core product (bf16 F)
 //   B = dB + Boff                        likewise
 //   B X = dB (.) X + Boff X              dB (.) X is an fp32 row scaling in the epilogue
-// In the last two iterations the X operand additionally carries its bf16 residual
-// (X = Xh + Xl): A gets Xh Xl^T + Xl Xh^T and B X gets Boff Xl as extra accumulation
-// terms. All products are "NT" (both operands K-contiguous): X is kept both as (M,N) and
-// transposed (N,M) bf16 copies, written by the epilogue that produces it.
+// Where the shape needs it (see split_plan below) late iterations additionally carry the
+// bf16 residual of an operand (X = Xh + Xl): A gets Xh Xl^T + Xl Xh^T and B X gets Boff Xl
+// as extra accumulation terms of the same tile. All products are "NT" (both operands
+// K-contiguous): X is kept both as (M,N) and transposed (N,M) bf16 copies, written by the
+// epilogue that produces it.
 //
 // Determinism: one workgroup owns one 128x128 output tile and its whole K loop, terms in
 // a fixed order, K tiles in ascending order; no split-K, no atomics. A matrix's result
@@ -68,6 +69,7 @@ struct NsGemm {
   float ca, cb, cc;
   float *A32;                // (E,M,M) fp32 A            GRAM out, BMAT in
   uint16_t *Fh;              // (E,M,M) bf16 off-diag A   GRAM out
+  uint16_t *Fl, *Bl;         // bf16 residuals of F and Boff; null unless this step splits them
   float *dA;                 // (E,M)   diag A            GRAM out, BMAT in
   uint16_t *Bh;              // (E,M,M) bf16 off-diag B   BMAT out
   float *dB;                 // (E,M)   diag B            BMAT out, BX in
@@ -179,15 +181,22 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
             p.A32[mm + (int64_t)gj * M + gi] = v;
             p.Fh[mm + (int64_t)gj * M + gi] = fh;
           }
+          if (p.Fl != nullptr) {
+            const uint16_t fl =
+                diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v - anc_bf16_bits_to_f32(fh));
+            p.Fl[mm + (int64_t)gi * M + gj] = fl;
+            if (tm != tn) p.Fl[mm + (int64_t)gj * M + gi] = fl;
+          }
           if (diag) p.dA[mv + gi] = v;
         } else if (EPI == EPI_BMAT) {
           const float a = p.A32[mm + (int64_t)gi * M + gj];
           const float di = p.dA[mv + gi], dj = p.dA[mv + gj];
-          uint16_t bh;
+          uint16_t bh, bl = 0;
           if (gi != gj) {
             const float a2 = (v + di * a) + a * dj;
             const float bv = p.cb * a + p.cc * a2;
             bh = (uint16_t)anc_bf16_rne_bits(bv);
+            bl = (uint16_t)anc_bf16_rne_bits(bv - anc_bf16_bits_to_f32(bh));
           } else {
             const float a2 = v + di * di;
             p.dB[mv + gi] = p.cb * di + p.cc * a2;
@@ -195,6 +204,10 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
           }
           p.Bh[mm + (int64_t)gi * M + gj] = bh;
           if (tm != tn) p.Bh[mm + (int64_t)gj * M + gi] = bh;
+          if (p.Bl != nullptr) {
+            p.Bl[mm + (int64_t)gi * M + gj] = bl;
+            if (tm != tn) p.Bl[mm + (int64_t)gj * M + gi] = bl;
+          }
         } else {
           const int64_t o = mn + (int64_t)gi * N + gj;
           const float x = p.X32[o];
@@ -406,9 +419,37 @@ struct Carve {
   }
 };
 
+// Which iterations carry bf16 residual operands. Rounding X to bf16 costs about 1e-3 of
+// relative Frobenius error per late iteration on square Gaussian inputs (less on wide
+// ones, more on small ones); measured against the fp32 numpy chain, 5 Polar-Express steps:
+//   no residuals         1024x1024 2.2e-3   1024x2048 1.4e-3   1024x3072 1.2e-3   256x256 2.8e-3
+//   X in the last two    1024x1024 1.4e-3                                         256x256 2.4e-3
+//   X, F, B in last three 1024x1024 7e-5                                          256x256 3e-4
+// The plan depends on (M, N, steps) only, never on the batch.
+struct SplitPlan {
+  int x_from;    // first iteration whose A and B X products add the residual of X
+  int fb_from;   // first iteration whose A A and B X products add the residuals of F and Boff
+};
+SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
+  SplitPlan sp{steps, steps};
+  if (mode != ANC_NS_BF16) return sp;
+  // The first iterations are insensitive (the singular values are still far below 1, so
+  // B X is a small correction to a X); residuals start at a fixed iteration index.
+  if (M >= 1024) {
+    if (N < 2 * M) sp.x_from = steps - 2 < 3 ? steps - 2 : 3;
+  } else {
+    sp.x_from = sp.fb_from = steps - 3 < 2 ? steps - 3 : 2;
+  }
+  if (sp.x_from < 0) sp.x_from = 0;
+  if (sp.fb_from < 0) sp.fb_from = 0;
+  return sp;
+}
+
 struct Plan {
   int nchunks;
   bool split;
+  SplitPlan sp;
+  uint16_t *Fl, *Bl;
   double *partials;
   float *recip;
   // bf16 modes
@@ -424,7 +465,8 @@ Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int ste
   Plan pl{};
   Carve c(base);
   pl.nchunks = (int)((M * N + ANC_GN_CHUNK - 1) / ANC_GN_CHUNK);
-  pl.split = (mode == ANC_NS_BF16);
+  pl.sp = split_plan(M, N, mode, steps);
+  pl.split = pl.sp.x_from < steps;
   pl.partials = c.take<double>(E * pl.nchunks);
   pl.recip = c.take<float>(E);
   if (mode == ANC_NS_FP32) {
@@ -444,10 +486,13 @@ Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int ste
     pl.A32 = c.take<float>(E * M * M);
     pl.Fh = c.take<uint16_t>(E * M * M);
     pl.Bh = c.take<uint16_t>(E * M * M);
+    if (pl.sp.fb_from < steps) {
+      pl.Fl = c.take<uint16_t>(E * M * M);
+      pl.Bl = c.take<uint16_t>(E * M * M);
+    }
     pl.dA = c.take<float>(E * M);
     pl.dB = c.take<float>(E * M);
   }
-  (void)steps;
   pl.bytes = c.off;
   return pl;
 }
@@ -469,7 +514,8 @@ int check_shape(int64_t E, int64_t M, int64_t N, int mode, const char *who) {
 
 extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode) {
   if (check_shape(E, M, N, mode, "anc_ns_workspace_bytes")) return -1;
-  return make_plan(0, E, M, N, mode, 0).bytes;
+  // sized for any step count: with steps >= 3 every optional buffer of the mode is present
+  return make_plan(0, E, M, N, mode, 64).bytes;
 }
 
 extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int steps,
@@ -495,7 +541,7 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
                      eps, pl.recip);
   ANC_LAUNCH_CHECK();
   const unsigned prep_grid = (unsigned)(E * (M / 64) * (N / 64));
-  const int split_from = pl.split ? (steps >= 2 ? steps - 2 : 0) : steps;   // first split iteration
+  const int split_from = pl.sp.x_from;   // first iteration with X residual terms
 
   if (mode == ANC_NS_FP32) {
     hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
@@ -544,11 +590,14 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
   int cur = 0;
   for (int k = 0; k < steps; ++k) {
     const bool split = k >= split_from;
+    const bool split_fb = k >= pl.sp.fb_from;
     const bool last = k + 1 == steps;
     const bool split_next = !last && (k + 1 >= split_from);
     NsGemm g{};
     g.M = (int)M; g.N = (int)N;
     g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB; g.X32 = X32;
+    g.Fl = split_fb ? pl.Fl : nullptr;
+    g.Bl = split_fb ? pl.Bl : nullptr;
     g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
     // A = X X^T
     NsGemm ga = g;
@@ -564,13 +613,19 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
     // B = b A + c A A
     NsGemm gb = g;
     gb.A[0] = pl.Fh; gb.B[0] = pl.Fh; gb.nterms = 1;
+    if (split_fb) {
+      gb.A[1] = pl.Fh; gb.B[1] = pl.Fl;
+      gb.A[2] = pl.Fl; gb.B[2] = pl.Fh;
+      gb.nterms = 3;
+    }
     gb.K = (int)M; gb.strideA = M * M; gb.strideB = M * M; gb.tiles_m = tM; gb.tiles_n = tM; gb.lower = 1;
     hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb);
     ANC_LAUNCH_CHECK();
     // X = a X + B X
     NsGemm gx = g;
     gx.A[0] = pl.Bh; gx.B[0] = pl.XhT[cur]; gx.nterms = 1;
-    if (split) { gx.A[1] = pl.Bh; gx.B[1] = pl.XlT[cur]; gx.nterms = 2; }
+    if (split) { gx.A[gx.nterms] = pl.Bh; gx.B[gx.nterms] = pl.XlT[cur]; ++gx.nterms; }
+    if (split_fb) { gx.A[gx.nterms] = pl.Bl; gx.B[gx.nterms] = pl.XhT[cur]; ++gx.nterms; }
     gx.K = (int)M; gx.strideA = M * M; gx.strideB = mn; gx.tiles_m = tM; gx.tiles_n = tN; gx.lower = 0;
     gx.Yh = last ? nullptr : pl.Xh[cur ^ 1];
     gx.YhT = last ? nullptr : pl.XhT[cur ^ 1];
