@@ -84,6 +84,8 @@ _PROTOS = {
     "anc_event_sync": (None, [u64]),
     "anc_event_elapsed_ms": (None, [u64, u64, C.POINTER(f32)]),
     "anc_copy_kernel": (None, [u64, u64, i64, u64]),
+    "anc_profile_enable": (None, [C.c_int]),
+    "anc_profile_read": (None, [C.POINTER(f32), C.POINTER(i64)]),
     "anc_gradnorm_num_partials": (i64, [i64]),
     "anc_gradnorm_partials": (None, [u64, i64, C.c_int, u64, i64, u64]),
     "anc_gradnorm_partials_multi": (None, [u64, i32, i64, u64, u64]),
@@ -104,6 +106,8 @@ _PROTOS = {
     "anc_ns_workspace_bytes": (i64, [i64, i64, i64, C.c_int]),
     "anc_ns_batched": (None, [u64, i64, i64, i64, C.c_int, C.POINTER(f32), f32, C.c_int, u64, i64,
                               u64]),
+    "anc_ns_flops": (None, [i64, i64, i64, C.c_int, C.c_int, C.POINTER(C.c_double),
+                            C.POINTER(C.c_double)]),
     "anc_bf16_to_f32": (None, [u64, u64, i64, u64]),
     "anc_f32_to_bf16": (None, [u64, u64, i64, u64]),
 }
@@ -180,6 +184,25 @@ def stream_create():
 
 def stream_sync(stream=0):
     api.anc_stream_sync(int(stream))
+
+
+PROF_KINDS = ("adamw", "gradnorm_partials", "gradnorm_finalize", "muon_momentum", "muon_update",
+              "ns_fro", "ns_prep", "ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx", "ns_gemm_f32",
+              "misc", "copy")
+
+
+def profile_enable(on=True):
+    init()
+    api.anc_profile_enable(int(bool(on)))
+
+
+def profile_read():
+    """{kind: (milliseconds, launches)} since the last read; synchronises the device."""
+    n = len(PROF_KINDS)
+    ms = (f32 * n)()
+    cnt = (i64 * n)()
+    api.anc_profile_read(ms, cnt)
+    return {k: (float(ms[i]), int(cnt[i])) for i, k in enumerate(PROF_KINDS)}
 
 
 class Event:

@@ -214,6 +214,7 @@ extern "C" int anc_adamw(uint64_t g, uint64_t m, uint64_t v, uint64_t p32, uint6
            h->seed_base + seed};
   const anc_step_ctl_t *c = (const anc_step_ctl_t *)ctl;
   const anc_adamw_hyper_t hh = *h;
+  AncProfScope prof(ANC_PROF_ADAMW, anc_stream(stream));
   dispatch_form_sr(hh.form, hh.sr, [&](auto F, auto S) {
     constexpr int f = decltype(F)::value, s = decltype(S)::value;
     if (g_dtype == ANC_BF16)
@@ -236,6 +237,7 @@ extern "C" int anc_adamw_multi(uint64_t desc_table, int32_t n_tensors, int64_t t
   const anc_adamw_desc_t *tab = (const anc_adamw_desc_t *)desc_table;
   const anc_step_ctl_t *c = (const anc_step_ctl_t *)ctl;
   const anc_adamw_hyper_t hh = *h;
+  AncProfScope prof(ANC_PROF_ADAMW, anc_stream(stream));
   dispatch_form_sr(hh.form, hh.sr, [&](auto F, auto S) {
     constexpr int f = decltype(F)::value, s = decltype(S)::value;
     hipLaunchKernelGGL((k_adamw_multi<f, s>), dim3((unsigned)total_blocks), dim3(kThreads), 0,
@@ -252,6 +254,7 @@ extern "C" int anc_cast_bf16(uint64_t p32, uint64_t p16, int64_t n, int sr, uint
   ANC_REQUIRE((p32 & 15) == 0 && (p16 & 7) == 0, "anc_cast_bf16: misaligned pointers");
   const int64_t blocks = (n + kBlockElems - 1) / kBlockElems;
   ANC_REQUIRE(blocks < (1ll << 31), "anc_cast_bf16: tensor too large for one launch");
+  AncProfScope prof(ANC_PROF_MISC, anc_stream(stream));
   if (sr)
     hipLaunchKernelGGL(k_cast_bf16<1>, dim3((unsigned)blocks), dim3(kThreads), 0, anc_stream(stream),
                        (const float *)p32, (uint16_t *)p16, n, seed);

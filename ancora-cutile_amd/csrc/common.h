@@ -25,6 +25,16 @@ int anc_hip_fail(hipError_t e, const char *what, const char *file, int line);
 
 static inline hipStream_t anc_stream(uint64_t s) { return reinterpret_cast<hipStream_t>(s); }
 
+// Optional per-launch timing (anc_profile_enable): when on, every kernel launch of the
+// library is bracketed by a pair of HIP events on its stream, attributed to a kernel kind.
+void anc_prof_begin(int kind, hipStream_t s);
+void anc_prof_end(hipStream_t s);
+struct AncProfScope {
+  hipStream_t s;
+  AncProfScope(int kind, hipStream_t st) : s(st) { anc_prof_begin(kind, s); }
+  ~AncProfScope() { anc_prof_end(s); }
+};
+
 // ---------------------------------------------------------------- bf16 bits
 // Round-to-nearest-even fp32 -> bf16 as the integer formula the reference uses on
 // the host (ancora/optim/adamw.py:63-65): u + 0x7FFF + ((u >> 16) & 1), then >> 16.

@@ -89,6 +89,7 @@ extern "C" int anc_gradnorm_partials(uint64_t g, int64_t n, int g_dtype, uint64_
   const int64_t chunks = anc_gradnorm_num_partials(n);
   ANC_REQUIRE(chunks < (1ll << 31), "anc_gradnorm_partials: tensor too large for one launch");
   double *out = (double *)partials + part_offset;
+  AncProfScope prof(ANC_PROF_GN_PARTIALS, anc_stream(stream));
   if (g_dtype == ANC_BF16)
     hipLaunchKernelGGL(k_gn_partials<ANC_BF16>, dim3((unsigned)chunks), dim3(kThreads), 0,
                        anc_stream(stream), (const void *)g, n, out);
@@ -106,6 +107,7 @@ extern "C" int anc_gradnorm_partials_multi(uint64_t desc_table, int32_t n_tensor
               "anc_gradnorm_partials_multi: bad arguments");
   ANC_REQUIRE(total_chunks > 0 && total_chunks < (1ll << 31),
               "anc_gradnorm_partials_multi: total_chunks=%lld out of range", (long long)total_chunks);
+  AncProfScope prof(ANC_PROF_GN_PARTIALS, anc_stream(stream));
   hipLaunchKernelGGL(k_gn_partials_multi, dim3((unsigned)total_chunks), dim3(kThreads), 0,
                      anc_stream(stream), (const anc_gn_desc_t *)desc_table, (int)n_tensors,
                      (double *)partials);
@@ -118,6 +120,7 @@ extern "C" int anc_gradnorm_finalize(uint64_t partials, int64_t n_partials, floa
   ANC_REQUIRE(partials != 0 && ctl != 0 && n_partials > 0,
               "anc_gradnorm_finalize: bad arguments (n_partials=%lld)", (long long)n_partials);
   ANC_REQUIRE((ctl & 7) == 0, "anc_gradnorm_finalize: ctl must be 8-byte aligned");
+  AncProfScope prof(ANC_PROF_GN_FINALIZE, anc_stream(stream));
   hipLaunchKernelGGL(k_gn_finalize, dim3(1), dim3(kFinThreads), 0, anc_stream(stream),
                      (const double *)partials, n_partials, max_norm, eps, (anc_step_ctl_t *)ctl);
   ANC_LAUNCH_CHECK();

@@ -327,6 +327,7 @@ extern "C" int anc_muon_momentum(uint64_t buf, uint64_t g, uint64_t u, int64_t K
   const anc_step_ctl_t *c = (const anc_step_ctl_t *)ctl;
   const dim3 grid((unsigned)((K * N) / kBlockElems)), block(kThreads);
   hipStream_t s = anc_stream(stream);
+  AncProfScope prof(ANC_PROF_MUON_MOM, s);
 #define MOM(GD, UD, TR) hipLaunchKernelGGL((k_mom<GD, UD, TR>), grid, block, 0, s, a, mom, nesterov, c)
   const int sel = (g_dtype == ANC_BF16 ? 4 : 0) | (u_dtype == ANC_BF16 ? 2 : 0) | (transpose_out ? 1 : 0);
   switch (sel) {
@@ -351,6 +352,7 @@ extern "C" int anc_muon_update(uint64_t p32, uint64_t p16, uint64_t O, int64_t K
   const anc_step_ctl_t *c = (const anc_step_ctl_t *)ctl;
   const dim3 grid((unsigned)((K * N) / kBlockElems)), block(kThreads);
   hipStream_t s = anc_stream(stream);
+  AncProfScope prof(ANC_PROF_MUON_UPD, s);
 #define UPD(OD, SR, TR) hipLaunchKernelGGL((k_upd<OD, SR, TR>), grid, block, 0, s, a, c)
   const int sel = (o_dtype == ANC_BF16 ? 4 : 0) | (sr ? 2 : 0) | (transpose_in ? 1 : 0);
   switch (sel) {
@@ -373,6 +375,7 @@ extern "C" int anc_muon_momentum_multi(uint64_t desc_table, int32_t n_weights, i
   const anc_muon_desc_t *tab = (const anc_muon_desc_t *)desc_table;
   const anc_step_ctl_t *c = (const anc_step_ctl_t *)ctl;
   const dim3 grid((unsigned)total_tiles), block(kThreads);
+  AncProfScope prof(ANC_PROF_MUON_MOM, anc_stream(stream));
   if (u_dtype == ANC_BF16)
     hipLaunchKernelGGL(k_mom_multi<ANC_BF16>, grid, block, 0, anc_stream(stream), tab, (int)n_weights,
                        mom, nesterov, c);
@@ -396,6 +399,7 @@ extern "C" int anc_muon_update_multi(uint64_t desc_table, int32_t n_weights, int
   const anc_step_ctl_t *c = (const anc_step_ctl_t *)ctl;
   const dim3 grid((unsigned)total_tiles), block(kThreads);
   hipStream_t s = anc_stream(stream);
+  AncProfScope prof(ANC_PROF_MUON_UPD, s);
   const int sel = (o_dtype == ANC_BF16 ? 2 : 0) | (sr ? 1 : 0);
   switch (sel) {
     case 0: hipLaunchKernelGGL((k_upd_multi<ANC_F32, 0>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, c); break;
@@ -414,6 +418,7 @@ extern "C" int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M,
   ANC_REQUIRE(((X | XT) & 7) == 0, "anc_transpose_bf16: pointers must be 8-byte aligned");
   const int64_t blocks = E * (M / kTile) * (N / kTile);
   ANC_REQUIRE(blocks < (1ll << 31), "anc_transpose_bf16: batch too large");
+  AncProfScope prof(ANC_PROF_MISC, anc_stream(stream));
   hipLaunchKernelGGL(k_transpose_bf16, dim3((unsigned)blocks), dim3(kThreads), 0, anc_stream(stream),
                      (const uint16_t *)X, (uint16_t *)XT, (int)M, (int)N);
   ANC_LAUNCH_CHECK();
@@ -425,6 +430,7 @@ extern "C" int anc_bf16_to_f32(uint64_t src, uint64_t dst, int64_t n, uint64_t s
               "anc_bf16_to_f32: bad arguments");
   const int64_t blocks = (n / 4 + kThreads - 1) / kThreads;
   ANC_REQUIRE(blocks < (1ll << 31), "anc_bf16_to_f32: too large");
+  AncProfScope prof(ANC_PROF_MISC, anc_stream(stream));
   hipLaunchKernelGGL(k_bf16_to_f32, dim3((unsigned)blocks), dim3(kThreads), 0, anc_stream(stream),
                      (const uint16_t *)src, (float *)dst, n);
   ANC_LAUNCH_CHECK();
@@ -435,6 +441,7 @@ extern "C" int anc_f32_to_bf16(uint64_t src, uint64_t dst, int64_t n, uint64_t s
               "anc_f32_to_bf16: bad arguments");
   const int64_t blocks = (n / 4 + kThreads - 1) / kThreads;
   ANC_REQUIRE(blocks < (1ll << 31), "anc_f32_to_bf16: too large");
+  AncProfScope prof(ANC_PROF_MISC, anc_stream(stream));
   hipLaunchKernelGGL(k_f32_to_bf16, dim3((unsigned)blocks), dim3(kThreads), 0, anc_stream(stream),
                      (const float *)src, (uint16_t *)dst, n);
   ANC_LAUNCH_CHECK();

@@ -518,6 +518,29 @@ extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int m
   return make_plan(0, E, M, N, mode, 64).bytes;
 }
 
+// Matrix-core work of one chain call: `executed` counts the tiles and terms actually
+// multiplied (symmetric products compute the lower tiles only; residual terms count),
+// `dense` is the textbook steps*(4 M^2 N + 2 M^3) per matrix.
+extern "C" int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
+                            double *executed, double *dense) {
+  if (int rc = check_shape(E, M, N, mode, "anc_ns_flops")) return rc;
+  ANC_REQUIRE(executed != nullptr && dense != nullptr && steps >= 0, "anc_ns_flops: bad arguments");
+  const double m = (double)M, n = (double)N, e = (double)E;
+  *dense = e * steps * (4.0 * m * m * n + 2.0 * m * m * m);
+  if (mode == ANC_NS_FP32) { *executed = *dense; return ANC_OK; }
+  const SplitPlan sp = split_plan(M, N, mode, steps);
+  const double tM = m / BM, tN = n / BN, tile = 2.0 * BM * BN;
+  double ex = 0.0;
+  for (int k = 0; k < steps; ++k) {
+    const bool sx = k >= sp.x_from, sfb = k >= sp.fb_from;
+    ex += tM * (tM + 1) / 2 * (sx ? 3 : 1) * tile * n;                   // A = X X^T
+    ex += tM * (tM + 1) / 2 * (sfb ? 3 : 1) * tile * m;                  // B = b A + c A A
+    ex += tM * tN * (1 + (sx ? 1 : 0) + (sfb ? 1 : 0)) * tile * m;       // X = a X + B X
+  }
+  *executed = e * ex;
+  return ANC_OK;
+}
+
 extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int steps,
                               const float *coef, float eps, int mode, uint64_t workspace,
                               int64_t workspace_bytes, uint64_t stream) {
@@ -534,18 +557,18 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
   const int64_t mn = M * N;
 
   // ---- X /= ||X||_F + eps
-  hipLaunchKernelGGL(k_fro_partials, dim3((unsigned)(E * pl.nchunks)), dim3(kThreads), 0, s, X32, mn,
-                     pl.nchunks, pl.partials);
+  { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_partials, dim3((unsigned)(E * pl.nchunks)), dim3(kThreads), 0, s, X32, mn,
+                     pl.nchunks, pl.partials); }
   ANC_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s, pl.partials, pl.nchunks,
-                     eps, pl.recip);
+  { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s, pl.partials, pl.nchunks,
+                     eps, pl.recip); }
   ANC_LAUNCH_CHECK();
   const unsigned prep_grid = (unsigned)(E * (M / 64) * (N / 64));
   const int split_from = pl.sp.x_from;   // first iteration with X residual terms
 
   if (mode == ANC_NS_FP32) {
-    hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
-                       (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr);
+    { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
+                       (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr); }
     ANC_LAUNCH_CHECK();
     float *cur = X32, *nxt = pl.Yf;
     const unsigned g_mm = (unsigned)(E * (M / BM) * (M / BN)), g_mn = (unsigned)(E * (M / BM) * (N / BN));
@@ -554,17 +577,17 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
       NsGemmF32 g{};
       g.A = cur; g.B = cur; g.K = (int)N; g.nn = 0; g.strideA = mn; g.strideB = mn;
       g.Mo = (int)M; g.No = (int)M; g.out = pl.Af; g.epi = EPI_GRAM;
-      hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mm), dim3(kGemmThreads), 0, s, g);
+      { AncProfScope prof(ANC_PROF_NS_GEMM_F32, s); hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mm), dim3(kGemmThreads), 0, s, g); }
       ANC_LAUNCH_CHECK();
       NsGemmF32 h{};
       h.A = pl.Af; h.B = pl.Af; h.K = (int)M; h.nn = 0; h.strideA = M * M; h.strideB = M * M;
       h.Mo = (int)M; h.No = (int)M; h.cb = b; h.cc = c; h.D = pl.Af; h.out = pl.Bf; h.epi = EPI_BMAT;
-      hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mm), dim3(kGemmThreads), 0, s, h);
+      { AncProfScope prof(ANC_PROF_NS_GEMM_F32, s); hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mm), dim3(kGemmThreads), 0, s, h); }
       ANC_LAUNCH_CHECK();
       NsGemmF32 y{};
       y.A = pl.Bf; y.B = cur; y.K = (int)M; y.nn = 1; y.strideA = M * M; y.strideB = mn;
       y.Mo = (int)M; y.No = (int)N; y.ca = a; y.D = cur; y.out = nxt; y.epi = EPI_BX;
-      hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mn), dim3(kGemmThreads), 0, s, y);
+      { AncProfScope prof(ANC_PROF_NS_GEMM_F32, s); hipLaunchKernelGGL(k_ns_gemm_f32, dim3(g_mn), dim3(kGemmThreads), 0, s, y); }
       ANC_LAUNCH_CHECK();
       float *tmp = cur; cur = nxt; nxt = tmp;
     }
@@ -575,15 +598,15 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
 
   // ---- bf16 matrix-core chain
   if (steps == 0) {
-    hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
-                       (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr);
+    { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
+                       (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr); }
     ANC_LAUNCH_CHECK();
     return ANC_OK;
   }
   const bool split0 = split_from <= 0;
-  hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
+  { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
                      pl.Xh[0], pl.XhT[0], split0 ? pl.Xl[0] : (uint16_t *)nullptr,
-                     split0 ? pl.XlT[0] : (uint16_t *)nullptr);
+                     split0 ? pl.XlT[0] : (uint16_t *)nullptr); }
   ANC_LAUNCH_CHECK();
   const int tM = (int)(M / BM), tN = (int)(N / BN);
   const unsigned g_sym = (unsigned)(E * tM * (tM + 1) / 2), g_mn = (unsigned)(E * tM * tN);
@@ -608,7 +631,7 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
       ga.nterms = 3;
     }
     ga.K = (int)N; ga.strideA = mn; ga.strideB = mn; ga.tiles_m = tM; ga.tiles_n = tM; ga.lower = 1;
-    hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga);
+    { AncProfScope prof(ANC_PROF_NS_GRAM, s); hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga); }
     ANC_LAUNCH_CHECK();
     // B = b A + c A A
     NsGemm gb = g;
@@ -619,7 +642,7 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
       gb.nterms = 3;
     }
     gb.K = (int)M; gb.strideA = M * M; gb.strideB = M * M; gb.tiles_m = tM; gb.tiles_n = tM; gb.lower = 1;
-    hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb);
+    { AncProfScope prof(ANC_PROF_NS_BMAT, s); hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb); }
     ANC_LAUNCH_CHECK();
     // X = a X + B X
     NsGemm gx = g;
@@ -631,7 +654,7 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
     gx.YhT = last ? nullptr : pl.XhT[cur ^ 1];
     gx.Yl = split_next ? pl.Xl[cur ^ 1] : nullptr;
     gx.YlT = split_next ? pl.XlT[cur ^ 1] : nullptr;
-    hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx);
+    { AncProfScope prof(ANC_PROF_NS_BX, s); hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx); }
     ANC_LAUNCH_CHECK();
     cur ^= 1;
   }

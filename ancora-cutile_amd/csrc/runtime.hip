@@ -20,6 +20,59 @@ int anc_hip_fail(hipError_t e, const char *what, const char *file, int line) {
 }
 
 extern "C" const char *anc_last_error(void) { return g_err; }
+
+// ---- per-launch profiler -------------------------------------------------------------
+#include <mutex>
+#include <vector>
+namespace {
+struct ProfRec { int kind; hipEvent_t start, stop; };
+std::mutex g_prof_mu;
+bool g_prof_on = false;
+std::vector<ProfRec> g_prof_recs;
+std::vector<hipEvent_t> g_prof_pool;
+hipEvent_t prof_event() {
+  if (!g_prof_pool.empty()) { hipEvent_t e = g_prof_pool.back(); g_prof_pool.pop_back(); return e; }
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) return nullptr;
+  return e;
+}
+}  // namespace
+
+void anc_prof_begin(int kind, hipStream_t s) {
+  if (!g_prof_on) return;
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  ProfRec r{kind, prof_event(), prof_event()};
+  if (r.start == nullptr || r.stop == nullptr) return;
+  (void)hipEventRecord(r.start, s);
+  g_prof_recs.push_back(r);
+}
+void anc_prof_end(hipStream_t s) {
+  if (!g_prof_on) return;
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  if (!g_prof_recs.empty()) (void)hipEventRecord(g_prof_recs.back().stop, s);
+}
+extern "C" int anc_profile_enable(int on) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  g_prof_on = on != 0;
+  return ANC_OK;
+}
+extern "C" int anc_profile_read(float *ms, int64_t *launches) {
+  ANC_REQUIRE(ms != nullptr && launches != nullptr, "anc_profile_read: null output");
+  ANC_HIP(hipDeviceSynchronize());
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  for (int k = 0; k < ANC_PROF_KINDS; ++k) { ms[k] = 0.0f; launches[k] = 0; }
+  for (const ProfRec &r : g_prof_recs) {
+    float t = 0.0f;
+    if (hipEventElapsedTime(&t, r.start, r.stop) == hipSuccess && r.kind >= 0 && r.kind < ANC_PROF_KINDS) {
+      ms[r.kind] += t;
+      launches[r.kind] += 1;
+    }
+    g_prof_pool.push_back(r.start);
+    g_prof_pool.push_back(r.stop);
+  }
+  g_prof_recs.clear();
+  return ANC_OK;
+}
 extern "C" int anc_abi_version(void) { return 1; }
 
 extern "C" int anc_init(int device) {
@@ -97,6 +150,7 @@ extern "C" int anc_fill_u32(uint64_t dptr, uint32_t value, int64_t n_words, uint
   if (n_words == 0) return ANC_OK;
   int64_t blocks = (n_words + 255) / 256;
   if (blocks > 16384) blocks = 16384;
+  AncProfScope prof(ANC_PROF_MISC, anc_stream(stream));
   hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)blocks), dim3(256), 0, anc_stream(stream),
                      (uint32_t *)dptr, value, n_words);
   ANC_LAUNCH_CHECK();
@@ -197,6 +251,7 @@ extern "C" int anc_copy_kernel(uint64_t dst, uint64_t src, int64_t n_bytes, uint
   int64_t n_vec = n_bytes / 16;
   int64_t blocks = (n_vec + 1023) / 1024;
   ANC_REQUIRE(blocks < (1ll << 31), "anc_copy_kernel: size too large");
+  AncProfScope prof(ANC_PROF_COPY, anc_stream(stream));
   hipLaunchKernelGGL(k_copy16, dim3((unsigned)blocks), dim3(256), 0, anc_stream(stream),
                      (const anc_u32x4 *)src, (anc_u32x4 *)dst, n_vec);
   ANC_LAUNCH_CHECK();

@@ -103,6 +103,14 @@ def ns_workspace_bytes(E, M, N, mode="bf16"):
     return int(n)
 
 
+def ns_flops(E, M, N, steps=5, mode="bf16"):
+    """(executed, dense) matrix-core FLOPs of one chain call over E (M,N) matrices."""
+    _lib.load()
+    ex, de = ctypes.c_double(0), ctypes.c_double(0)
+    api.anc_ns_flops(E, M, N, int(steps), MODES[mode], ctypes.byref(ex), ctypes.byref(de))
+    return ex.value, de.value
+
+
 def ns_batched(X32, E, M, N, si, steps=5, eps=1e-7, schedule=_KELLER, mode="bf16", workspace=None):
     """Native driver: X32 is a DevBuf of E packed (M,N) fp32 matrices, M <= N, both multiples of
     128; overwritten with the orthogonalised result."""

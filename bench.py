@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the Muon + AdamW optimizer step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (config.workload = "qwen3-0.6b-hybrid-step"): the full Qwen3-0.6B-shaped
+parameter set, 596,049,920 parameters -- Muon on the 196 projection matrices
+(q 1024x2048, k/v 1024x1024, o 2048x1024, gate/up 1024x3072, down 3072x1024 per layer),
+AdamW on the tied embedding 151936x1024 and the RMSNorm / q,k-norm gains; fp32 master
+weights, bf16 gradients ~N(0,1e-3) with 1% of rows scaled x100, global grad-norm clip at 1.0,
+stochastic-rounded bf16 weight downcast, 5 Polar-Express Newton-Schulz iterations.
+A step = grad-norm + clip scale + Muon (momentum, NS chain, update) + AdamW, with every
+tensor already resident in HBM when the timed region starts.
+
+Prints ONE JSON line. `value` is milliseconds per step (lower is better). `roofline` is the
+dominant kernel, the bf16 matrix-core GEMM of the Newton-Schulz chain: executed FLOPs over
+the summed duration of its launches, measured with HIP events on the launch stream, against
+the 2.5 PFLOP/s dense bf16 peak. `cpu_baseline` times the numpy restatement of the
+reference's host path on a bounded sample and scales it to the full step.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "Qwen3-0.6B Muon+AdamW step ms; AdamW HBM GB/s; NS-GEMM MFMA util %"
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 matrix-core peak
+PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E peak
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def synth(shapes, seed=0):
+    """Synthetic weights (fp32) and gradients (bf16 bits) of the workload."""
+    from ancora_cutile_amd.bf16 import bf16_bits
+    rng = np.random.default_rng(seed)
+    params, grads = {}, {}
+    for name, shape in shapes.items():
+        n = int(np.prod(shape))
+        if len(shape) == 1:
+            p = (1.0 + 0.05 * rng.standard_normal(n, dtype=np.float32)).reshape(shape)
+        else:
+            p = (0.02 * rng.standard_normal(n, dtype=np.float32)).reshape(shape)
+        g = (1e-3 * rng.standard_normal(n, dtype=np.float32)).reshape(shape)
+        if len(shape) >= 2:                      # 1% of rows carry a x100 outlier scale
+            rows = shape[0]
+            k = max(1, rows // 100)
+            g[rng.choice(rows, k, replace=False)] *= 100.0
+        params[name] = p
+        grads[name] = bf16_bits(g).reshape(shape)
+    return params, grads
+
+
+def cpu_baseline(shapes, lr_adam=3e-4):
+    """Numpy restatement of the reference host path (Muon.step + host_ns, AdamW test-oracle
+    formula) timed on a bounded sample: one matrix of each Newton-Schulz shape and a 16M-element
+    AdamW slice, scaled by the counts of the full parameter set."""
+    from oracle.adamw_ref import adamw_step_div
+    from oracle.muon_ref import muon_momentum, ns_any_shape, muon_update, PE_SCHEDULE
+    try:
+        from threadpoolctl import threadpool_info
+        blas = [i for i in threadpool_info() if i.get("user_api") == "blas"]
+        threads = max([i["num_threads"] for i in blas], default=1)
+    except Exception:
+        threads = 1
+    rng = np.random.default_rng(0)
+    groups = {}
+    adam_elems = 0
+    from ancora_cutile_amd.hybrid import resident_is_muon
+
+    class _Shape:                     # what the routing predicate looks at
+        def __init__(self, shape):
+            self.shape, self.ndim = shape, len(shape)
+
+    for name, shape in shapes.items():
+        if len(shape) == 2 and resident_is_muon(name, _Shape(shape)):
+            groups[shape] = groups.get(shape, 0) + 1
+        else:
+            adam_elems += int(np.prod(shape))
+    total_ms = 0.0
+    for shape, count in groups.items():
+        W = (0.02 * rng.standard_normal(shape)).astype(np.float32)
+        g = (1e-3 * rng.standard_normal(shape)).astype(np.float32)
+        buf = np.zeros(shape, np.float32)
+        t0 = time.perf_counter()
+        buf, u = muon_momentum(buf, g)
+        o = ns_any_shape(u, PE_SCHEDULE, 5)
+        W = muon_update(W, o, 0.02)
+        total_ms += (time.perf_counter() - t0) * 1e3 * count
+    n = 1 << 24
+    p = rng.standard_normal(n).astype(np.float32)
+    m = np.zeros(n, np.float32)
+    v = np.zeros(n, np.float32)
+    g = (1e-3 * rng.standard_normal(n)).astype(np.float32)
+    t0 = time.perf_counter()
+    adamw_step_div(p, m, v, g, lr_adam, 0.9, 0.95, 1e-8, 0.1, 1)
+    total_ms += (time.perf_counter() - t0) * 1e3 * adam_elems / n
+    return {"value": round(total_ms, 1), "unit": "ms/step", "cores": int(threads), "kind": "port",
+            "sample": "numpy oracle: one momentum+NS+update per Muon shape x its count "
+                      f"({', '.join(f'{c}x{s}' for s, c in groups.items())}) + AdamW on a 16.8M-element "
+                      f"slice scaled to {adam_elems} elements; host has {os.cpu_count()} cpus, "
+                      f"{len(os.sched_getaffinity(0))} usable, BLAS threads {threads}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=28, help=argparse.SUPPRESS)   # smaller sets for debugging
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this optimizer step runs on one GPU; --gpus must be 1 "
+                 "(no multi-GPU path is built, see DESIGN.md)")
+
+    from ancora_cutile_amd import HybridOptimizer, DevBuf, PE_SCHEDULE, _lib
+    from ancora_cutile_amd.hybrid import resident_is_muon
+    from ancora_cutile_amd.muon_ns import ns_flops
+    from ancora_cutile_amd.shapes import qwen3_shapes
+
+    _lib.init(0)
+    info = _lib.device_info()
+    log(f"device: {info['name']} {info['arch']} cus={info['cu_count']} clock={info['clock_khz']} kHz")
+    shapes = qwen3_shapes(layers=args.layers)
+    t0 = time.perf_counter()
+    params, grads = synth(shapes)
+    n_params = sum(p.size for p in params.values())
+    log(f"synthetic set: {n_params} params in {len(params)} tensors ({time.perf_counter() - t0:.1f} s)")
+
+    opt = HybridOptimizer(params, is_muon=resident_is_muon,
+                          muon_kw=dict(lr=0.02, momentum=0.95, ns_steps=5, schedule=PE_SCHEDULE,
+                                       sr=True, seed=1),
+                          adamw_kw=dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.1, sr=True, seed=2),
+                          max_grad_norm=1.0, grad_dtype=np.uint16)
+    n_muon = sum(params[n].size for n in opt.muon_names)
+    n_adam = sum(params[n].size for n in opt.adamw_names)
+    del params
+    # gradients resident in HBM before anything is timed
+    gdev = {}
+    for opt_part, names in ((opt.muon, opt.muon_names), (opt.adamw, opt.adamw_names)):
+        for n in names:
+            s = opt_part.st[n]
+            s["g"].upload(grads[n].reshape(s["g"].shape))
+            gdev[n] = s["g"]
+    del grads
+    _lib.stream_sync(0)
+    log(f"muon params {n_muon}, adamw params {n_adam}; state resident")
+
+    for _ in range(args.warmup):
+        opt.step(gdev, 0)
+    _lib.api.anc_device_sync()
+    e0, e1 = _lib.Event(), _lib.Event()
+    t0 = time.perf_counter()
+    e0.record(0)
+    for _ in range(args.steps):
+        opt.step(gdev, 0)
+    e1.record(0)
+    e1.sync()
+    _lib.api.anc_device_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ev_ms = e0.elapsed_ms(e1) / args.steps
+    ms_per_step = max(wall_ms, ev_ms)
+    ctl = opt.last_ctl
+
+    # per-kernel durations: HIP events around every launch, on the launch stream
+    _lib.profile_enable(True)
+    prof_steps = 2
+    for _ in range(prof_steps):
+        opt.step(gdev, 0)
+    prof = _lib.profile_read()
+    _lib.profile_enable(False)
+    kind_ms = {k: v[0] / prof_steps for k, v in prof.items() if v[1]}
+    launches = {k: v[1] // prof_steps for k, v in prof.items() if v[1]}
+
+    executed = dense = 0.0
+    for b in opt.muon.engine.batches:
+        ex, de = ns_flops(b.E, b.M, b.Nn, 5, "bf16")
+        executed += ex
+        dense += de
+    gemm_ms = sum(kind_ms.get(k, 0.0) for k in ("ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx"))
+    gemm_launches = sum(launches.get(k, 0) for k in ("ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx"))
+    achieved = executed / (gemm_ms * 1e-3) / 1e12 if gemm_ms else 0.0
+    adamw_gbps = 28.0 * n_adam / (kind_ms["adamw"] * 1e-3) / 1e9
+    gn_gbps = 2.0 * n_params / (kind_ms["gradnorm_partials"] * 1e-3) / 1e9
+    elem_ms = kind_ms["muon_momentum"] + kind_ms["muon_update"]
+    elem_gbps = 24.0 * n_muon / (elem_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": METRIC, "value": round(ms_per_step, 3), "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "qwen3-0.6b-hybrid-step", "params": n_params, "muon_params": n_muon,
+                   "adamw_params": n_adam, "muon_matrices": sum(b.E for b in opt.muon.engine.batches),
+                   "grads": "bf16 resident in HBM, 1% rows x100", "clip": 1.0,
+                   "weight_downcast": "stochastic bf16", "ns": "5 x polar-express",
+                   "layers": args.layers},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "k_ns_gemm", "launches_per_step": gemm_launches,
+                     "avg_launch_ms": round(gemm_ms / max(1, gemm_launches), 4),
+                     "executed_tflop_per_step": round(executed / 1e12, 3),
+                     "dense_tflop_per_step": round(dense / 1e12, 3)},
+        "adamw_hbm": {"bound": "hbm", "achieved": round(adamw_gbps, 1), "peak": PEAK_HBM_GBPS,
+                      "unit": "GB/s", "frac": round(adamw_gbps / PEAK_HBM_GBPS, 4),
+                      "bytes_per_elem": 28, "ms": round(kind_ms["adamw"], 4)},
+        "gradnorm_hbm": {"achieved": round(gn_gbps, 1), "unit": "GB/s",
+                         "frac": round(gn_gbps / PEAK_HBM_GBPS, 4), "bytes_per_elem": 2,
+                         "ms": round(kind_ms["gradnorm_partials"], 4)},
+        "muon_elementwise_hbm": {"achieved": round(elem_gbps, 1), "unit": "GB/s",
+                                 "frac": round(elem_gbps / PEAK_HBM_GBPS, 4), "bytes_per_param": 24,
+                                 "ms": round(elem_ms, 4)},
+        "ns_mfma_util_pct": round(100 * achieved / PEAK_BF16_TFLOPS, 2),
+        "kernel_ms_per_step": {k: round(v, 4) for k, v in kind_ms.items()},
+        "event_ms_per_step": round(ev_ms, 3), "wall_ms_per_step": round(wall_ms, 3),
+        "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
+        "device": {"name": info["name"], "arch": info["arch"], "cus": info["cu_count"],
+                   "clock_khz": info["clock_khz"]},
+    }
+    opt.free()
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(shapes)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

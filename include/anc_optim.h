@@ -87,6 +87,29 @@ int anc_event_elapsed_ms(uint64_t start, uint64_t stop, float *ms);
  * reference for HBM traffic counters and the measured copy ceiling. */
 int anc_copy_kernel(uint64_t dst, uint64_t src, int64_t n_bytes, uint64_t stream);
 
+/* ------------------------------------------------------------- profiling ----
+ * Per-kernel timing with HIP events on the launch stream, for the benchmarks (the
+ * reference times with perf_counter around cudaStreamSynchronize,
+ * tests/kernels/_bench_ns_fused.py:34-40). While enabled every kernel launch of the
+ * library is bracketed by an event pair; anc_profile_read synchronises the device,
+ * adds the elapsed times per kernel kind and clears the record. */
+#define ANC_PROF_ADAMW        0
+#define ANC_PROF_GN_PARTIALS  1
+#define ANC_PROF_GN_FINALIZE  2
+#define ANC_PROF_MUON_MOM     3
+#define ANC_PROF_MUON_UPD     4
+#define ANC_PROF_NS_FRO       5
+#define ANC_PROF_NS_PREP      6
+#define ANC_PROF_NS_GRAM      7   /* A = X X^T           (bf16 matrix-core GEMM) */
+#define ANC_PROF_NS_BMAT      8   /* B = b A + c A A     (bf16 matrix-core GEMM) */
+#define ANC_PROF_NS_BX        9   /* X = a X + B X       (bf16 matrix-core GEMM) */
+#define ANC_PROF_NS_GEMM_F32 10   /* any GEMM of the fp32 validation chain        */
+#define ANC_PROF_MISC        11   /* casts, conversions, transposes, fill         */
+#define ANC_PROF_COPY        12
+#define ANC_PROF_KINDS       13
+int anc_profile_enable(int on);
+int anc_profile_read(float *ms /* [ANC_PROF_KINDS] */, int64_t *launches /* [ANC_PROF_KINDS] */);
+
 /* --------------------------------------------------------- element types --- */
 #define ANC_F32   0
 #define ANC_BF16  1
@@ -277,6 +300,12 @@ int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N,
                    int steps, const float *coef /* host, 3*steps */, float eps,
                    int mode, uint64_t workspace, int64_t workspace_bytes,
                    uint64_t stream);
+
+/* Matrix-core FLOPs of one anc_ns_batched call: `executed` counts the tiles and terms the
+ * kernels really multiply (lower-triangle tiles of the symmetric products, residual terms),
+ * `dense` is steps*(4 M^2 N + 2 M^3) per matrix. Roofline figures use `executed`. */
+int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
+                 double *executed, double *dense);
 
 /* fp32 <-> bf16 conversion of packed batches (entry/exit of the bf16-typed
  * reference drivers): dst_f32 = float(src_bf16); dst_bf16 = RNE(src_f32). */

@@ -1,0 +1,95 @@
+"""Host-side checks that need no GPU: the C ABI library loads and exports every symbol the
+header declares, struct layouts match, routing, and the absence of any CPU fallback."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "anc_optim.h")
+
+
+def _declared():
+    txt = open(HEADER).read()
+    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+    return sorted(set(re.findall(r"\b(anc_[a-z0-9_]+)\s*\(", txt)))
+
+
+def test_library_exports_every_declared_symbol():
+    from ancora_cutile_amd import _lib
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = _declared()
+    assert len(names) >= 35
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/anc_optim.h but not exported"
+    assert sorted(_lib.EXPORTS) == names, "ctypes prototypes and header disagree"
+    _lib.load()
+    assert _lib.api.anc_abi_version() == 1
+
+
+def test_struct_sizes_match_header():
+    from ancora_cutile_amd import _lib
+    assert ctypes.sizeof(_lib.StepCtl) == 32
+    assert ctypes.sizeof(_lib.AdamWHyper) == 48
+    assert ctypes.sizeof(_lib.AdamWDesc) == 72
+    assert ctypes.sizeof(_lib.GnDesc) == 40
+    assert ctypes.sizeof(_lib.MuonDesc) == 72
+    assert ctypes.sizeof(_lib.DeviceInfo) == 24 + 16 + 128
+
+
+def test_no_gpu_means_error_not_fallback():
+    """Without a GPU the product path must raise; it never computes on the CPU."""
+    from ancora_cutile_amd import _lib
+    if os.path.exists("/dev/kfd"):
+        pytest.skip("a GPU is present")
+    from ancora_cutile_amd import AdamW
+    with pytest.raises(_lib.AncoraError):
+        AdamW({"w": np.zeros((64,), np.float32)})
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "ancora-cutile_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", src, flags=re.M), f
+                assert "oracle/" not in src and "oracle." not in src.replace("oracle. ", ""), f
+
+
+def test_routing_predicates():
+    from ancora_cutile_amd import default_is_muon, resident_is_muon
+    from oracle.muon_ref import default_is_muon as ref
+    names = ["embed", "lm_head", "final_norm", "layer0.input_ln", "layer0.q_norm", "layer0.q_proj",
+             "layer1.o_proj", "layer5.down_proj", "layer1.ffn.router", "layer1.ffn.gate_proj"]
+    for n in names:
+        for arr in (np.zeros((128, 256)), np.zeros(64), np.zeros((4, 128, 128)), np.zeros((1024, 16))):
+            assert default_is_muon(n, arr) == ref(n, arr)
+    assert resident_is_muon("layer1.ffn.gate_proj", np.zeros((16, 128, 128)))
+    assert not resident_is_muon("layer1.ffn.router", np.zeros((1024, 16)))
+    assert not resident_is_muon("layer1.ffn.router", np.zeros((1024, 128)))
+    assert not resident_is_muon("embed", np.zeros((1024, 128)))
+    assert resident_is_muon("layer0.o_proj", np.zeros((2048, 1024)))
+
+
+def test_schedule_toggle_and_constants():
+    from ancora_cutile_amd import muon_ns
+    assert (muon_ns.NTM, muon_ns.NTN, muon_ns.NTK) == (128, 128, 64)
+    prev = muon_ns.set_polar_express(True)
+    assert prev is None and muon_ns._resolve(muon_ns._KELLER) is muon_ns.PE_SCHEDULE
+    assert muon_ns._resolve(None) is None                      # explicit None still means Keller
+    assert muon_ns.set_polar_express(False) is muon_ns.PE_SCHEDULE
+    assert muon_ns._coef_at(muon_ns.PE_SCHEDULE, 7) == muon_ns.PE_SCHEDULE[-1]
+    assert muon_ns._coef_at(None, 0) == (3.4445, -4.7750, 2.0315)
+    from ancora_cutile_amd.adamw import _pick_otm, C
+    assert C == 64 and _pick_otm(256) == 128 and _pick_otm(3) == 1 and _pick_otm(6) == 2
+
+
+def test_bf16_host_helpers_match_oracle():
+    from ancora_cutile_amd.bf16 import bf16_bits, bits_f32
+    from oracle.bf16_ref import bf16_rne_bits, bits_to_f32
+    x = np.random.default_rng(0).standard_normal(1000).astype(np.float32)
+    assert np.array_equal(bf16_bits(x), bf16_rne_bits(x))
+    assert np.array_equal(bits_f32(bf16_bits(x)), bits_to_f32(bf16_rne_bits(x)))
