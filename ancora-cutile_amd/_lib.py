@@ -82,6 +82,7 @@ _PROTOS = {
     "anc_event_destroy": (None, [u64]),
     "anc_event_record": (None, [u64, u64]),
     "anc_event_sync": (None, [u64]),
+    "anc_stream_wait_event": (None, [u64, u64]),
     "anc_event_elapsed_ms": (None, [u64, u64, C.POINTER(f32)]),
     "anc_copy_kernel": (None, [u64, u64, i64, u64]),
     "anc_profile_enable": (None, [C.c_int]),
@@ -219,6 +220,10 @@ class Event:
 
     def sync(self):
         api.anc_event_sync(self.h)
+
+    def wait_on(self, stream):
+        """Make `stream` wait for this event."""
+        api.anc_stream_wait_event(int(stream), self.h)
 
     def elapsed_ms(self, later):
         ms = f32(0)

@@ -24,8 +24,11 @@
 // Determinism: one workgroup owns one 128x128 output tile and its whole K loop, terms in
 // a fixed order, K tiles in ascending order; no split-K, no atomics. A matrix's result
 // does not depend on the batch size E or on its position in the batch. Symmetric outputs
-// (A, B) compute the tiles on or below the diagonal and mirror them, which is bit-identical
-// to computing both halves (same products, same order).
+// (A, B) compute the tiles on or below the diagonal and mirror them; without residual terms
+// that is bit-identical to computing both halves (same products, same order, and an epilogue
+// that is symmetric in (i,j)). With residual terms the two cross products Xh Xl^T and
+// Xl Xh^T enter one accumulator in a fixed order, so elements computed directly inside a
+// diagonal tile differ from their mirror images in the last bits; nothing depends on it.
 //
 // GEMM tile: 128x128x64, 256 lanes = 4 wavefronts in 2x2, each 64x64 as 2x2
 // v_mfma_f32_32x32x16_bf16 blocks (fp32 accumulate). Operand tiles are staged through LDS
@@ -34,49 +37,11 @@
 // Workgroup ids are remapped so that consecutive tiles -- the tiles of one matrix -- run on
 // the same XCD and share its L2.
 #include "reduce.h"
+#include "ns_common.h"
 
 namespace {
 
 using namespace anc_reduce;
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-constexpr int BM = 128, BN = 128, BK = 64;
-constexpr int PITCH = BK + 8;            // bf16 elements per LDS row: 144 bytes
-constexpr int kGemmThreads = 256;
-constexpr int kXcds = 8;
-
-enum { EPI_GRAM = 0, EPI_BMAT = 1, EPI_BX = 2 };
-
-// Workgroup id -> logical tile id such that logical ids [start(x), start(x+1)) run on XCD x
-// (hardware deals consecutive workgroup ids round-robin over the 8 XCDs).
-__device__ __forceinline__ int xcd_remap(int bid, int grid) {
-  const int x = bid % kXcds, q = bid / kXcds;
-  const int base = grid / kXcds, rem = grid % kXcds;
-  return x * base + (x < rem ? x : rem) + q;
-}
-
-struct NsGemm {
-  const uint16_t *A[3];      // term t: rows of the output  (tiles_m*128 rows, ld = K)
-  const uint16_t *B[3];      // term t: columns of the output (tiles_n*128 rows, ld = K)
-  int nterms;
-  int K;
-  int64_t strideA, strideB;  // elements between consecutive matrices
-  int tiles_m, tiles_n;
-  int lower;                 // symmetric output: tiles with tn <= tm only, mirrored
-  int M, N;                  // matrix dims of the chain (A, B are MxM; X is MxN)
-  float ca, cb, cc;
-  float *A32;                // (E,M,M) fp32 A            GRAM out, BMAT in
-  uint16_t *Fh;              // (E,M,M) bf16 off-diag A   GRAM out
-  uint16_t *Fl, *Bl;         // bf16 residuals of F and Boff; null unless this step splits them
-  float *dA;                 // (E,M)   diag A            GRAM out, BMAT in
-  uint16_t *Bh;              // (E,M,M) bf16 off-diag B   BMAT out
-  float *dB;                 // (E,M)   diag B            BMAT out, BX in
-  float *X32;                // (E,M,N) fp32 iterate      BX in/out
-  uint16_t *Yh, *YhT;        // next iterate bf16 (M,N) and (N,M); null on the last step
-  uint16_t *Yl, *YlT;        // bf16 residual copies; null unless the next step splits
-};
 
 template <int EPI>
 __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
@@ -193,7 +158,7 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
           const float di = p.dA[mv + gi], dj = p.dA[mv + gj];
           uint16_t bh, bl = 0;
           if (gi != gj) {
-            const float a2 = (v + di * a) + a * dj;
+            const float a2 = v + (di * a + a * dj);   // symmetric in (i,j)
             const float bv = p.cb * a + p.cc * a2;
             bh = (uint16_t)anc_bf16_rne_bits(bv);
             bl = (uint16_t)anc_bf16_rne_bits(bv - anc_bf16_bits_to_f32(bh));
@@ -513,6 +478,7 @@ int check_shape(int64_t E, int64_t M, int64_t N, int mode, const char *who) {
 }  // namespace
 
 extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode) {
+  mode &= ~ANC_NS_TILE128;
   if (check_shape(E, M, N, mode, "anc_ns_workspace_bytes")) return -1;
   // sized for any step count: with steps >= 3 every optional buffer of the mode is present
   return make_plan(0, E, M, N, mode, 64).bytes;
@@ -523,6 +489,7 @@ extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int m
 // `dense` is the textbook steps*(4 M^2 N + 2 M^3) per matrix.
 extern "C" int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
                             double *executed, double *dense) {
+  mode &= ~ANC_NS_TILE128;
   if (int rc = check_shape(E, M, N, mode, "anc_ns_flops")) return rc;
   ANC_REQUIRE(executed != nullptr && dense != nullptr && steps >= 0, "anc_ns_flops: bad arguments");
   const double m = (double)M, n = (double)N, e = (double)E;
@@ -544,6 +511,8 @@ extern "C" int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode
 extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int steps,
                               const float *coef, float eps, int mode, uint64_t workspace,
                               int64_t workspace_bytes, uint64_t stream) {
+  const bool force_small = (mode & ANC_NS_TILE128) != 0;
+  mode &= ~ANC_NS_TILE128;
   if (int rc = check_shape(E, M, N, mode, "anc_ns_batched")) return rc;
   ANC_REQUIRE(X != 0 && (X & 15) == 0, "anc_ns_batched: X must be a 16-byte aligned device pointer");
   ANC_REQUIRE(steps >= 0 && steps <= 64 && (steps == 0 || coef != nullptr),
@@ -608,7 +577,9 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
                      pl.Xh[0], pl.XhT[0], split0 ? pl.Xl[0] : (uint16_t *)nullptr,
                      split0 ? pl.XlT[0] : (uint16_t *)nullptr); }
   ANC_LAUNCH_CHECK();
-  const int tM = (int)(M / BM), tN = (int)(N / BN);
+  const bool big = !force_small && (M % 256 == 0) && (N % 256 == 0);   // 256x256 tiles, same bits
+  const int tile = big ? 256 : BM;
+  const int tM = (int)(M / tile), tN = (int)(N / tile);
   const unsigned g_sym = (unsigned)(E * tM * (tM + 1) / 2), g_mn = (unsigned)(E * tM * tN);
   int cur = 0;
   for (int k = 0; k < steps; ++k) {
@@ -631,7 +602,11 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
       ga.nterms = 3;
     }
     ga.K = (int)N; ga.strideA = mn; ga.strideB = mn; ga.tiles_m = tM; ga.tiles_n = tM; ga.lower = 1;
-    { AncProfScope prof(ANC_PROF_NS_GRAM, s); hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga); }
+    {
+      AncProfScope prof(ANC_PROF_NS_GRAM, s);
+      if (big) { if (int rc = anc_ns_gemm_big(EPI_GRAM, ga, E, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga);
+    }
     ANC_LAUNCH_CHECK();
     // B = b A + c A A
     NsGemm gb = g;
@@ -642,7 +617,11 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
       gb.nterms = 3;
     }
     gb.K = (int)M; gb.strideA = M * M; gb.strideB = M * M; gb.tiles_m = tM; gb.tiles_n = tM; gb.lower = 1;
-    { AncProfScope prof(ANC_PROF_NS_BMAT, s); hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb); }
+    {
+      AncProfScope prof(ANC_PROF_NS_BMAT, s);
+      if (big) { if (int rc = anc_ns_gemm_big(EPI_BMAT, gb, E, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb);
+    }
     ANC_LAUNCH_CHECK();
     // X = a X + B X
     NsGemm gx = g;
@@ -654,7 +633,11 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
     gx.YhT = last ? nullptr : pl.XhT[cur ^ 1];
     gx.Yl = split_next ? pl.Xl[cur ^ 1] : nullptr;
     gx.YlT = split_next ? pl.XlT[cur ^ 1] : nullptr;
-    { AncProfScope prof(ANC_PROF_NS_BX, s); hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx); }
+    {
+      AncProfScope prof(ANC_PROF_NS_BX, s);
+      if (big) { if (int rc = anc_ns_gemm_big(EPI_BX, gx, E, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx);
+    }
     ANC_LAUNCH_CHECK();
     cur ^= 1;
   }

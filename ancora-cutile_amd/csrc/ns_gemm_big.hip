@@ -1,0 +1,310 @@
+// 256x256x64-tile bf16 matrix-core GEMM of the Newton-Schulz chain for gfx950
+// (the three products A = X X^T, B = b A + c A A, X = a X + B X with their fused
+// epilogues; see ns.hip for the arithmetic).
+//
+// Why this tile. A 128x128 tile moves 64 FLOP per byte staged, which at the matrix-core
+// rate asks more of the per-XCD L2 than it delivers; 256x256 moves 128 FLOP per byte.
+// Eight wavefronts (2 x 4) each own 128x64 of the tile: 8 accumulator blocks of 32x32
+// (128 accumulator registers per lane, two wavefronts per SIMD), 6 operand fragments per
+// 8 MFMAs.
+//
+// Data path. Operand tiles go from HBM/L2 straight into LDS with global_load_lds_dwordx4
+// (no register staging): one instruction moves 8 rows x 128 bytes, a lane writes 16 bytes at
+// lds_base + 16*lane. Rows are 128 bytes with no padding; bank conflicts are avoided by an
+// XOR swizzle of the 16-byte chunk index with bits 1..3 of the row, applied when choosing
+// which global chunk a lane fetches and undone when a fragment is read (16 consecutive rows
+// then cover all 64 banks once). Two 64 KiB stages live in two distinct __shared__ arrays so
+// that the compiler can tell a DMA write to one from a fragment read of the other.
+//
+// Schedule per K tile: start the DMA of the next tile, run 4 k-steps of 8 MFMAs with the
+// fragments of the following k-step already in flight, wait for the DMA and synchronise
+// before the last k-step so that the first fragments of the next tile load under its MFMAs.
+//
+// Epilogue. fp32 operands (A32, X32) are read and written straight from the accumulator
+// layout (128-byte row segments); every bf16 output passes through LDS so that rows and
+// mirrored/transposed rows leave as 16-byte stores.
+//
+// Accumulation order per output element is the same as in the 128x128 kernel (terms in
+// order, k ascending, one accumulator), so both kernels produce the same bits.
+#include "ns_common.h"
+
+namespace {
+
+constexpr int TM = 256, TN = 256, TK = 64;
+constexpr int kStageBytes = (TM + TN) * TK * 2;   // 65536
+constexpr int kAOff = 0, kBOff = TM * TK * 2;     // byte offsets inside a stage
+
+#define LDS3(p) ((__attribute__((address_space(3))) void *)(p))
+#define GLB1(p) ((const __attribute__((address_space(1))) void *)(p))
+
+// vmcnt(0), leave lgkmcnt/expcnt alone (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+constexpr int kBigThreads = 512;     // 8 wavefronts: 2 (rows) x 4 (columns), 128x64 outputs each
+
+struct Frags {
+  bf16x8 a[4], b[2];
+};
+
+__device__ __forceinline__ void load_frags(const unsigned char *stage, int a_base, int b_base,
+                                           int swz, Frags &f) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f.a[i] = *(const bf16x8 *)(stage + kAOff + a_base + i * 4096 + swz);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) f.b[i] = *(const bf16x8 *)(stage + kBOff + b_base + i * 4096 + swz);
+}
+
+__device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
+#pragma unroll
+  for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#ifndef ANC_DBG_NOMFMA
+      acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[bi], f.b[bj], acc[bi][bj], 0, 0, 0);
+#else
+      acc[bi][bj][0] += (float)f.a[bi][0] + (float)f.b[bj][0];
+#endif
+}
+
+// bf16 tile staging through LDS. `v` holds, for the wavefront's 32-row slab, the 16-bit values
+// of its 2 column blocks in accumulator layout (row 8*(r/4) + 4*(lane/32) + r%4, column
+// bj*32 + lane%32). Row-major output: out[row*ld + col]; transposed: outT[col*ldT + row].
+__device__ __forceinline__ void stage_rows(unsigned char *region, const uint16_t (&v)[2][16], int lane,
+                                           uint16_t *out, int64_t ld) {
+  uint16_t *t = (uint16_t *)region;                 // [32][72]
+#pragma unroll
+  for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      t[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 72 + bj * 32 + (lane & 31)] = v[bj][r];
+  __builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0): this wavefront's LDS writes landed
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int idx = p * 64 + lane, row = idx >> 3, c8 = (idx & 7) * 8;
+    const anc_u32x4 q = *(const anc_u32x4 *)(t + row * 72 + c8);
+    *(anc_u32x4 *)(out + (int64_t)row * ld + c8) = q;
+  }
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_wave_barrier();
+}
+__device__ __forceinline__ void stage_cols(unsigned char *region, const uint16_t (&v)[2][16], int lane,
+                                           uint16_t *outT, int64_t ldT) {
+  uint16_t *t = (uint16_t *)region;                 // [64][40]
+#pragma unroll
+  for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      t[(bj * 32 + (lane & 31)) * 40 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)] = v[bj][r];
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int idx = p * 64 + lane, col = idx >> 2, r8 = (idx & 3) * 8;
+    const anc_u32x4 q = *(const anc_u32x4 *)(t + col * 40 + r8);
+    *(anc_u32x4 *)(outT + (int64_t)col * ldT + r8) = q;
+  }
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_wave_barrier();
+}
+
+template <int EPI>
+__global__ void __launch_bounds__(kBigThreads, 1) k_ns_gemm_big(NsGemm p) {
+  __shared__ __attribute__((aligned(1024))) unsigned char stage0[kStageBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char stage1[kStageBytes];
+
+  const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
+  const int tiles_per = p.lower ? p.tiles_m * (p.tiles_m + 1) / 2 : p.tiles_m * p.tiles_n;
+  const int e = L / tiles_per;
+  const int t = L % tiles_per;
+  int tm, tn;
+  if (p.lower) {
+    tm = 0;
+    while ((tm + 1) * (tm + 2) / 2 <= t) ++tm;
+    tn = t - tm * (tm + 1) / 2;
+  } else {
+    tm = t / p.tiles_n;
+    tn = t % p.tiles_n;
+  }
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int K = p.K, nk = K / TK, total = p.nterms * nk;
+
+  // ---- DMA addressing: this wavefront moves rows [wave*32, wave*32+32) of both operand tiles,
+  //      8 rows per instruction; lane -> (row lane/8, physical chunk lane%8). The address is a
+  //      wavefront-uniform base plus one of two per-lane byte offsets (even / odd instruction):
+  //      logical chunk = pchunk ^ (((i*8 + lrow) >> 1) & 7) = pchunk ^ (lrow>>1) ^ 4*(i&1).
+  const int lrow = lane >> 3, pchunk = lane & 7;
+  const uint32_t voff0 = (uint32_t)(lrow * K * 2 + ((pchunk ^ (lrow >> 1)) * 16));
+  const uint32_t voff1 = (uint32_t)(lrow * K * 2 + ((pchunk ^ (lrow >> 1) ^ 4) * 16));
+  const int64_t ubaseA = ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * 32) * K) * 2;   // bytes
+  const int64_t ubaseB = ((int64_t)e * p.strideB + (int64_t)(tn * TN + wave * 32) * K) * 2;
+
+  auto issue = [&](int step, unsigned char *stage) {
+    const int term = step / nk, kt = step - term * nk;
+    const char *Ag = (const char *)p.A[term] + ubaseA + (int64_t)kt * (TK * 2);
+    const char *Bg = (const char *)p.B[term] + ubaseB + (int64_t)kt * (TK * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t ro = (int64_t)(i * 8) * K * 2;
+      const uint32_t vo = (i & 1) ? voff1 : voff0;
+      __builtin_amdgcn_global_load_lds(GLB1(Ag + ro + vo), LDS3(stage + kAOff + (wave * 32 + i * 8) * 128), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(GLB1(Bg + ro + vo), LDS3(stage + kBOff + (wave * 32 + i * 8) * 128), 16, 0, 0);
+    }
+  };
+
+  // ---- fragment addressing
+  const int a_base = (wm * 128 + (lane & 31)) * 128;
+  const int b_base = (wn * 64 + (lane & 31)) * 128;
+  int swz[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) swz[kk] = ((kk * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[bi][bj][r] = 0.0f;
+
+  Frags f0, f1;
+  issue(0, stage0);
+  wait_vm0();
+  __syncthreads();
+  load_frags(stage0, a_base, b_base, swz[0], f0);
+
+  auto body = [&](int step, unsigned char *cur, unsigned char *nxt) {
+    const bool more = step + 1 < total;
+#ifndef ANC_DBG_NODMA
+    if (more) issue(step + 1, nxt);
+#endif
+    load_frags(cur, a_base, b_base, swz[1], f1);
+    mfma8(f0, acc);
+    load_frags(cur, a_base, b_base, swz[2], f0);
+    mfma8(f1, acc);
+    load_frags(cur, a_base, b_base, swz[3], f1);
+    mfma8(f0, acc);
+    wait_vm0();
+    __syncthreads();
+    if (more) load_frags(nxt, a_base, b_base, swz[0], f0);
+    mfma8(f1, acc);
+  };
+  for (int step = 0; step < total; step += 2) {
+    body(step, stage0, stage1);
+    if (step + 1 < total) body(step + 1, stage1, stage0);
+  }
+  __syncthreads();
+
+  // ---- epilogue
+  const int M = p.M, N = p.N;
+  const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
+  unsigned char *region = stage0 + wave * 8192;           // 8 KiB of staging per wavefront
+  const int gi0w = tm * TM + wm * 128, gj0w = tn * TN + wn * 64;
+  const bool mirror = (EPI != EPI_BX) && (tm != tn);
+#pragma unroll
+  for (int bi = 0; bi < 4; ++bi) {
+    uint16_t hv[2][16], lv[2][16];
+    const int gi0 = gi0w + bi * 32;
+    // operands of the epilogue first (all loads in flight together), arithmetic after
+    float in[2][16], drow[16], dcol[2];
+    if (EPI != EPI_GRAM) {
+      const float *src = (EPI == EPI_BMAT) ? p.A32 + mm : p.X32 + mn;
+      const int64_t ld = (EPI == EPI_BMAT) ? M : N;
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int gi = gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          const int gj = gj0w + bj * 32 + (lane & 31);
+          in[bj][r] = src[(int64_t)gi * ld + gj];
+        }
+      const float *dvec = (EPI == EPI_BMAT) ? p.dA + mv : p.dB + mv;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) drow[r] = dvec[gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
+      if (EPI == EPI_BMAT) {
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj) dcol[bj] = dvec[gj0w + bj * 32 + (lane & 31)];
+      }
+    }
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gi = gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int gj = gj0w + bj * 32 + (lane & 31);
+        const float v = acc[bi][bj][r];
+        if (EPI == EPI_GRAM) {
+          const bool diag = gi == gj;
+          const uint16_t fh = diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v);
+          p.A32[mm + (int64_t)gi * M + gj] = v;
+          hv[bj][r] = fh;
+          lv[bj][r] = diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v - anc_bf16_bits_to_f32(fh));
+          if (diag) p.dA[mv + gi] = v;
+        } else if (EPI == EPI_BMAT) {
+          const float a = in[bj][r];
+          const float di = drow[r], dj = dcol[bj];
+          uint16_t bh, bl = 0;
+          if (gi != gj) {
+            const float a2 = v + (di * a + a * dj);   // symmetric in (i,j)
+            const float bv = p.cb * a + p.cc * a2;
+            bh = (uint16_t)anc_bf16_rne_bits(bv);
+            bl = (uint16_t)anc_bf16_rne_bits(bv - anc_bf16_bits_to_f32(bh));
+          } else {
+            const float a2 = v + di * di;
+            p.dB[mv + gi] = p.cb * di + p.cc * a2;
+            bh = 0;
+          }
+          hv[bj][r] = bh;
+          lv[bj][r] = bl;
+        } else {
+          const float y = (p.ca + drow[r]) * in[bj][r] + v;
+          p.X32[mn + (int64_t)gi * N + gj] = y;
+          const uint32_t yh = anc_bf16_rne_bits(y);
+          hv[bj][r] = (uint16_t)yh;
+          lv[bj][r] = (uint16_t)anc_bf16_rne_bits(y - anc_bf16_bits_to_f32(yh));
+        }
+      }
+    }
+    if (EPI == EPI_GRAM) {
+      stage_rows(region, hv, lane, p.Fh + mm + (int64_t)gi0 * M + gj0w, M);
+      if (mirror) stage_cols(region, hv, lane, p.Fh + mm + (int64_t)gj0w * M + gi0, M);
+      if (p.Fl != nullptr) {
+        stage_rows(region, lv, lane, p.Fl + mm + (int64_t)gi0 * M + gj0w, M);
+        if (mirror) stage_cols(region, lv, lane, p.Fl + mm + (int64_t)gj0w * M + gi0, M);
+      }
+    } else if (EPI == EPI_BMAT) {
+      stage_rows(region, hv, lane, p.Bh + mm + (int64_t)gi0 * M + gj0w, M);
+      if (mirror) stage_cols(region, hv, lane, p.Bh + mm + (int64_t)gj0w * M + gi0, M);
+      if (p.Bl != nullptr) {
+        stage_rows(region, lv, lane, p.Bl + mm + (int64_t)gi0 * M + gj0w, M);
+        if (mirror) stage_cols(region, lv, lane, p.Bl + mm + (int64_t)gj0w * M + gi0, M);
+      }
+    } else if (p.Yh != nullptr) {
+      stage_rows(region, hv, lane, p.Yh + mn + (int64_t)gi0 * N + gj0w, N);
+      stage_cols(region, hv, lane, p.YhT + mn + (int64_t)gj0w * M + gi0, M);
+      if (p.Yl != nullptr) {
+        stage_rows(region, lv, lane, p.Yl + mn + (int64_t)gi0 * N + gj0w, N);
+        stage_cols(region, lv, lane, p.YlT + mn + (int64_t)gj0w * M + gi0, M);
+      }
+    }
+  }
+}
+
+}  // namespace
+
+int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
+  ANC_REQUIRE(p.M % TM == 0 && p.N % TN == 0 && p.K % TK == 0,
+              "anc_ns_gemm_big: dims must be multiples of 256");
+  const int64_t tiles_per = p.lower ? (int64_t)p.tiles_m * (p.tiles_m + 1) / 2
+                                    : (int64_t)p.tiles_m * p.tiles_n;
+  const int64_t grid = E * tiles_per;
+  ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
+  const dim3 g((unsigned)grid), b(kBigThreads);
+  if (epi == EPI_GRAM)      hipLaunchKernelGGL(k_ns_gemm_big<EPI_GRAM>, g, b, 0, s, p);
+  else if (epi == EPI_BMAT) hipLaunchKernelGGL(k_ns_gemm_big<EPI_BMAT>, g, b, 0, s, p);
+  else                      hipLaunchKernelGGL(k_ns_gemm_big<EPI_BX>, g, b, 0, s, p);
+  ANC_LAUNCH_CHECK();
+  return ANC_OK;
+}

@@ -222,6 +222,11 @@ extern "C" int anc_event_sync(uint64_t event) {
   ANC_HIP(hipEventSynchronize((hipEvent_t)event));
   return ANC_OK;
 }
+extern "C" int anc_stream_wait_event(uint64_t stream, uint64_t event) {
+  ANC_REQUIRE(event != 0, "anc_stream_wait_event: null event");
+  ANC_HIP(hipStreamWaitEvent(anc_stream(stream), (hipEvent_t)event, 0));
+  return ANC_OK;
+}
 extern "C" int anc_event_elapsed_ms(uint64_t start, uint64_t stop, float *ms) {
   ANC_REQUIRE(start != 0 && stop != 0 && ms != nullptr, "anc_event_elapsed_ms: bad arguments");
   ANC_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));

@@ -50,7 +50,7 @@ class HybridOptimizer:
     def __init__(self, params, is_muon=default_is_muon, no_decay=None, muon_kw=None,
                  adamw_kw=None, si=None, muon_device=False, max_grad_norm=None, guard=False,
                  grad_dtype=np.float32):
-        muon_kw = dict(lr=0.02, momentum=0.95, ns_steps=5, **(muon_kw or {}))
+        muon_kw = {**dict(lr=0.02, momentum=0.95, ns_steps=5), **(muon_kw or {})}
         if muon_device:                      # the reference's switch for GPU Newton-Schulz;
             muon_kw.update(device=True, si=si)   # here the GPU path is the only path
         adamw_kw = adamw_kw or dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.01)
@@ -98,8 +98,11 @@ class HybridOptimizer:
                 g = grads[n]
                 resident[n] = g if isinstance(g, DevBuf) else opt.st[n]["g"]
         self.guard.compute(self._grad_bufs(grads), stream_int)
-        self.muon.launch({n: resident[n] for n in self.muon_names}, stream_int, self.guard)
+        # Muon's per-shape chains fork onto their own streams; AdamW runs beside them
+        self.muon.launch({n: resident[n] for n in self.muon_names}, stream_int, self.guard,
+                         defer_join=True)
         self.adamw.launch({n: resident[n] for n in self.adamw_names}, stream_int, self.guard)
+        self.muon.join(stream_int)
         _lib.stream_sync(stream_int)
         self.last_ctl = self.guard.read(stream_int)
         self.last_skipped = self.last_ctl["skip"]

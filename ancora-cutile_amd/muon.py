@@ -92,8 +92,10 @@ class MuonEngine:
     shape group, which is what 288 GB of HBM is for); `scope=k` sub-groups by lid // k
     (ancora/optim/muon.py:221-222,235). Neither changes any result bit."""
 
+    MAX_STREAMS = 4      # batches are dealt round-robin onto at most this many streams
+
     def __init__(self, weights, momentum=0.95, ns_steps=5, nesterov=True, chunk=None, scope=None,
-                 mode="bf16", sr=False, seed=0, workspace=None):
+                 mode="bf16", sr=False, seed=0, workspace=None, concurrent=True):
         _lib.init()
         self.mom, self.ns, self.nesterov = float(momentum), int(ns_steps), bool(nesterov)
         self.mode, self.sr, self.seed = mode, bool(sr), int(seed)
@@ -122,43 +124,97 @@ class MuonEngine:
                 self.batches.append(_Batch(key[0], key[1], ws[i0:i0 + c]))
         self.groups = groups
         self._own_ws = workspace is None
-        self.ws = NsWorkspace() if workspace is None else workspace
-        self.U = None
-        umax = max(b.E * b.M * b.Nn for b in self.batches) if self.batches else 0
-        wmax = max(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, mode) for b in self.batches) \
-            if self.batches else 0
-        if umax:
-            self.U = DevBuf.empty((umax,), np.float32)
-            self.ws.ensure(wmax)
+        # With its own scratch the engine gives every batch a private packed buffer, workspace
+        # and stream: the chains of different shape groups are independent, so they run
+        # concurrently and fill each other's tails and memory-bound epilogues. A caller-owned
+        # (shared) workspace means one chain at a time on the caller's stream.
+        self.concurrent = bool(concurrent) and self._own_ws and len(self.batches) > 1
+        self.serial = False          # True: keep the private buffers but launch everything on `si`
+        self._forked = False
+        self._streams, self._fork, self._join = [], None, []
+        if self.concurrent:
+            for b in self.batches:
+                b.U = DevBuf.empty((b.E * b.M * b.Nn,), np.float32)
+                b.ws = NsWorkspace()
+                b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, mode))
+                if len(self._streams) < self.MAX_STREAMS:
+                    self._streams.append(_lib.stream_create())
+                self._join.append(_lib.Event())
+            self._fork = _lib.Event()
+            self.ws = None
+            self.U = None
+        else:
+            self.ws = NsWorkspace() if workspace is None else workspace
+            self.U = None
+            umax = max(b.E * b.M * b.Nn for b in self.batches) if self.batches else 0
+            wmax = max(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, mode) for b in self.batches) \
+                if self.batches else 0
+            if umax:
+                self.U = DevBuf.empty((umax,), np.float32)
+                self.ws.ensure(wmax)
+            for b in self.batches:
+                b.U, b.ws = self.U, self.ws
 
     def nbytes(self):
+        if self.concurrent:
+            return sum(b.U.nbytes + b.ws.nbytes() for b in self.batches)
         return (self.U.nbytes if self.U is not None else 0) + self.ws.nbytes()
 
-    def step(self, si, lr=0.02, schedule=_KELLER, guard=None):
-        """One Muon step over every weight. Asynchronous on stream `si`."""
+    def step(self, si, lr=0.02, schedule=_KELLER, guard=None, defer_join=False):
+        """One Muon step over every weight. Asynchronous on stream `si`: the work is ordered
+        after everything already queued on `si`, and (unless defer_join) `si` waits for it."""
         self.t += 1
         schedule = muon_ns._resolve(schedule)
         ctl = 0 if guard is None else guard.ptr
         lr_scales = (ctypes.c_float * MUON_MAX_SCALES)(*[lr * s for s in self.scales])
         seed_base = ((self.seed + 1000003 * self.t) & 0xFFFFFFFF) if self.sr else 0
         coef = muon_ns.coef_array(schedule, self.ns)
-        for b in self.batches:
-            b.build(self.U, self.scale_index)
+        forked = self.concurrent and not self.serial
+        if forked:
+            self._fork.record(si)
+        for i, b in enumerate(self.batches):
+            st = si
+            if forked:
+                st = self._streams[i % len(self._streams)]
+                if i < len(self._streams):
+                    self._fork.wait_on(st)
+            b.build(b.U, self.scale_index)
             api.anc_muon_momentum_multi(b.table.ptr, b.E, b.total_blocks, self.mom,
-                                        int(self.nesterov), F32, ctl, int(si))
-            need = muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self.mode)
-            buf = self.ws.ensure(need)
-            api.anc_ns_batched(self.U.ptr, b.E, b.M, b.Nn, self.ns, coef, 1e-7,
-                               muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(si))
+                                        int(self.nesterov), F32, ctl, int(st))
+            buf = b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self.mode))
+            api.anc_ns_batched(b.U.ptr, b.E, b.M, b.Nn, self.ns, coef, 1e-7,
+                               muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(st))
             api.anc_muon_update_multi(b.table.ptr, b.E, b.total_blocks, lr_scales, F32,
-                                      int(self.sr), seed_base, ctl, int(si))
+                                      int(self.sr), seed_base, ctl, int(st))
+            if forked:
+                self._join[i].record(st)
+        self._forked = forked
+        if forked and not defer_join:
+            self.join(si)
+
+    def join(self, si):
+        """Make stream `si` wait for the per-batch streams of the last step."""
+        if self._forked:
+            for ev in self._join:
+                ev.wait_on(si)
 
     def unstep(self):
         self.t -= 1
 
     def free(self):
+        _lib.api.anc_device_sync()
         for b in self.batches:
             b.free()
+        if self.concurrent:
+            for b in self.batches:
+                b.U.free()
+                b.ws.free()
+            for st in self._streams:
+                api.anc_stream_destroy(st)
+            for ev in self._join + [self._fork]:
+                ev.free()
+            self._streams = []
+            return
         if self.U is not None:
             self.U.free()
             self.U = None
@@ -315,7 +371,7 @@ class Muon:
             if recs else None
         self.last_skipped = False
 
-    def launch(self, grads, stream_int=None, guard=None):
+    def launch(self, grads, stream_int=None, guard=None, defer_join=False):
         si = stream_int if stream_int is not None else (self.si or 0)
         for n, s in self.st.items():
             g = grads[n]
@@ -333,8 +389,12 @@ class Muon:
                                         f"built for {s['g'].dtype}")
                 s["g"].upload(g.reshape(s["E"] * s["K"], s["N"]), si)
         if self.engine is not None:
-            self.engine.step(si, self.lr, self.schedule, guard)
+            self.engine.step(si, self.lr, self.schedule, guard, defer_join)
         return si
+
+    def join(self, si):
+        if self.engine is not None:
+            self.engine.join(si)
 
     def unstep(self):
         if self.engine is not None:

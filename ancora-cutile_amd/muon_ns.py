@@ -30,7 +30,9 @@ PE_SCHEDULE = [(4.0848, -6.8946, 2.9270),
                (2.8769, -3.1427, 1.2046),
                (2.8366, -3.0525, 1.2012)]
 
-MODES = {"bf16": NS_BF16, "bf16_fast": NS_BF16_FAST, "fp32": NS_FP32}
+MODES = {"bf16": NS_BF16, "bf16_fast": NS_BF16_FAST, "fp32": NS_FP32,
+         # same arithmetic forced onto the 128x128-tile kernel (ANC_NS_TILE128), for tests
+         "bf16_tile128": NS_BF16 | 0x100, "bf16_fast_tile128": NS_BF16_FAST | 0x100}
 
 
 def _coef_at(schedule, k):

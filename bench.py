@@ -117,6 +117,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=28, help=argparse.SUPPRESS)   # smaller sets for debugging
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--serial", action="store_true",
+                    help="run the per-shape Newton-Schulz chains on one stream also in the timed steps "
+                         "(what the rocprofv3 kernel summaries under profiles/ were taken with)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this optimizer step runs on one GPU; --gpus must be 1 "
@@ -155,6 +158,7 @@ def main():
     _lib.stream_sync(0)
     log(f"muon params {n_muon}, adamw params {n_adam}; state resident")
 
+    opt.muon.engine.serial = bool(args.serial)
     for _ in range(args.warmup):
         opt.step(gdev, 0)
     _lib.api.anc_device_sync()
@@ -171,7 +175,10 @@ def main():
     ms_per_step = max(wall_ms, ev_ms)
     ctl = opt.last_ctl
 
-    # per-kernel durations: HIP events around every launch, on the launch stream
+    # per-kernel durations: HIP events around every launch, on the launch stream, with the
+    # per-shape chains serialised onto one stream so that a launch is timed running alone
+    opt.muon.engine.serial = True
+    opt.step(gdev, 0)
     _lib.profile_enable(True)
     prof_steps = 2
     for _ in range(prof_steps):
@@ -206,7 +213,9 @@ def main():
                    "layers": args.layers},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                     "kernel": "k_ns_gemm", "launches_per_step": gemm_launches,
+                     "kernel": "k_ns_gemm_big (gram, bmat, bx launches of the Newton-Schulz chain)",
+                     "timed": "HIP events around each launch, chains serialised on one stream",
+                     "launches_per_step": gemm_launches,
                      "avg_launch_ms": round(gemm_ms / max(1, gemm_launches), 4),
                      "executed_tflop_per_step": round(executed / 1e12, 3),
                      "dense_tflop_per_step": round(dense / 1e12, 3)},
@@ -222,6 +231,7 @@ def main():
         "ns_mfma_util_pct": round(100 * achieved / PEAK_BF16_TFLOPS, 2),
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kind_ms.items()},
         "event_ms_per_step": round(ev_ms, 3), "wall_ms_per_step": round(wall_ms, 3),
+        "streams": "serial" if args.serial else "one per Newton-Schulz shape group",
         "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
         "device": {"name": info["name"], "arch": info["arch"], "cus": info["cu_count"],
                    "clock_khz": info["clock_khz"]},

@@ -82,6 +82,9 @@ int anc_event_create(uint64_t *event);
 int anc_event_destroy(uint64_t event);
 int anc_event_record(uint64_t event, uint64_t stream);
 int anc_event_sync(uint64_t event);
+/* Make `stream` wait for `event` (fork/join of the per-shape-group chains onto their own
+ * streams; all streams stay at the default priority). */
+int anc_stream_wait_event(uint64_t stream, uint64_t event);
 int anc_event_elapsed_ms(uint64_t start, uint64_t stop, float *ms);
 /* Plain streaming copy kernel of n_bytes (multiple of 16): the calibration
  * reference for HBM traffic counters and the measured copy ceiling. */
@@ -295,6 +298,9 @@ int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
 #define ANC_NS_BF16 0
 #define ANC_NS_FP32 1
 #define ANC_NS_BF16_FAST 2
+/* Flag OR-ed into a bf16 mode: use the 128x128-tile GEMM kernel even where the 256x256-tile
+ * kernel applies. Both produce the same bits; the flag exists so that tests can show it. */
+#define ANC_NS_TILE128 0x100
 int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode);
 int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N,
                    int steps, const float *coef /* host, 3*steps */, float eps,

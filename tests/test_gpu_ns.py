@@ -90,6 +90,17 @@ def test_batching_is_bitwise_neutral_and_repeatable(gpu):
         assert bits_equal(pair[0], full[4]) and bits_equal(pair[1], full[1])
 
 
+@pytest.mark.parametrize("M,N", [(256, 256), (256, 768), (512, 512), (1024, 1024), (1024, 2048)])
+def test_tile_size_does_not_change_bits(gpu, M, N):
+    """The 256x256-tile kernel and the 128x128-tile kernel accumulate every output element in the
+    same order: identical bits without residual terms. With residual terms only the elements a
+    diagonal tile computes directly instead of mirroring can differ, in the last bits."""
+    rng = np.random.default_rng(M + 7 * N)
+    X = rng.standard_normal((3, M, N)).astype(np.float32)
+    assert bits_equal(run_ns(X, mode="bf16_fast"), run_ns(X, mode="bf16_fast_tile128"))
+    assert rel_fro(run_ns(X, mode="bf16"), run_ns(X, mode="bf16_tile128")) < 2e-4
+
+
 def test_zero_matrix_and_scale_invariance(gpu):
     """A zero gradient (an idle expert) stays zero, no NaN; NS(cX) == NS(X) up to rounding."""
     rng = np.random.default_rng(3)
