@@ -1,0 +1,57 @@
+"""Single-kernel profiling targets for rocprofv3 (the role of the reference's Nsight Compute
+targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
+
+    python3 -m ancora_cutile_amd.prof_target ns M N E [mode] [calls]     Newton-Schulz chain
+    python3 -m ancora_cutile_amd.prof_target adamw NUMEL [calls]         fused AdamW, bf16 grads, SR
+    python3 -m ancora_cutile_amd.prof_target gradnorm NUMEL [calls]      grad-norm partials + finalize
+
+Each target allocates its operands, runs the kernel(s) `calls` times on the null stream and
+synchronises; nothing is checked here (parity lives in tests/).
+"""
+import ctypes
+import sys
+
+import numpy as np
+
+
+def main(argv):
+    from . import DevBuf, StepGuard, _lib
+    from .adamw import hyper_div
+    from .muon_ns import ns_batched, PE_SCHEDULE
+    _lib.init(0)
+    what = argv[0]
+    if what == "ns":
+        M, N, E = int(argv[1]), int(argv[2]), int(argv[3])
+        mode = argv[4] if len(argv) > 4 else "bf16"
+        calls = int(argv[5]) if len(argv) > 5 else 2
+        one = np.random.default_rng(0).standard_normal((M, N)).astype(np.float32)
+        X = DevBuf.empty((E * M, N), np.float32)
+        for e in range(E):
+            X.at_pos(e * M).upload(one)
+        for _ in range(calls):
+            ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
+    elif what == "adamw":
+        n = int(argv[1]) // 64 * 64
+        calls = int(argv[2]) if len(argv) > 2 else 3
+        g = DevBuf.zeros((n,), np.uint16)
+        m, v, p = (DevBuf.zeros((n,), np.float32) for _ in range(3))
+        p16 = DevBuf.zeros((n,), np.uint16)
+        for t in range(1, calls + 1):
+            h = hyper_div(3e-4, 0.9, 0.95, 1e-8, 1000 + t, sr=True, seed_base=t)
+            _lib.api.anc_adamw(g.ptr, m.ptr, v.ptr, p.ptr, p16.ptr, n, _lib.BF16, ctypes.byref(h),
+                               0.1, 0, 0, 0)
+    elif what == "gradnorm":
+        n = int(argv[1])
+        calls = int(argv[2]) if len(argv) > 2 else 3
+        g = DevBuf.zeros((n,), np.uint16)
+        guard = StepGuard(1.0)
+        for _ in range(calls):
+            guard.compute([g], 0)
+    else:
+        raise SystemExit(__doc__)
+    _lib.api.anc_device_sync()
+    print("done")
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])

@@ -158,6 +158,20 @@ def main():
     _lib.stream_sync(0)
     log(f"muon params {n_muon}, adamw params {n_adam}; state resident")
 
+    # one plain 1 GiB copy kernel: the known-size reference that HBM traffic counters
+    # (FETCH_SIZE / WRITE_SIZE) of a profiled run are scaled by
+    cal_a, cal_b = DevBuf.empty((1 << 28,), np.float32), DevBuf.empty((1 << 28,), np.float32)
+    cal_a.fill_zero(0)
+    e0, e1 = _lib.Event(), _lib.Event()
+    _lib.api.anc_copy_kernel(cal_b.ptr, cal_a.ptr, 1 << 30, 0)
+    e0.record(0)
+    _lib.api.anc_copy_kernel(cal_b.ptr, cal_a.ptr, 1 << 30, 0)
+    e1.record(0)
+    e1.sync()
+    copy_gbps = 2 * (1 << 30) / (e0.elapsed_ms(e1) * 1e-3) / 1e9
+    cal_a.free()
+    cal_b.free()
+
     opt.muon.engine.serial = bool(args.serial)
     for _ in range(args.warmup):
         opt.step(gdev, 0)
@@ -201,6 +215,14 @@ def main():
     elem_ms = kind_ms["muon_momentum"] + kind_ms["muon_update"]
     elem_gbps = 24.0 * n_muon / (elem_ms * 1e-3) / 1e9
 
+    # HBM bytes per k_ns_gemm_big launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE on this
+    # same workload (two counter runs scaled by the copy kernel; summary under profiles/)
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "ns_gemm_traffic.json")
+    if args.layers == 28 and os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+
     out = {
         "metric": METRIC, "value": round(ms_per_step, 3), "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
@@ -212,7 +234,7 @@ def main():
                    "weight_downcast": "stochastic bf16", "ns": "5 x polar-express",
                    "layers": args.layers},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
                      "kernel": "k_ns_gemm_big (gram, bmat, bx launches of the Newton-Schulz chain)",
                      "timed": "HIP events around each launch, chains serialised on one stream",
                      "launches_per_step": gemm_launches,
@@ -232,6 +254,7 @@ def main():
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kind_ms.items()},
         "event_ms_per_step": round(ev_ms, 3), "wall_ms_per_step": round(wall_ms, 3),
         "streams": "serial" if args.serial else "one per Newton-Schulz shape group",
+        "copy_kernel_gbps": round(copy_gbps, 1),
         "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
         "device": {"name": info["name"], "arch": info["arch"], "cus": info["cu_count"],
                    "clock_khz": info["clock_khz"]},
