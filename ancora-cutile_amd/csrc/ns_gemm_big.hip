@@ -1,38 +1,40 @@
-// 256x256x64-tile bf16 matrix-core GEMM of the Newton-Schulz chain for gfx950
-// (the three products A = X X^T, B = b A + c A A, X = a X + B X with their fused
-// epilogues; see ns.hip for the arithmetic).
+// Tiled bf16 matrix-core GEMM of the Newton-Schulz chain for gfx950 (the three products
+// A = X X^T, B = b A + c A A, X = a X + B X with their fused epilogues; see ns.hip for the
+// arithmetic), for shapes that are multiples of 256.
 //
-// Why this tile. A 128x128 tile moves 64 FLOP per byte staged, which at the matrix-core
-// rate asks more of the per-XCD L2 than it delivers; 256x256 moves 128 FLOP per byte.
-// Eight wavefronts (2 x 4) each own 128x64 of the tile: 8 accumulator blocks of 32x32
-// (128 accumulator registers per lane, two wavefronts per SIMD), 6 operand fragments per
-// 8 MFMAs.
+// Tile. A 128x128 tile moves 64 FLOP per byte staged, which at the matrix-core rate asks more
+// of the per-XCD L2 than it delivers. Every wavefront here owns 128x64 outputs: 8 accumulator
+// blocks of 32x32 (128 accumulator registers per lane), 6 operand fragments per 8 MFMAs.
+//   symmetric products (A, B): 256x256x64 tile, 8 wavefronts (2 x 4), two 64 KiB LDS stages,
+//     128 FLOP per byte staged, one workgroup per CU;
+//   X = a X + B X: 128x256x32 tile, 4 wavefronts (1 x 4), two 24 KiB stages. Its epilogue moves
+//     12 bytes of HBM traffic per element (fp32 X read and written, two bf16 copies written)
+//     and is the longer phase; the small LDS footprint lets several workgroups share a CU, so
+//     the epilogue of one runs under the MFMAs of another.
 //
-// Data path. Operand tiles go from HBM/L2 straight into LDS with global_load_lds_dwordx4
-// (no register staging): one instruction moves 8 rows x 128 bytes, a lane writes 16 bytes at
-// lds_base + 16*lane. Rows are 128 bytes with no padding; bank conflicts are avoided by an
-// XOR swizzle of the 16-byte chunk index with bits 1..3 of the row, applied when choosing
-// which global chunk a lane fetches and undone when a fragment is read (16 consecutive rows
-// then cover all 64 banks once). Two 64 KiB stages live in two distinct __shared__ arrays so
-// that the compiler can tell a DMA write to one from a fragment read of the other.
+// Data path. Operand tiles go from HBM/L2 straight into LDS with global_load_lds_dwordx4 (no
+// register staging): one instruction moves 1 KiB, a lane writes 16 bytes at lds_base + 16*lane.
+// LDS rows are TK*2 bytes with no padding; bank conflicts are avoided by an XOR swizzle of the
+// 16-byte chunk index with row bits (bits 1..3 for 128-byte rows, bits 2..3 for 64-byte rows),
+// applied when choosing which global chunk a lane fetches and undone when a fragment is read:
+// 16 consecutive rows then cover all 64 banks once. The two stages live in two distinct
+// __shared__ arrays so that the compiler can tell a DMA write to one from a fragment read of
+// the other.
 //
-// Schedule per K tile: start the DMA of the next tile, run 4 k-steps of 8 MFMAs with the
-// fragments of the following k-step already in flight, wait for the DMA and synchronise
-// before the last k-step so that the first fragments of the next tile load under its MFMAs.
+// Schedule per K tile: start the DMA of the next tile, run the k-steps of 8 MFMAs with the
+// fragments of the following k-step already in flight, wait for the DMA and synchronise before
+// the last k-step so that the first fragments of the next tile load under its MFMAs.
 //
 // Epilogue. fp32 operands (A32, X32) are read and written straight from the accumulator
-// layout (128-byte row segments); every bf16 output passes through LDS so that rows and
-// mirrored/transposed rows leave as 16-byte stores.
+// layout (128-byte row segments), all loads of a 32-row slab issued before its arithmetic;
+// every bf16 output passes through LDS so that rows and mirrored/transposed rows leave as
+// 16-byte stores.
 //
-// Accumulation order per output element is the same as in the 128x128 kernel (terms in
-// order, k ascending, one accumulator), so both kernels produce the same bits.
+// Accumulation order per output element is the same in every tile configuration and in the
+// 128x128 kernel of ns.hip (terms in order, k ascending, one accumulator).
 #include "ns_common.h"
 
 namespace {
-
-constexpr int TM = 256, TN = 256, TK = 64;
-constexpr int kStageBytes = (TM + TN) * TK * 2;   // 65536
-constexpr int kAOff = 0, kBOff = TM * TK * 2;     // byte offsets inside a stage
 
 #define LDS3(p) ((__attribute__((address_space(3))) void *)(p))
 #define GLB1(p) ((const __attribute__((address_space(1))) void *)(p))
@@ -40,18 +42,17 @@ constexpr int kAOff = 0, kBOff = TM * TK * 2;     // byte offsets inside a stage
 // vmcnt(0), leave lgkmcnt/expcnt alone (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-constexpr int kBigThreads = 512;     // 8 wavefronts: 2 (rows) x 4 (columns), 128x64 outputs each
-
 struct Frags {
   bf16x8 a[4], b[2];
 };
 
-__device__ __forceinline__ void load_frags(const unsigned char *stage, int a_base, int b_base,
-                                           int swz, Frags &f) {
+template <int TK>
+__device__ __forceinline__ void load_frags(const unsigned char *sa, const unsigned char *sb, int a_base,
+                                           int b_base, int swz, Frags &f) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) f.a[i] = *(const bf16x8 *)(stage + kAOff + a_base + i * 4096 + swz);
+  for (int i = 0; i < 4; ++i) f.a[i] = *(const bf16x8 *)(sa + a_base + i * (32 * TK * 2) + swz);
 #pragma unroll
-  for (int i = 0; i < 2; ++i) f.b[i] = *(const bf16x8 *)(stage + kBOff + b_base + i * 4096 + swz);
+  for (int i = 0; i < 2; ++i) f.b[i] = *(const bf16x8 *)(sb + b_base + i * (32 * TK * 2) + swz);
 }
 
 __device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
@@ -108,10 +109,21 @@ __device__ __forceinline__ void stage_cols(unsigned char *region, const uint16_t
   __builtin_amdgcn_wave_barrier();
 }
 
-template <int EPI>
-__global__ void __launch_bounds__(kBigThreads, 1) k_ns_gemm_big(NsGemm p) {
-  __shared__ __attribute__((aligned(1024))) unsigned char stage0[kStageBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char stage1[kStageBytes];
+constexpr int kStageRegion = 6144;      // bytes of epilogue staging per wavefront (>= 64*40*2)
+
+template <int EPI, int TM, int TN, int TK, int MINBLOCKS>
+__global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemm p) {
+  constexpr int NWN = TN / 64, NWAVES = (TM / 128) * NWN;
+  constexpr int ROWB = TK * 2;                      // bytes per LDS row
+  constexpr int CPR = TK / 8;                       // 16-byte chunks per row
+  constexpr int RPI = 64 / CPR;                     // rows per DMA instruction
+  constexpr int IA = TM / RPI / NWAVES, IB = TN / RPI / NWAVES;   // DMA instructions per wavefront
+  constexpr int KSTEPS = TK / 16;
+  constexpr int kStage = (TM + TN) * ROWB;
+  static_assert(kStage >= NWAVES * kStageRegion, "epilogue staging must fit in one stage");
+  static_assert(TM % (RPI * NWAVES) == 0 && TN % (RPI * NWAVES) == 0, "DMA split");
+  __shared__ __attribute__((aligned(1024))) unsigned char stage0[kStage];
+  __shared__ __attribute__((aligned(1024))) unsigned char stage1[kStage];
 
   const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
   const int tiles_per = p.lower ? p.tiles_m * (p.tiles_m + 1) / 2 : p.tiles_m * p.tiles_n;
@@ -128,38 +140,47 @@ __global__ void __launch_bounds__(kBigThreads, 1) k_ns_gemm_big(NsGemm p) {
   }
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave / NWN, wn = wave % NWN;
   const int K = p.K, nk = K / TK, total = p.nterms * nk;
 
-  // ---- DMA addressing: this wavefront moves rows [wave*32, wave*32+32) of both operand tiles,
-  //      8 rows per instruction; lane -> (row lane/8, physical chunk lane%8). The address is a
-  //      wavefront-uniform base plus one of two per-lane byte offsets (even / odd instruction):
-  //      logical chunk = pchunk ^ (((i*8 + lrow) >> 1) & 7) = pchunk ^ (lrow>>1) ^ 4*(i&1).
-  const int lrow = lane >> 3, pchunk = lane & 7;
-  const uint32_t voff0 = (uint32_t)(lrow * K * 2 + ((pchunk ^ (lrow >> 1)) * 16));
-  const uint32_t voff1 = (uint32_t)(lrow * K * 2 + ((pchunk ^ (lrow >> 1) ^ 4) * 16));
-  const int64_t ubaseA = ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * 32) * K) * 2;   // bytes
-  const int64_t ubaseB = ((int64_t)e * p.strideB + (int64_t)(tn * TN + wave * 32) * K) * 2;
+  // ---- DMA addressing: this wavefront moves IA*RPI rows of the A tile and IB*RPI rows of the B
+  //      tile, RPI rows per instruction; lane -> (row lane/CPR, physical chunk lane%CPR). The
+  //      global address is a wavefront-uniform base plus a per-lane byte offset that carries
+  //      the swizzle: 128-byte rows use chunk ^ ((row>>1)&7), which alternates with the parity
+  //      of the instruction index (RPI = 8); 64-byte rows use chunk ^ ((row>>2)&3), the same
+  //      for every instruction (RPI = 16).
+  const int lrow = lane / CPR, pchunk = lane % CPR;
+  const int key0 = (TK == 64) ? (lrow >> 1) : ((lrow >> 2) & 3);
+  const uint32_t voff0 = (uint32_t)(lrow * K * 2 + ((pchunk ^ key0) * 16));
+  const uint32_t voff1 = (uint32_t)(lrow * K * 2 + ((pchunk ^ key0 ^ (TK == 64 ? 4 : 0)) * 16));
+  const int64_t ubaseA = ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * (IA * RPI)) * K) * 2;   // bytes
+  const int64_t ubaseB = ((int64_t)e * p.strideB + (int64_t)(tn * TN + wave * (IB * RPI)) * K) * 2;
 
   auto issue = [&](int step, unsigned char *stage) {
     const int term = step / nk, kt = step - term * nk;
-    const char *Ag = (const char *)p.A[term] + ubaseA + (int64_t)kt * (TK * 2);
-    const char *Bg = (const char *)p.B[term] + ubaseB + (int64_t)kt * (TK * 2);
+    const char *Ag = (const char *)p.A[term] + ubaseA + (int64_t)kt * ROWB;
+    const char *Bg = (const char *)p.B[term] + ubaseB + (int64_t)kt * ROWB;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int64_t ro = (int64_t)(i * 8) * K * 2;
+    for (int i = 0; i < IA; ++i) {
+      const int64_t ro = (int64_t)(i * RPI) * K * 2;
       const uint32_t vo = (i & 1) ? voff1 : voff0;
-      __builtin_amdgcn_global_load_lds(GLB1(Ag + ro + vo), LDS3(stage + kAOff + (wave * 32 + i * 8) * 128), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(GLB1(Bg + ro + vo), LDS3(stage + kBOff + (wave * 32 + i * 8) * 128), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(GLB1(Ag + ro + vo), LDS3(stage + (wave * IA + i) * 1024), 16, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < IB; ++i) {
+      const int64_t ro = (int64_t)(i * RPI) * K * 2;
+      const uint32_t vo = (i & 1) ? voff1 : voff0;
+      __builtin_amdgcn_global_load_lds(GLB1(Bg + ro + vo), LDS3(stage + TM * ROWB + (wave * IB + i) * 1024), 16, 0, 0);
     }
   };
 
   // ---- fragment addressing
-  const int a_base = (wm * 128 + (lane & 31)) * 128;
-  const int b_base = (wn * 64 + (lane & 31)) * 128;
-  int swz[4];
+  const int a_base = (wm * 128 + (lane & 31)) * ROWB;
+  const int b_base = TM * ROWB + (wn * 64 + (lane & 31)) * ROWB;
+  int swz[KSTEPS];
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) swz[kk] = ((kk * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
+  for (int kk = 0; kk < KSTEPS; ++kk)
+    swz[kk] = ((kk * 2 + (lane >> 5)) ^ (TK == 64 ? ((lane >> 1) & 7) : ((lane >> 2) & 3))) * 16;
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -169,27 +190,28 @@ __global__ void __launch_bounds__(kBigThreads, 1) k_ns_gemm_big(NsGemm p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[bi][bj][r] = 0.0f;
 
-  Frags f0, f1;
+  Frags f[2];
   issue(0, stage0);
   wait_vm0();
   __syncthreads();
-  load_frags(stage0, a_base, b_base, swz[0], f0);
+  load_frags<TK>(stage0, stage0, a_base, b_base, swz[0], f[0]);
 
+  // one K tile: fragments of k-step kk+1 are requested before the MFMAs of k-step kk; f[kk&1]
+  // holds k-step kk (KSTEPS is even, so every tile starts and ends on f[0] / f[1]).
   auto body = [&](int step, unsigned char *cur, unsigned char *nxt) {
     const bool more = step + 1 < total;
 #ifndef ANC_DBG_NODMA
     if (more) issue(step + 1, nxt);
 #endif
-    load_frags(cur, a_base, b_base, swz[1], f1);
-    mfma8(f0, acc);
-    load_frags(cur, a_base, b_base, swz[2], f0);
-    mfma8(f1, acc);
-    load_frags(cur, a_base, b_base, swz[3], f1);
-    mfma8(f0, acc);
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS - 1; ++kk) {
+      load_frags<TK>(cur, cur, a_base, b_base, swz[kk + 1], f[(kk + 1) & 1]);
+      mfma8(f[kk & 1], acc);
+    }
     wait_vm0();
     __syncthreads();
-    if (more) load_frags(nxt, a_base, b_base, swz[0], f0);
-    mfma8(f1, acc);
+    if (more) load_frags<TK>(nxt, nxt, a_base, b_base, swz[0], f[0]);
+    mfma8(f[(KSTEPS - 1) & 1], acc);
   };
   for (int step = 0; step < total; step += 2) {
     body(step, stage0, stage1);
@@ -200,7 +222,7 @@ __global__ void __launch_bounds__(kBigThreads, 1) k_ns_gemm_big(NsGemm p) {
   // ---- epilogue
   const int M = p.M, N = p.N;
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
-  unsigned char *region = stage0 + wave * 8192;           // 8 KiB of staging per wavefront
+  unsigned char *region = stage0 + wave * kStageRegion;
   const int gi0w = tm * TM + wm * 128, gj0w = tn * TN + wn * 64;
   const bool mirror = (EPI != EPI_BX) && (tm != tn);
 #pragma unroll
@@ -289,22 +311,34 @@ __global__ void __launch_bounds__(kBigThreads, 1) k_ns_gemm_big(NsGemm p) {
         stage_cols(region, lv, lane, p.YlT + mn + (int64_t)gj0w * M + gi0, M);
       }
     }
-  }
+    }
+}
+
+template <int EPI>
+int launch_sym(const NsGemm &p, int64_t E, hipStream_t s) {
+  const int64_t grid = E * ((int64_t)p.tiles_m * (p.tiles_m + 1) / 2);
+  ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
+  hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 64, 1>), dim3((unsigned)grid), dim3(512), 0, s, p);
+  ANC_LAUNCH_CHECK();
+  return ANC_OK;
 }
 
 }  // namespace
 
+// Symmetric products run on 256x256 tiles (p.tiles_m = p.tiles_n = M/256, lower triangle);
+// X = a X + B X runs on 128x256 tiles (the tile counts of p are recomputed here).
 int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
-  ANC_REQUIRE(p.M % TM == 0 && p.N % TN == 0 && p.K % TK == 0,
+  ANC_REQUIRE(p.M % 256 == 0 && p.N % 256 == 0 && p.K % 64 == 0,
               "anc_ns_gemm_big: dims must be multiples of 256");
-  const int64_t tiles_per = p.lower ? (int64_t)p.tiles_m * (p.tiles_m + 1) / 2
-                                    : (int64_t)p.tiles_m * p.tiles_n;
-  const int64_t grid = E * tiles_per;
+  if (epi == EPI_GRAM) return launch_sym<EPI_GRAM>(p, E, s);
+  if (epi == EPI_BMAT) return launch_sym<EPI_BMAT>(p, E, s);
+  NsGemm q = p;
+  q.tiles_m = p.M / 128;
+  q.tiles_n = p.N / 256;
+  q.lower = 0;
+  const int64_t grid = E * (int64_t)q.tiles_m * q.tiles_n;
   ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
-  const dim3 g((unsigned)grid), b(kBigThreads);
-  if (epi == EPI_GRAM)      hipLaunchKernelGGL(k_ns_gemm_big<EPI_GRAM>, g, b, 0, s, p);
-  else if (epi == EPI_BMAT) hipLaunchKernelGGL(k_ns_gemm_big<EPI_BMAT>, g, b, 0, s, p);
-  else                      hipLaunchKernelGGL(k_ns_gemm_big<EPI_BX>, g, b, 0, s, p);
+  hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 2>), dim3((unsigned)grid), dim3(256), 0, s, q);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
