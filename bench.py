@@ -110,6 +110,91 @@ def cpu_baseline(shapes, lr_adam=3e-4):
                       f"{len(os.sched_getaffinity(0))} usable, BLAS threads {threads}"}
 
 
+def side_workload(args):
+    """Configs 3 and 5 as stand-alone timings (same JSON shape, their own metric names)."""
+    from ancora_cutile_amd import DevBuf, StepGuard, AdamW, PE_SCHEDULE, _lib
+    from ancora_cutile_amd.muon_ns import ns_batched, ns_flops
+    _lib.init(0)
+    info = _lib.device_info()
+    e0, e1 = _lib.Event(), _lib.Event()
+    if args.workload == "ns":
+        groups = ((1024, 1024, 56), (1024, 2048, 56), (1024, 3072, 84))
+        res = {}
+        for mode in ("bf16", "fp32"):
+            steps = args.steps if mode == "bf16" else 1
+            total_ms, ex_t, de_t = 0.0, 0.0, 0.0
+            for (M, N, E) in groups:
+                one = np.random.default_rng(M + N).standard_normal((M, N)).astype(np.float32)
+                X = DevBuf.empty((E * M, N), np.float32)
+                for e in range(E):
+                    X.at_pos(e * M).upload(one)
+                ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
+                e0.record(0)
+                for _ in range(steps):
+                    ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
+                e1.record(0)
+                e1.sync()
+                total_ms += e0.elapsed_ms(e1) / steps
+                ex, de = ns_flops(E, M, N, 5, mode)
+                ex_t += ex
+                de_t += de
+                X.free()
+            res[mode] = {"ms": round(total_ms, 3), "executed_tflop": round(ex_t / 1e12, 3),
+                         "dense_tflop": round(de_t / 1e12, 3),
+                         "executed_tflops_per_s": round(ex_t / total_ms / 1e9, 1)}
+        out = {"metric": "196-matrix Newton-Schulz chain ms (5 x Polar-Express)", "value": res["bf16"]["ms"],
+               "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": 1, "ms_per_step": res["bf16"]["ms"],
+               "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+               "data": "synthetic", "config": {"workload": "ns-196-matrices", "groups": [list(g) for g in groups]},
+               "modes": res}
+    else:
+        n = 1_200_000_000
+        rng = np.random.default_rng(0)
+        from ancora_cutile_amd.bf16 import bf16_bits
+        chunk = bf16_bits(1e-3 * rng.standard_normal(1 << 24, dtype=np.float32))
+        g = DevBuf.empty((n,), np.uint16)
+        for off in range(0, n, 1 << 24):
+            k = min(1 << 24, n - off)
+            DevBuf(shape=(k,), dtype=np.uint16, ptr=g.ptr + 2 * off).upload(chunk[:k])
+        m, v, p = (DevBuf.zeros((n,), np.float32) for _ in range(3))
+        p16 = DevBuf.zeros((n,), np.uint16)
+        guard = StepGuard(1.0)
+        import ctypes
+        from ancora_cutile_amd.adamw import hyper_div
+
+        def step(t):
+            guard.compute([g], 0)
+            h = hyper_div(3e-4, 0.9, 0.95, 1e-8, 1000 + t, sr=True, seed_base=t)
+            _lib.api.anc_adamw(g.ptr, m.ptr, v.ptr, p.ptr, p16.ptr, n, _lib.BF16, ctypes.byref(h), 0.1, 0,
+                               guard.ptr, 0)
+        for t in range(args.warmup):
+            step(t)
+        e0.record(0)
+        for t in range(args.steps):
+            step(t)
+        e1.record(0)
+        e1.sync()
+        ms = e0.elapsed_ms(e1) / args.steps
+        _lib.profile_enable(True)
+        step(0)
+        pr = _lib.profile_read()
+        _lib.profile_enable(False)
+        a_ms, g_ms = pr["adamw"][0], pr["gradnorm_partials"][0]
+        out = {"metric": "flat 1.2e9-element grad-norm + clip + AdamW + SR downcast ms", "value": round(ms, 3),
+               "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
+               "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+               "data": "synthetic", "config": {"workload": "adamw-flat-1.2e9", "step": 1000},
+               "roofline": {"bound": "hbm", "achieved": round(30.0 * n / (ms * 1e-3) / 1e9, 1),
+                            "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                            "frac": round(30.0 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "traffic": None,
+                            "bytes_per_elem": 30},
+               "adamw_kernel": {"ms": round(a_ms, 3), "gbps": round(28.0 * n / (a_ms * 1e-3) / 1e9, 1)},
+               "gradnorm_kernel": {"ms": round(g_ms, 3), "gbps": round(2.0 * n / (g_ms * 1e-3) / 1e9, 1)},
+               "clip_scale": guard.read(0)["clip_scale"]}
+    out["device"] = {"name": info["name"], "arch": info["arch"], "cus": info["cu_count"]}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -117,6 +202,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=28, help=argparse.SUPPRESS)   # smaller sets for debugging
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--workload", default="qwen3", choices=("qwen3", "moe", "ns", "adamw"),
+                    help="qwen3: the headline hybrid step (default). moe: the 16-layer MoE family "
+                         "(config 4). ns: the 196-matrix Newton-Schulz stress, bf16 and fp32 modes "
+                         "(config 3). adamw: one flat 1.2e9-element buffer (config 5)")
     ap.add_argument("--serial", action="store_true",
                     help="run the per-shape Newton-Schulz chains on one stream also in the timed steps "
                          "(what the rocprofv3 kernel summaries under profiles/ were taken with)")
@@ -125,15 +214,20 @@ def main():
         sys.exit("bench.py: this optimizer step runs on one GPU; --gpus must be 1 "
                  "(no multi-GPU path is built, see DESIGN.md)")
 
+    if args.workload in ("ns", "adamw"):
+        return side_workload(args)
     from ancora_cutile_amd import HybridOptimizer, DevBuf, PE_SCHEDULE, _lib
     from ancora_cutile_amd.hybrid import resident_is_muon
     from ancora_cutile_amd.muon_ns import ns_flops
-    from ancora_cutile_amd.shapes import qwen3_shapes
+    from ancora_cutile_amd.shapes import qwen3_shapes, moe_shapes
 
     _lib.init(0)
     info = _lib.device_info()
     log(f"device: {info['name']} {info['arch']} cus={info['cu_count']} clock={info['clock_khz']} kHz")
-    shapes = qwen3_shapes(layers=args.layers)
+    if args.workload == "moe":
+        shapes = moe_shapes(layers=16)
+    else:
+        shapes = qwen3_shapes(layers=args.layers)
     t0 = time.perf_counter()
     params, grads = synth(shapes)
     n_params = sum(p.size for p in params.values())
@@ -219,20 +313,22 @@ def main():
     # same workload (two counter runs scaled by the copy kernel; summary under profiles/)
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "ns_gemm_traffic.json")
-    if args.layers == 28 and os.path.exists(tpath):
+    if args.workload == "qwen3" and args.layers == 28 and os.path.exists(tpath):
         with open(tpath) as f:
             traffic = json.load(f).get("hbm_bytes_per_launch")
 
     out = {
-        "metric": METRIC, "value": round(ms_per_step, 3), "unit": "ms", "n_gpus": 1,
+        "metric": METRIC if args.workload == "qwen3" else "MoE-16L Muon+AdamW step ms",
+        "value": round(ms_per_step, 3), "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "qwen3-0.6b-hybrid-step", "params": n_params, "muon_params": n_muon,
+        "config": {"workload": "qwen3-0.6b-hybrid-step" if args.workload == "qwen3" else "moe-16l-hybrid-step",
+                   "params": n_params, "muon_params": n_muon,
                    "adamw_params": n_adam, "muon_matrices": sum(b.E for b in opt.muon.engine.batches),
                    "grads": "bf16 resident in HBM, 1% rows x100", "clip": 1.0,
                    "weight_downcast": "stochastic bf16", "ns": "5 x polar-express",
-                   "layers": args.layers},
+                   "layers": 16 if args.workload == "moe" else args.layers},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
                      "kernel": "k_ns_gemm_big (gram, bmat, bx launches of the Newton-Schulz chain)",
