@@ -18,7 +18,7 @@ OUT = os.path.join(CSRC, "libancora_optim.so")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
          "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-unused-command-line-argument"]
+         "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
 
 
 def build(verbose=True):

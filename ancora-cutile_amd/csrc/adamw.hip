@@ -18,9 +18,24 @@
 
 namespace {
 
+#ifndef ADAMW_UNROLL
+#define ADAMW_UNROLL 4
+#endif
+#ifndef ADAMW_LD_NT
+#define ADAMW_LD_NT 1
+#endif
+#ifndef ADAMW_ST_NT
+#define ADAMW_ST_NT 1
+#endif
 constexpr int kThreads = 256;
 constexpr int kVec = 4;
-constexpr int kUnroll = 4;
+constexpr int kUnroll = ADAMW_UNROLL;
+template <typename T> __device__ __forceinline__ T ld_(const T *p) {
+  return ADAMW_LD_NT ? __builtin_nontemporal_load(p) : *p;
+}
+template <typename T> __device__ __forceinline__ void st_(T *p, T v) {
+  if (ADAMW_ST_NT) __builtin_nontemporal_store(v, p); else *p = v;
+}
 constexpr int kSlab = kThreads * kVec;          // 1024 elements
 constexpr int kBlockElems = kSlab * kUnroll;    // 4096 elements
 
@@ -63,17 +78,17 @@ __device__ __forceinline__ void adamw_block(const Tensor &t, int64_t blk,
     live[j] = e < t.n;
     if (live[j]) {
       if (GD == ANC_BF16) {
-        const anc_u32x2 gb = anc_ld_stream((const anc_u32x2 *)((const uint16_t *)t.g + e));
+        const anc_u32x2 gb = ld_((const anc_u32x2 *)((const uint16_t *)t.g + e));
         g4[j].x = __uint_as_float(gb.x << 16);
         g4[j].y = __uint_as_float(gb.x & 0xFFFF0000u);
         g4[j].z = __uint_as_float(gb.y << 16);
         g4[j].w = __uint_as_float(gb.y & 0xFFFF0000u);
       } else {
-        g4[j] = anc_ld_stream((const anc_f32x4 *)((const float *)t.g + e));
+        g4[j] = ld_((const anc_f32x4 *)((const float *)t.g + e));
       }
-      m4[j] = anc_ld_stream((const anc_f32x4 *)(t.m + e));
-      v4[j] = anc_ld_stream((const anc_f32x4 *)(t.v + e));
-      p4[j] = anc_ld_stream((const anc_f32x4 *)(t.p32 + e));
+      m4[j] = ld_((const anc_f32x4 *)(t.m + e));
+      v4[j] = ld_((const anc_f32x4 *)(t.v + e));
+      p4[j] = ld_((const anc_f32x4 *)(t.p32 + e));
     }
   }
 #pragma unroll
@@ -99,10 +114,10 @@ __device__ __forceinline__ void adamw_block(const Tensor &t, int64_t blk,
     anc_f32x4 vo = {vv[0], vv[1], vv[2], vv[3]};
     anc_f32x4 po = {pp[0], pp[1], pp[2], pp[3]};
     anc_u32x2 ho = {(hb[0] & 0xFFFFu) | (hb[1] << 16), (hb[2] & 0xFFFFu) | (hb[3] << 16)};
-    anc_st_stream((anc_f32x4 *)(t.m + e), mo);
-    anc_st_stream((anc_f32x4 *)(t.v + e), vo);
-    anc_st_stream((anc_f32x4 *)(t.p32 + e), po);
-    anc_st_stream((anc_u32x2 *)(t.p16 + e), ho);
+    st_((anc_f32x4 *)(t.m + e), mo);
+    st_((anc_f32x4 *)(t.v + e), vo);
+    st_((anc_f32x4 *)(t.p32 + e), po);
+    st_((anc_u32x2 *)(t.p16 + e), ho);
   }
 }
 

@@ -111,7 +111,37 @@ __device__ __forceinline__ void stage_cols(unsigned char *region, const uint16_t
 
 constexpr int kStageRegion = 6144;      // bytes of epilogue staging per wavefront (>= 64*40*2)
 
-template <int EPI, int TM, int TN, int TK, int MINBLOCKS>
+// vmcnt(n): wait until at most n vector-memory operations of this wavefront are outstanding
+// (they complete in issue order), leaving lgkmcnt/expcnt alone.
+template <int N> __device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// One LDS-DMA instruction: lane l of the wavefront copies 16 bytes from g (per lane) to LDS byte
+// address lds_base + 16*l (lds_base wavefront-uniform, carried in M0). Written as inline
+// assembly so that the stage ring's explicit vmcnt waits are the only ones: the compiler's own
+// wait insertion is conservative about LDS-DMA writes that it cannot prove distinct from later
+// LDS reads and would drain the ring on every tile.
+__device__ __forceinline__ void dma16(const void *g, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g)
+               : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_addr(const void *p) {
+  return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void *)p);
+}
+
+// Workgroup barrier that orders LDS traffic only: this wavefront's LDS reads and writes have
+// completed (lgkmcnt 0) before it arrives. Unlike __syncthreads() it carries no fence over
+// global memory, so LDS-DMA loads of younger stages stay in flight across it; the caller waits
+// (wait_vm<N>) for the DMA it needs before calling this.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS>
 __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemm p) {
   constexpr int NWN = TN / 64, NWAVES = (TM / 128) * NWN;
   constexpr int ROWB = TK * 2;                      // bytes per LDS row
@@ -120,10 +150,19 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   constexpr int IA = TM / RPI / NWAVES, IB = TN / RPI / NWAVES;   // DMA instructions per wavefront
   constexpr int KSTEPS = TK / 16;
   constexpr int kStage = (TM + TN) * ROWB;
-  static_assert(kStage >= NWAVES * kStageRegion, "epilogue staging must fit in one stage");
+  constexpr int IPS = IA + IB;                      // DMA instructions per wavefront per stage
+  constexpr int WPS = kStage / kStageRegion;        // wavefronts whose epilogue staging fits in a stage
+  static_assert(NS >= 2 && NS <= 4 && (NS - 2) * IPS < 64, "stage ring");
+  static_assert(WPS * NS >= NWAVES, "epilogue staging must fit in the stages");
   static_assert(TM % (RPI * NWAVES) == 0 && TN % (RPI * NWAVES) == 0, "DMA split");
+  // NS stages, each its own __shared__ array (distinct objects for the compiler's alias analysis)
   __shared__ __attribute__((aligned(1024))) unsigned char stage0[kStage];
   __shared__ __attribute__((aligned(1024))) unsigned char stage1[kStage];
+  __shared__ __attribute__((aligned(1024))) unsigned char stage2[NS > 2 ? kStage : 16];
+  __shared__ __attribute__((aligned(1024))) unsigned char stage3[NS > 3 ? kStage : 16];
+  auto st = [&](int i) -> unsigned char * {
+    return i == 0 ? stage0 : i == 1 ? stage1 : i == 2 ? stage2 : stage3;
+  };
 
   const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
   const int tiles_per = p.lower ? p.tiles_m * (p.tiles_m + 1) / 2 : p.tiles_m * p.tiles_n;
@@ -164,13 +203,13 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     for (int i = 0; i < IA; ++i) {
       const int64_t ro = (int64_t)(i * RPI) * K * 2;
       const uint32_t vo = (i & 1) ? voff1 : voff0;
-      __builtin_amdgcn_global_load_lds(GLB1(Ag + ro + vo), LDS3(stage + (wave * IA + i) * 1024), 16, 0, 0);
+      dma16(Ag + ro + vo, lds_addr(stage + (wave * IA + i) * 1024));
     }
 #pragma unroll
     for (int i = 0; i < IB; ++i) {
       const int64_t ro = (int64_t)(i * RPI) * K * 2;
       const uint32_t vo = (i & 1) ? voff1 : voff0;
-      __builtin_amdgcn_global_load_lds(GLB1(Bg + ro + vo), LDS3(stage + TM * ROWB + (wave * IB + i) * 1024), 16, 0, 0);
+      dma16(Bg + ro + vo, lds_addr(stage + TM * ROWB + (wave * IB + i) * 1024));
     }
   };
 
@@ -190,39 +229,47 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[bi][bj][r] = 0.0f;
 
+  // Stage ring. Tile k lives in stage k % NS. The DMA of tile k+NS-1 is started at the top of
+  // tile k, into the stage that tile k-1 was read from (every wavefront left it before the
+  // barrier inside tile k-1). Before the last k-step of tile k each wavefront waits until its
+  // own DMA of tile k+1 has landed (NS-2 younger tiles may still be in flight), all
+  // wavefronts synchronise, and the first fragments of tile k+1 load under the last MFMAs.
   Frags f[2];
-  issue(0, stage0);
-  wait_vm0();
-  __syncthreads();
+#pragma unroll
+  for (int s0 = 0; s0 < NS - 1; ++s0)
+    if (s0 < total) issue(s0, st(s0));
+  if (total >= NS - 1) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
+  lds_barrier();
   load_frags<TK>(stage0, stage0, a_base, b_base, swz[0], f[0]);
 
-  // one K tile: fragments of k-step kk+1 are requested before the MFMAs of k-step kk; f[kk&1]
-  // holds k-step kk (KSTEPS is even, so every tile starts and ends on f[0] / f[1]).
-  auto body = [&](int step, unsigned char *cur, unsigned char *nxt) {
+  // f[kk&1] holds k-step kk (KSTEPS is even, so every tile starts on f[0] and ends on f[1]).
+  auto body = [&](int step, unsigned char *cur, unsigned char *nxt, unsigned char *fill) {
     const bool more = step + 1 < total;
+    const bool refill = step + NS - 1 < total;
 #ifndef ANC_DBG_NODMA
-    if (more) issue(step + 1, nxt);
+    if (refill) issue(step + NS - 1, fill);
 #endif
 #pragma unroll
     for (int kk = 0; kk < KSTEPS - 1; ++kk) {
       load_frags<TK>(cur, cur, a_base, b_base, swz[kk + 1], f[(kk + 1) & 1]);
       mfma8(f[kk & 1], acc);
     }
-    wait_vm0();
-    __syncthreads();
+    if (refill) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
+    lds_barrier();
     if (more) load_frags<TK>(nxt, nxt, a_base, b_base, swz[0], f[0]);
     mfma8(f[(KSTEPS - 1) & 1], acc);
   };
-  for (int step = 0; step < total; step += 2) {
-    body(step, stage0, stage1);
-    if (step + 1 < total) body(step + 1, stage1, stage0);
+  for (int step = 0; step < total; step += NS) {
+#pragma unroll
+    for (int s0 = 0; s0 < NS; ++s0)
+      if (step + s0 < total) body(step + s0, st(s0), st((s0 + 1) % NS), st((s0 + NS - 1) % NS));
   }
   __syncthreads();
 
   // ---- epilogue
   const int M = p.M, N = p.N;
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
-  unsigned char *region = stage0 + wave * kStageRegion;
+  unsigned char *region = st(wave / WPS) + (wave % WPS) * kStageRegion;
   const int gi0w = tm * TM + wm * 128, gj0w = tn * TN + wn * 64;
   const bool mirror = (EPI != EPI_BX) && (tm != tn);
 #pragma unroll
@@ -318,7 +365,7 @@ template <int EPI>
 int launch_sym(const NsGemm &p, int64_t E, hipStream_t s) {
   const int64_t grid = E * ((int64_t)p.tiles_m * (p.tiles_m + 1) / 2);
   ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
-  hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 64, 1>), dim3((unsigned)grid), dim3(512), 0, s, p);
+  hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 32, 4, 1>), dim3((unsigned)grid), dim3(512), 0, s, p);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
@@ -328,7 +375,7 @@ int launch_sym(const NsGemm &p, int64_t E, hipStream_t s) {
 // Symmetric products run on 256x256 tiles (p.tiles_m = p.tiles_n = M/256, lower triangle);
 // X = a X + B X runs on 128x256 tiles (the tile counts of p are recomputed here).
 int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
-  ANC_REQUIRE(p.M % 256 == 0 && p.N % 256 == 0 && p.K % 64 == 0,
+  ANC_REQUIRE(p.M % 256 == 0 && p.N % 256 == 0 && p.K % 32 == 0,
               "anc_ns_gemm_big: dims must be multiples of 256");
   if (epi == EPI_GRAM) return launch_sym<EPI_GRAM>(p, E, s);
   if (epi == EPI_BMAT) return launch_sym<EPI_BMAT>(p, E, s);
@@ -338,7 +385,7 @@ int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
   q.lower = 0;
   const int64_t grid = E * (int64_t)q.tiles_m * q.tiles_n;
   ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
-  hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 2>), dim3((unsigned)grid), dim3(256), 0, s, q);
+  hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, q);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
