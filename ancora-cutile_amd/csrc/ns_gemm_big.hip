@@ -33,6 +33,9 @@
 // Accumulation order per output element is the same in every tile configuration and in the
 // 128x128 kernel of ns.hip (terms in order, k ascending, one accumulator).
 #include "ns_common.h"
+#ifndef ANC_DBG_EPI
+#define ANC_DBG_EPI 0
+#endif
 
 namespace {
 
@@ -84,7 +87,7 @@ __device__ __forceinline__ void stage_rows(unsigned char *region, const uint16_t
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, row = idx >> 3, c8 = (idx & 7) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + row * 72 + c8);
-    *(anc_u32x4 *)(out + (int64_t)row * ld + c8) = q;
+    anc_st_stream((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
@@ -103,7 +106,7 @@ __device__ __forceinline__ void stage_cols(unsigned char *region, const uint16_t
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, col = idx >> 2, r8 = (idx & 3) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + col * 40 + r8);
-    *(anc_u32x4 *)(outT + (int64_t)col * ldT + r8) = q;
+    anc_st_stream((anc_u32x4 *)(outT + (int64_t)col * ldT + r8), q);
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
@@ -267,6 +270,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   __syncthreads();
 
   // ---- epilogue
+#ifdef ANC_DBG_NOEPI
+  if (acc[0][0][0] + acc[3][1][7] != 12345.678f) return;
+#endif
   const int M = p.M, N = p.N;
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
   unsigned char *region = st(wave / WPS) + (wave % WPS) * kStageRegion;
@@ -287,7 +293,11 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         for (int r = 0; r < 16; ++r) {
           const int gi = gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
           const int gj = gj0w + bj * 32 + (lane & 31);
-          in[bj][r] = src[(int64_t)gi * ld + gj];
+#if (ANC_DBG_EPI & 1)
+          in[bj][r] = 1.0f;
+#else
+          in[bj][r] = anc_ld_stream(src + (int64_t)gi * ld + gj);
+#endif
         }
       const float *dvec = (EPI == EPI_BMAT) ? p.dA + mv : p.dB + mv;
 #pragma unroll
@@ -329,7 +339,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           lv[bj][r] = bl;
         } else {
           const float y = (p.ca + drow[r]) * in[bj][r] + v;
-          p.X32[mn + (int64_t)gi * N + gj] = y;
+#if !(ANC_DBG_EPI & 2)
+          anc_st_stream(p.X32 + mn + (int64_t)gi * N + gj, y);
+#endif
           const uint32_t yh = anc_bf16_rne_bits(y);
           hv[bj][r] = (uint16_t)yh;
           lv[bj][r] = (uint16_t)anc_bf16_rne_bits(y - anc_bf16_bits_to_f32(yh));
@@ -351,8 +363,12 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         if (mirror) stage_cols(region, lv, lane, p.Bl + mm + (int64_t)gj0w * M + gi0, M);
       }
     } else if (p.Yh != nullptr) {
+#if !(ANC_DBG_EPI & 4)
       stage_rows(region, hv, lane, p.Yh + mn + (int64_t)gi0 * N + gj0w, N);
+#endif
+#if !(ANC_DBG_EPI & 8)
       stage_cols(region, hv, lane, p.YhT + mn + (int64_t)gj0w * M + gi0, M);
+#endif
       if (p.Yl != nullptr) {
         stage_rows(region, lv, lane, p.Yl + mn + (int64_t)gi0 * N + gj0w, N);
         stage_cols(region, lv, lane, p.YlT + mn + (int64_t)gj0w * M + gi0, M);
@@ -365,6 +381,14 @@ template <int EPI>
 int launch_sym(const NsGemm &p, int64_t E, hipStream_t s) {
   const int64_t grid = E * ((int64_t)p.tiles_m * (p.tiles_m + 1) / 2);
   ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
+#ifdef ANC_EXPERIMENT
+  { const char *sv = getenv("ANC_CFG_SYM");
+    if (sv && atoi(sv) == 1) {
+      hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 64, 2, 1>), dim3((unsigned)grid), dim3(512), 0, s, p);
+      ANC_LAUNCH_CHECK();
+      return ANC_OK;
+    } }
+#endif
   hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 32, 4, 1>), dim3((unsigned)grid), dim3(512), 0, s, p);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
@@ -383,6 +407,18 @@ int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
   q.tiles_m = p.M / 128;
   q.tiles_n = p.N / 256;
   q.lower = 0;
+#ifdef ANC_EXPERIMENT
+  { const char *sv = getenv("ANC_CFG_BX");
+    const int c = sv ? atoi(sv) : 0;
+    if (c) {
+      q.tiles_m = p.M / 256;
+      const int64_t g2 = E * (int64_t)q.tiles_m * q.tiles_n;
+      if (c == 1) hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 256, 256, 32, 4, 1>), dim3((unsigned)g2), dim3(512), 0, s, q);
+      else hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 256, 256, 64, 2, 1>), dim3((unsigned)g2), dim3(512), 0, s, q);
+      ANC_LAUNCH_CHECK();
+      return ANC_OK;
+    } }
+#endif
   const int64_t grid = E * (int64_t)q.tiles_m * q.tiles_n;
   ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
   hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, q);
