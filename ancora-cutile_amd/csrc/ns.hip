@@ -46,7 +46,12 @@ using namespace anc_reduce;
 template <int EPI>
 __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
   __shared__ __attribute__((aligned(16))) uint16_t sA[BM * PITCH];
-  __shared__ __attribute__((aligned(16))) uint16_t sB[BN * PITCH];
+  // B tile: [n][k] rows of PITCH for the symmetric products; [k][n] rows of NPITCH (320 bytes:
+  // consecutive rows start 64 bytes apart in the banks) for X = a X + B X, which reads the
+  // iterate (K, N) row-major as it lies in memory and transposes while reading fragments.
+  constexpr int NPITCH = BN + 32;
+  constexpr bool BT = (EPI == EPI_BX);
+  __shared__ __attribute__((aligned(16))) uint16_t sB[BT ? BK * NPITCH : BN * PITCH];
 
   const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
   const int tiles_per = p.lower ? p.tiles_m * (p.tiles_m + 1) / 2 : p.tiles_m * p.tiles_n;
@@ -81,18 +86,21 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
   auto gload = [&](int step) {
     const int term = step / nk, kt = step - term * nk;
     const uint16_t *Ap = p.A[term] + (int64_t)e * p.strideA + (int64_t)(tm * BM + lrow) * K + kt * BK + lk;
-    const uint16_t *Bp = p.B[term] + (int64_t)e * p.strideB + (int64_t)(tn * BN + lrow) * K + kt * BK + lk;
+    // (k, n) tile: 16 lanes per 256-byte row, 16 rows per pass
+    const uint16_t *Bp = BT ? p.B[term] + (int64_t)e * p.strideB + (int64_t)(kt * BK + (tid >> 4)) * p.N + tn * BN + (tid & 15) * 8
+                            : p.B[term] + (int64_t)e * p.strideB + (int64_t)(tn * BN + lrow) * K + kt * BK + lk;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       ra[i] = *(const anc_u32x4 *)(Ap + (int64_t)(32 * i) * K);
-      rb[i] = *(const anc_u32x4 *)(Bp + (int64_t)(32 * i) * K);
+      rb[i] = BT ? *(const anc_u32x4 *)(Bp + (int64_t)(16 * i) * p.N) : *(const anc_u32x4 *)(Bp + (int64_t)(32 * i) * K);
     }
   };
   auto lstore = [&]() {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       *(anc_u32x4 *)&sA[(lrow + 32 * i) * PITCH + lk] = ra[i];
-      *(anc_u32x4 *)&sB[(lrow + 32 * i) * PITCH + lk] = rb[i];
+      if (BT) *(anc_u32x4 *)&sB[((tid >> 4) + 16 * i) * NPITCH + (tid & 15) * 8] = rb[i];
+      else *(anc_u32x4 *)&sB[(lrow + 32 * i) * PITCH + lk] = rb[i];
     }
   };
 
@@ -101,6 +109,8 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
   __syncthreads();
   const int arow = (wm * 64 + (lane & 31)) * PITCH + (lane >> 5) * 8;
   const int brow = (wn * 64 + (lane & 31)) * PITCH + (lane >> 5) * 8;
+  // transposing reads: lane s of each 16-lane group addresses row s/4, columns 4*(s%4)..+3
+  const int btr = (8 * (lane >> 5) + ((lane & 15) >> 2)) * NPITCH + wn * 64 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   for (int step = 0; step < total; ++step) {
     const bool more = step + 1 < total;
     if (more) gload(step + 1);
@@ -110,7 +120,9 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
 #pragma unroll
       for (int bi = 0; bi < 2; ++bi) a[bi] = *(const bf16x8 *)&sA[arow + bi * 32 * PITCH + kk * 16];
 #pragma unroll
-      for (int bj = 0; bj < 2; ++bj) b[bj] = *(const bf16x8 *)&sB[brow + bj * 32 * PITCH + kk * 16];
+      for (int bj = 0; bj < 2; ++bj)
+        b[bj] = BT ? anc_lds_tr_frag(&sB[btr + kk * 16 * NPITCH + bj * 32], &sB[btr + (kk * 16 + 4) * NPITCH + bj * 32])
+                   : *(const bf16x8 *)&sB[brow + bj * 32 * PITCH + kk * 16];
 #pragma unroll
       for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
@@ -175,19 +187,13 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
           }
         } else {
           const int64_t o = mn + (int64_t)gi * N + gj;
-          const float x = p.X32[o];
+          const float x = anc_bf16_bits_to_f32(p.Xh[o]) + anc_bf16_bits_to_f32(p.Xl[o]);
           const float y = (p.ca + p.dB[mv + gi]) * x + v;
-          p.X32[o] = y;
+          if (p.X32 != nullptr) p.X32[o] = y;
           if (p.Yh != nullptr) {
             const uint32_t yh = anc_bf16_rne_bits(y);
-            const int64_t ot = mn + (int64_t)gj * M + gi;
             p.Yh[o] = (uint16_t)yh;
-            p.YhT[ot] = (uint16_t)yh;
-            if (p.Yl != nullptr) {
-              const uint16_t yl = (uint16_t)anc_bf16_rne_bits(y - anc_bf16_bits_to_f32(yh));
-              p.Yl[o] = yl;
-              p.YlT[ot] = yl;
-            }
+            p.Yl[o] = (uint16_t)anc_bf16_rne_bits(y - anc_bf16_bits_to_f32(yh));
           }
         }
       }
@@ -317,59 +323,35 @@ k_fro_finalize(const double *__restrict__ partials, int nchunks, float eps, floa
   }
 }
 
-// X *= recip[e] in place; optional bf16 copies: Xh (M,N), XhT (N,M) and the residuals Xl, XlT.
+// Normalisation X * recip[e]. With Xh == null the fp32 matrix is scaled in place (fp32 chain,
+// steps == 0); otherwise X is left alone and the scaled iterate leaves as the bf16 pair
+// Xh = bf16(x), Xl = bf16(x - Xh), both (M,N) row-major. 8 elements per lane.
 __global__ void __launch_bounds__(kThreads)
-k_ns_prep(float *__restrict__ X, const float *__restrict__ recip, int M, int N,
-          uint16_t *__restrict__ Xh, uint16_t *__restrict__ XhT,
-          uint16_t *__restrict__ Xl, uint16_t *__restrict__ XlT) {
-  __shared__ uint16_t th[64][66], tl[64][66];
-  const int tiles_n = N / 64, tiles_m = M / 64;
-  const int64_t per = (int64_t)tiles_m * tiles_n;
-  const int64_t e = (int64_t)blockIdx.x / per, tile = (int64_t)blockIdx.x % per;
-  const int tr = (int)(tile / tiles_n), tc = (int)(tile % tiles_n);
-  const float rc = recip[e];
-  const int64_t mn = e * (int64_t)M * N;
-  const int c4 = (threadIdx.x & 15) * 4, r0 = threadIdx.x >> 4;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = r0 + 16 * i;
-    const int64_t o = mn + (int64_t)(tr * 64 + r) * N + tc * 64 + c4;
-    anc_f32x4 x = *(const anc_f32x4 *)(X + o);
-    float xs[4] = {x.x * rc, x.y * rc, x.z * rc, x.w * rc};
-    anc_f32x4 xo = {xs[0], xs[1], xs[2], xs[3]};
-    *(anc_f32x4 *)(X + o) = xo;
-    if (Xh != nullptr) {
-      uint32_t h[4], l[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        h[k] = anc_bf16_rne_bits(xs[k]);
-        l[k] = anc_bf16_rne_bits(xs[k] - anc_bf16_bits_to_f32(h[k]));
-        th[r][c4 + k] = (uint16_t)h[k];
-        tl[r][c4 + k] = (uint16_t)l[k];
-      }
-      anc_u32x2 ho = {(h[0] & 0xFFFFu) | (h[1] << 16), (h[2] & 0xFFFFu) | (h[3] << 16)};
-      *(anc_u32x2 *)(Xh + o) = ho;
-      if (Xl != nullptr) {
-        anc_u32x2 lo = {(l[0] & 0xFFFFu) | (l[1] << 16), (l[2] & 0xFFFFu) | (l[3] << 16)};
-        *(anc_u32x2 *)(Xl + o) = lo;
-      }
-    }
+k_ns_prep(float *__restrict__ X, const float *__restrict__ recip, int64_t mn, int64_t total8,
+          uint16_t *__restrict__ Xh, uint16_t *__restrict__ Xl) {
+  const int64_t i8 = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i8 >= total8) return;
+  const int64_t o = i8 * 8;
+  const float rc = recip[o / mn];
+  const anc_f32x4 x0 = anc_ld_stream((const anc_f32x4 *)(X + o));
+  const anc_f32x4 x1 = anc_ld_stream((const anc_f32x4 *)(X + o + 4));
+  const float xs[8] = {x0.x * rc, x0.y * rc, x0.z * rc, x0.w * rc, x1.x * rc, x1.y * rc, x1.z * rc, x1.w * rc};
+  if (Xh == nullptr) {
+    const anc_f32x4 y0 = {xs[0], xs[1], xs[2], xs[3]}, y1 = {xs[4], xs[5], xs[6], xs[7]};
+    *(anc_f32x4 *)(X + o) = y0;
+    *(anc_f32x4 *)(X + o + 4) = y1;
+    return;
   }
-  if (Xh == nullptr) return;
-  __syncthreads();
+  uint32_t h[8], l[8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = r0 + 16 * i;
-    const int64_t ot = mn + (int64_t)(tc * 64 + r) * M + tr * 64 + c4;
-    const uint32_t a0 = th[c4][r], a1 = th[c4 + 1][r], a2 = th[c4 + 2][r], a3 = th[c4 + 3][r];
-    anc_u32x2 ho = {a0 | (a1 << 16), a2 | (a3 << 16)};
-    *(anc_u32x2 *)(XhT + ot) = ho;
-    if (XlT != nullptr) {
-      const uint32_t b0 = tl[c4][r], b1 = tl[c4 + 1][r], b2 = tl[c4 + 2][r], b3 = tl[c4 + 3][r];
-      anc_u32x2 lo = {b0 | (b1 << 16), b2 | (b3 << 16)};
-      *(anc_u32x2 *)(XlT + ot) = lo;
-    }
+  for (int k = 0; k < 8; ++k) {
+    h[k] = anc_bf16_rne_bits(xs[k]) & 0xFFFFu;
+    l[k] = anc_bf16_rne_bits(xs[k] - anc_bf16_bits_to_f32(h[k])) & 0xFFFFu;
   }
+  const anc_u32x4 ho = {h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+  const anc_u32x4 lo = {l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16)};
+  anc_st_stream((anc_u32x4 *)(Xh + o), ho);
+  anc_st_stream((anc_u32x4 *)(Xl + o), lo);
 }
 
 // ------------------------------------------------------------------------- workspace
@@ -418,7 +400,7 @@ struct Plan {
   double *partials;
   float *recip;
   // bf16 modes
-  uint16_t *Xh[2], *XhT[2], *Xl[2], *XlT[2];
+  uint16_t *Xh[2], *Xl[2];
   float *A32, *dA, *dB;
   uint16_t *Fh, *Bh;
   // fp32 mode
@@ -441,13 +423,8 @@ Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int ste
   } else {
     for (int i = 0; i < 2; ++i) {
       pl.Xh[i] = c.take<uint16_t>(E * M * N);
-      pl.XhT[i] = c.take<uint16_t>(E * M * N);
+      pl.Xl[i] = c.take<uint16_t>(E * M * N);
     }
-    if (pl.split)
-      for (int i = 0; i < 2; ++i) {
-        pl.Xl[i] = c.take<uint16_t>(E * M * N);
-        pl.XlT[i] = c.take<uint16_t>(E * M * N);
-      }
     pl.A32 = c.take<float>(E * M * M);
     pl.Fh = c.take<uint16_t>(E * M * M);
     pl.Bh = c.take<uint16_t>(E * M * M);
@@ -532,12 +509,13 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
   { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s, pl.partials, pl.nchunks,
                      eps, pl.recip); }
   ANC_LAUNCH_CHECK();
-  const unsigned prep_grid = (unsigned)(E * (M / 64) * (N / 64));
+  const int64_t total8 = E * mn / 8;
+  const unsigned prep_grid = (unsigned)((total8 + kThreads - 1) / kThreads);
   const int split_from = pl.sp.x_from;   // first iteration with X residual terms
 
   if (mode == ANC_NS_FP32) {
-    { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
-                       (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr); }
+    { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, mn, total8,
+                       (uint16_t *)nullptr, (uint16_t *)nullptr); }
     ANC_LAUNCH_CHECK();
     float *cur = X32, *nxt = pl.Yf;
     const unsigned g_mm = (unsigned)(E * (M / BM) * (M / BN)), g_mn = (unsigned)(E * (M / BM) * (N / BN));
@@ -567,15 +545,13 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
 
   // ---- bf16 matrix-core chain
   if (steps == 0) {
-    { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
-                       (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr, (uint16_t *)nullptr); }
+    { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, mn, total8,
+                       (uint16_t *)nullptr, (uint16_t *)nullptr); }
     ANC_LAUNCH_CHECK();
     return ANC_OK;
   }
-  const bool split0 = split_from <= 0;
-  { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, (int)M, (int)N,
-                     pl.Xh[0], pl.XhT[0], split0 ? pl.Xl[0] : (uint16_t *)nullptr,
-                     split0 ? pl.XlT[0] : (uint16_t *)nullptr); }
+  { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, mn, total8,
+                     pl.Xh[0], pl.Xl[0]); }
   ANC_LAUNCH_CHECK();
   const bool big = !force_small && (M % 256 == 0) && (N % 256 == 0);   // 256x256 tiles, same bits
   const int tile = big ? 256 : BM;
@@ -586,10 +562,9 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
     const bool split = k >= split_from;
     const bool split_fb = k >= pl.sp.fb_from;
     const bool last = k + 1 == steps;
-    const bool split_next = !last && (k + 1 >= split_from);
     NsGemm g{};
     g.M = (int)M; g.N = (int)N;
-    g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB; g.X32 = X32;
+    g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB;
     g.Fl = split_fb ? pl.Fl : nullptr;
     g.Bl = split_fb ? pl.Bl : nullptr;
     g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
@@ -625,14 +600,14 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
     ANC_LAUNCH_CHECK();
     // X = a X + B X
     NsGemm gx = g;
-    gx.A[0] = pl.Bh; gx.B[0] = pl.XhT[cur]; gx.nterms = 1;
-    if (split) { gx.A[gx.nterms] = pl.Bh; gx.B[gx.nterms] = pl.XlT[cur]; ++gx.nterms; }
-    if (split_fb) { gx.A[gx.nterms] = pl.Bl; gx.B[gx.nterms] = pl.XhT[cur]; ++gx.nterms; }
+    gx.A[0] = pl.Bh; gx.B[0] = pl.Xh[cur]; gx.nterms = 1;
+    if (split) { gx.A[gx.nterms] = pl.Bh; gx.B[gx.nterms] = pl.Xl[cur]; ++gx.nterms; }
+    if (split_fb) { gx.A[gx.nterms] = pl.Bl; gx.B[gx.nterms] = pl.Xh[cur]; ++gx.nterms; }
     gx.K = (int)M; gx.strideA = M * M; gx.strideB = mn; gx.tiles_m = tM; gx.tiles_n = tN; gx.lower = 0;
+    gx.Xh = pl.Xh[cur]; gx.Xl = pl.Xl[cur];
     gx.Yh = last ? nullptr : pl.Xh[cur ^ 1];
-    gx.YhT = last ? nullptr : pl.XhT[cur ^ 1];
-    gx.Yl = split_next ? pl.Xl[cur ^ 1] : nullptr;
-    gx.YlT = split_next ? pl.XlT[cur ^ 1] : nullptr;
+    gx.Yl = last ? nullptr : pl.Xl[cur ^ 1];
+    gx.X32 = last ? X32 : nullptr;
     {
       AncProfScope prof(ANC_PROF_NS_BX, s);
       if (big) { if (int rc = anc_ns_gemm_big(EPI_BX, gx, E, s)) return rc; }

@@ -5,6 +5,21 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+// B-operand fragment of v_mfma_f32_32x32x16_bf16 from a (k, n) row-major LDS tile: two
+// ds_read_b64_tr_b16. Within each group of 16 lanes, lane i receives the i%4-th 16-bit element
+// of the 8 bytes addressed by lanes i/4, i/4+4, i/4+8, i/4+12 of the group. With lane s of a
+// group pointing at row k0 + s/4, columns n0 + 4*(s%4) .. +3, lane i therefore receives
+// column n0 + i of rows k0 .. k0+3. `p0` addresses rows k0.., `p1` rows k0+4..; the result
+// holds 8 consecutive k of one column, the layout the matrix instruction wants.
+__device__ __forceinline__ bf16x8 anc_lds_tr_frag(const void *p0, const void *p1) {
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p0);
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p1);
+  const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, v);
+}
 
 constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int PITCH = BK + 8;            // bf16 elements per LDS row: 144 bytes
@@ -23,7 +38,8 @@ __device__ __forceinline__ int xcd_remap(int bid, int grid) {
 
 struct NsGemm {
   const uint16_t *A[3];      // term t: rows of the output  (tiles_m*128 rows, ld = K)
-  const uint16_t *B[3];      // term t: columns of the output (tiles_n*128 rows, ld = K)
+  const uint16_t *B[3];      // term t: columns of the output. GRAM, BMAT: one row per column, ld = K
+                             // ("NT" product); BX: the iterate itself, (K, N) row-major, ld = N
   int nterms;
   int K;
   int64_t strideA, strideB;  // elements between consecutive matrices
@@ -37,9 +53,9 @@ struct NsGemm {
   float *dA;                 // (E,M)   diag A            GRAM out, BMAT in
   uint16_t *Bh;              // (E,M,M) bf16 off-diag B   BMAT out
   float *dB;                 // (E,M)   diag B            BMAT out, BX in
-  float *X32;                // (E,M,N) fp32 iterate      BX in/out
-  uint16_t *Yh, *YhT;        // next iterate bf16 (M,N) and (N,M); null on the last step
-  uint16_t *Yl, *YlT;        // bf16 residual copies; null unless the next step splits
+  const uint16_t *Xh, *Xl;   // (E,M,N) current iterate as a bf16 pair, X = Xh + Xl   BX in
+  uint16_t *Yh, *Yl;         // (E,M,N) next iterate as a bf16 pair   BX out, null on the last step
+  float *X32;                // (E,M,N) fp32 result                   BX out on the last step, else null
 };
 
 

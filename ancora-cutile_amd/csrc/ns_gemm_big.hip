@@ -58,6 +58,20 @@ __device__ __forceinline__ void load_frags(const unsigned char *sa, const unsign
   for (int i = 0; i < 2; ++i) f.b[i] = *(const bf16x8 *)(sb + b_base + i * (32 * TK * 2) + swz);
 }
 
+// Same fragments when the B tile is stored (k, n) row-major with 512-byte rows (the X = a X + B X
+// product reads the iterate as it lies in memory): the A fragments as above, the B fragments
+// through transposing LDS reads. tb[bj] is the lane's byte offset for k-step 0 of column
+// block bj (it carries the swizzle); a k-step advances 16 rows, the second read 4 rows.
+template <int TK>
+__device__ __forceinline__ void load_frags_bt(const unsigned char *st, int a_base, int swz, const int (&tb)[2],
+                                              int kk, Frags &f) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f.a[i] = *(const bf16x8 *)(st + a_base + i * (32 * TK * 2) + swz);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    f.b[i] = anc_lds_tr_frag(st + tb[i] + kk * (16 * 512), st + tb[i] + kk * (16 * 512) + 4 * 512);
+}
+
 __device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi)
@@ -197,11 +211,22 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const uint32_t voff1 = (uint32_t)(lrow * K * 2 + ((pchunk ^ key0 ^ (TK == 64 ? 4 : 0)) * 16));
   const int64_t ubaseA = ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * (IA * RPI)) * K) * 2;   // bytes
   const int64_t ubaseB = ((int64_t)e * p.strideB + (int64_t)(tn * TN + wave * (IB * RPI)) * K) * 2;
+  // (k, n) B tile: TK rows of TN*2 = 512 bytes, two rows per DMA instruction; lane -> (row
+  // lane/32, physical chunk lane%32); the chunk index is XORed with 4*(row&3), so that the 4
+  // rows a transposing read touches per 32 lanes fall into 4 different 64-byte bank windows.
+  // row&3 = 2*(instruction parity) + lane/32.
+  constexpr bool BT = (EPI == EPI_BX);
+  static_assert(!BT || (TN == 256 && IB % 2 == 0 && IB * NWAVES * 2 == TK), "(k,n) tile layout");
+  const int ldn = p.N;
+  const uint32_t voffB0 = (uint32_t)((lane >> 5) * ldn * 2 + (((lane & 31) ^ (((lane >> 5)) << 2)) * 16));
+  const uint32_t voffB1 = (uint32_t)((lane >> 5) * ldn * 2 + (((lane & 31) ^ ((2 + (lane >> 5)) << 2)) * 16));
+  const int64_t ubaseBT = ((int64_t)e * p.strideB + (int64_t)tn * TN + (int64_t)(wave * IB * 2) * ldn) * 2;
 
   auto issue = [&](int step, unsigned char *stage) {
     const int term = step / nk, kt = step - term * nk;
     const char *Ag = (const char *)p.A[term] + ubaseA + (int64_t)kt * ROWB;
-    const char *Bg = (const char *)p.B[term] + ubaseB + (int64_t)kt * ROWB;
+    const char *Bg = BT ? (const char *)p.B[term] + ubaseBT + (int64_t)kt * TK * ldn * 2
+                        : (const char *)p.B[term] + ubaseB + (int64_t)kt * ROWB;
 #pragma unroll
     for (int i = 0; i < IA; ++i) {
       const int64_t ro = (int64_t)(i * RPI) * K * 2;
@@ -210,8 +235,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     }
 #pragma unroll
     for (int i = 0; i < IB; ++i) {
-      const int64_t ro = (int64_t)(i * RPI) * K * 2;
-      const uint32_t vo = (i & 1) ? voff1 : voff0;
+      const int64_t ro = BT ? (int64_t)(i * 2) * ldn * 2 : (int64_t)(i * RPI) * K * 2;
+      const uint32_t vo = BT ? ((i & 1) ? voffB1 : voffB0) : ((i & 1) ? voff1 : voff0);
       dma16(Bg + ro + vo, lds_addr(stage + TM * ROWB + (wave * IB + i) * 1024));
     }
   };
@@ -223,6 +248,20 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #pragma unroll
   for (int kk = 0; kk < KSTEPS; ++kk)
     swz[kk] = ((kk * 2 + (lane >> 5)) ^ (TK == 64 ? ((lane >> 1) & 7) : ((lane >> 2) & 3))) * 16;
+
+  int tb[2] = {0, 0};
+  if (BT) {
+    const int s16 = lane & 15, g16 = lane >> 4;
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj) {
+      const int chunk = wn * 8 + bj * 4 + 2 * (g16 & 1) + ((s16 & 3) >> 1);
+      tb[bj] = TM * ROWB + (8 * (g16 >> 1) + (s16 >> 2)) * 512 + ((chunk ^ ((s16 >> 2) << 2)) * 16) + (s16 & 1) * 8;
+    }
+  }
+  auto frags = [&](const unsigned char *stg, int kk, Frags &f) {
+    if (BT) load_frags_bt<TK>(stg, a_base, swz[kk], tb, kk, f);
+    else load_frags<TK>(stg, stg, a_base, b_base, swz[kk], f);
+  };
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -243,7 +282,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     if (s0 < total) issue(s0, st(s0));
   if (total >= NS - 1) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
   lds_barrier();
-  load_frags<TK>(stage0, stage0, a_base, b_base, swz[0], f[0]);
+  frags(stage0, 0, f[0]);
 
   // f[kk&1] holds k-step kk (KSTEPS is even, so every tile starts on f[0] and ends on f[1]).
   auto body = [&](int step, unsigned char *cur, unsigned char *nxt, unsigned char *fill) {
@@ -254,12 +293,12 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #endif
 #pragma unroll
     for (int kk = 0; kk < KSTEPS - 1; ++kk) {
-      load_frags<TK>(cur, cur, a_base, b_base, swz[kk + 1], f[(kk + 1) & 1]);
+      frags(cur, kk + 1, f[(kk + 1) & 1]);
       mfma8(f[kk & 1], acc);
     }
     if (refill) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
     lds_barrier();
-    if (more) load_frags<TK>(nxt, nxt, a_base, b_base, swz[0], f[0]);
+    if (more) frags(nxt, 0, f[0]);
     mfma8(f[(KSTEPS - 1) & 1], acc);
   };
   for (int step = 0; step < total; step += NS) {
@@ -278,15 +317,46 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   unsigned char *region = st(wave / WPS) + (wave % WPS) * kStageRegion;
   const int gi0w = tm * TM + wm * 128, gj0w = tn * TN + wn * 64;
   const bool mirror = (EPI != EPI_BX) && (tm != tn);
+
+  // X = a X + B X reads the iterate at the output position (the bf16 pair Xh, Xl). A 32x64 slab
+  // of each is 32 rows of 128 bytes: 4 DMA instructions (8 rows each, lane -> row lane/8, chunk
+  // lane%8) put it into a buffer private to the wavefront, two slabs ahead of the arithmetic, so
+  // that full cache lines are requested and the latency runs under the previous slabs. The
+  // 16-byte chunk index is XORed with 4*((row>>2)&1): the two half-wavefronts, which read rows
+  // 4 apart, then use different banks. The same buffer stages the slab's bf16 outputs.
+  constexpr int kInBuf = 8192, kBufPerStage = kStage / kInBuf;
+  static_assert(EPI != EPI_BX || (kBufPerStage * NS >= 2 * NWAVES && kInBuf >= kStageRegion), "epilogue buffers");
+  auto inbuf = [&](int bi) -> unsigned char * {
+    const int q = wave * 2 + (bi & 1);
+    return st(q / kBufPerStage) + (q % kBufPerStage) * kInBuf;
+  };
+  const uint32_t vo_in = (uint32_t)((lane >> 3) * N * 2 + (((lane & 7) ^ ((lane >> 5) << 2)) * 16));
+  auto fetch_in = [&](int bi) {
+    const int64_t ub = (mn + (int64_t)(gi0w + bi * 32) * N + gj0w) * 2;
+    unsigned char *b = inbuf(bi);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t ro = (int64_t)(8 * j) * N * 2;
+      dma16((const char *)p.Xh + ub + ro + vo_in, lds_addr(b + j * 1024));
+      dma16((const char *)p.Xl + ub + ro + vo_in, lds_addr(b + 4096 + j * 1024));
+    }
+  };
+  int in_lane[2] = {0, 0};
+  if (EPI == EPI_BX) {
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+      in_lane[bj] = 4 * (lane >> 5) * 128 + (((bj * 4 + ((lane & 31) >> 3)) ^ ((lane >> 5) << 2)) * 16) + (lane & 7) * 2;
+    fetch_in(0);
+    fetch_in(1);
+  }
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi) {
     uint16_t hv[2][16], lv[2][16];
     const int gi0 = gi0w + bi * 32;
     // operands of the epilogue first (all loads in flight together), arithmetic after
     float in[2][16], drow[16], dcol[2];
-    if (EPI != EPI_GRAM) {
-      const float *src = (EPI == EPI_BMAT) ? p.A32 + mm : p.X32 + mn;
-      const int64_t ld = (EPI == EPI_BMAT) ? M : N;
+    if (EPI == EPI_BMAT) {
+      const float *src = p.A32 + mm;
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
@@ -296,9 +366,26 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #if (ANC_DBG_EPI & 1)
           in[bj][r] = 1.0f;
 #else
-          in[bj][r] = anc_ld_stream(src + (int64_t)gi * ld + gj);
+          in[bj][r] = anc_ld_stream(src + (int64_t)gi * M + gj);
 #endif
         }
+    }
+    if (EPI == EPI_BX) {
+      // X = Xh + Xl is exact in fp32 (8 + 8 significant bits)
+      wait_vm<0>();
+      const unsigned char *b = inbuf(bi);
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int ro = (8 * (r >> 2) + (r & 3)) * 128;
+          const uint16_t xh = *(const uint16_t *)(b + in_lane[bj] + ro);
+          const uint16_t xl = *(const uint16_t *)(b + 4096 + in_lane[bj] + ro);
+          in[bj][r] = anc_bf16_bits_to_f32(xh) + anc_bf16_bits_to_f32(xl);
+        }
+      region = const_cast<unsigned char *>(b);
+    }
+    if (EPI != EPI_GRAM) {
       const float *dvec = (EPI == EPI_BMAT) ? p.dA + mv : p.dB + mv;
 #pragma unroll
       for (int r = 0; r < 16; ++r) drow[r] = dvec[gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
@@ -339,9 +426,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           lv[bj][r] = bl;
         } else {
           const float y = (p.ca + drow[r]) * in[bj][r] + v;
-#if !(ANC_DBG_EPI & 2)
-          anc_st_stream(p.X32 + mn + (int64_t)gi * N + gj, y);
-#endif
+          if (p.X32 != nullptr) anc_st_stream(p.X32 + mn + (int64_t)gi * N + gj, y);
           const uint32_t yh = anc_bf16_rne_bits(y);
           hv[bj][r] = (uint16_t)yh;
           lv[bj][r] = (uint16_t)anc_bf16_rne_bits(y - anc_bf16_bits_to_f32(yh));
@@ -362,33 +447,24 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         stage_rows(region, lv, lane, p.Bl + mm + (int64_t)gi0 * M + gj0w, M);
         if (mirror) stage_cols(region, lv, lane, p.Bl + mm + (int64_t)gj0w * M + gi0, M);
       }
-    } else if (p.Yh != nullptr) {
-#if !(ANC_DBG_EPI & 4)
-      stage_rows(region, hv, lane, p.Yh + mn + (int64_t)gi0 * N + gj0w, N);
-#endif
-#if !(ANC_DBG_EPI & 8)
-      stage_cols(region, hv, lane, p.YhT + mn + (int64_t)gj0w * M + gi0, M);
-#endif
-      if (p.Yl != nullptr) {
+    } else {
+      if (p.Yh != nullptr) {
+        stage_rows(region, hv, lane, p.Yh + mn + (int64_t)gi0 * N + gj0w, N);
         stage_rows(region, lv, lane, p.Yl + mn + (int64_t)gi0 * N + gj0w, N);
-        stage_cols(region, lv, lane, p.YlT + mn + (int64_t)gj0w * M + gi0, M);
       }
+      // this slab's buffer is free again (its inputs are in registers, its staged outputs
+      // were read back before stage_rows returned): fetch the slab after the next into it
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      asm volatile("" ::: "memory");
+      if (bi + 2 < 4) fetch_in(bi + 2);
     }
-    }
+  }
 }
 
 template <int EPI>
 int launch_sym(const NsGemm &p, int64_t E, hipStream_t s) {
   const int64_t grid = E * ((int64_t)p.tiles_m * (p.tiles_m + 1) / 2);
   ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
-#ifdef ANC_EXPERIMENT
-  { const char *sv = getenv("ANC_CFG_SYM");
-    if (sv && atoi(sv) == 1) {
-      hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 64, 2, 1>), dim3((unsigned)grid), dim3(512), 0, s, p);
-      ANC_LAUNCH_CHECK();
-      return ANC_OK;
-    } }
-#endif
   hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 32, 4, 1>), dim3((unsigned)grid), dim3(512), 0, s, p);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
@@ -407,18 +483,6 @@ int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
   q.tiles_m = p.M / 128;
   q.tiles_n = p.N / 256;
   q.lower = 0;
-#ifdef ANC_EXPERIMENT
-  { const char *sv = getenv("ANC_CFG_BX");
-    const int c = sv ? atoi(sv) : 0;
-    if (c) {
-      q.tiles_m = p.M / 256;
-      const int64_t g2 = E * (int64_t)q.tiles_m * q.tiles_n;
-      if (c == 1) hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 256, 256, 32, 4, 1>), dim3((unsigned)g2), dim3(512), 0, s, q);
-      else hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 256, 256, 64, 2, 1>), dim3((unsigned)g2), dim3(512), 0, s, q);
-      ANC_LAUNCH_CHECK();
-      return ANC_OK;
-    } }
-#endif
   const int64_t grid = E * (int64_t)q.tiles_m * q.tiles_n;
   ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
   hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, q);
