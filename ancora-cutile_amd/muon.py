@@ -367,6 +367,10 @@ class Muon:
                                  p16=s["p16"].at_pos(e * K), G=s["g"].at_pos(e * K), K=K, N=N,
                                  name=n, e=e))
         self._recs = recs
+        self._recs_of = {}
+        for r in recs:
+            self._recs_of.setdefault(r["name"], []).append(r)
+        self._gptr = {}                       # name -> pointer of the resident gradient last bound
         self.engine = MuonEngine(recs, momentum, ns_steps, nesterov, chunk, None, mode, sr, seed) \
             if recs else None
         self.last_skipped = False
@@ -376,10 +380,16 @@ class Muon:
         for n, s in self.st.items():
             g = grads[n]
             if isinstance(g, DevBuf):
-                for r in self._recs:
-                    if r["name"] == n:
-                        r["G"] = g.view((s["E"] * s["K"], s["N"])).at_pos(r["e"] * s["K"])
+                if self._gptr.get(n) != (g.ptr, g.dtype.str):
+                    gv = g.view((s["E"] * s["K"], s["N"]))
+                    for r in self._recs_of[n]:
+                        r["G"] = gv.at_pos(r["e"] * s["K"])
+                    self._gptr[n] = (g.ptr, g.dtype.str)
             else:
+                if n in self._gptr:               # back to the optimizer's own gradient buffer
+                    for r in self._recs_of[n]:
+                        r["G"] = s["g"].at_pos(r["e"] * s["K"])
+                    del self._gptr[n]
                 g = np.asarray(g)
                 if g.dtype != s["g"].dtype:
                     if s["g"].dtype == np.float32:
