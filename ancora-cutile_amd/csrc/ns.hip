@@ -8,18 +8,20 @@
 //
 // Precision design (bf16 modes). The reference stores X, A and B as bf16 between the
 // GEMMs, which leaves it about 6e-3 (relative Frobenius) from the fp32 numpy result.
-// Here the iterate stays in fp32 in HBM and is rounded to bf16 only as a matrix-core
-// operand, and the diagonals of A and B -- the entries that approach 1 and b+c while the
-// off-diagonal part goes to zero -- never pass through bf16:
+// Here the iterate is carried between steps as a bf16 pair X = Xh + Xl (Xh = bf16(x),
+// Xl = bf16(x - Xh): 16 significant bits, 4 bytes per element like fp32 but directly usable
+// as matrix-core operands), and the diagonals of A and B -- the entries that approach 1 and
+// b+c while the off-diagonal part goes to zero -- never pass through bf16:
 //   A = dA + F    dA = diag(A) kept as an fp32 vector, F = off-diagonal part
 //   A A = dA^2 + dA F + F dA + F F       only F F is a matrix-core product (bf16 F)
 //   B = dB + Boff                        likewise
 //   B X = dB (.) X + Boff X              dB (.) X is an fp32 row scaling in the epilogue
-// Where the shape needs it (see split_plan below) late iterations additionally carry the
-// bf16 residual of an operand (X = Xh + Xl): A gets Xh Xl^T + Xl Xh^T and B X gets Boff Xl
-// as extra accumulation terms of the same tile. All products are "NT" (both operands
-// K-contiguous): X is kept both as (M,N) and transposed (N,M) bf16 copies, written by the
-// epilogue that produces it.
+// Xh alone is the matrix-core operand of the early iterations. Where the shape needs it (see
+// split_plan below) late iterations add the residual products: A gets Xh Xl^T + Xl Xh^T and
+// B X gets Boff Xl as extra accumulation terms of the same tile. The symmetric products are
+// "NT" (both operands K-contiguous rows of X or F); B X reads the iterate (K, N) row-major
+// as it lies in memory and transposes inside LDS reads, so X exists in one layout only. The
+// fp32 input is read once (normalisation) and the fp32 result written once (last step).
 //
 // Determinism: one workgroup owns one 128x128 output tile and its whole K loop, terms in
 // a fixed order, K tiles in ascending order; no split-K, no atomics. A matrix's result

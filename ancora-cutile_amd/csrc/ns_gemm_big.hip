@@ -5,30 +5,34 @@
 // Tile. A 128x128 tile moves 64 FLOP per byte staged, which at the matrix-core rate asks more
 // of the per-XCD L2 than it delivers. Every wavefront here owns 128x64 outputs: 8 accumulator
 // blocks of 32x32 (128 accumulator registers per lane), 6 operand fragments per 8 MFMAs.
-//   symmetric products (A, B): 256x256x64 tile, 8 wavefronts (2 x 4), two 64 KiB LDS stages,
+//   symmetric products (A, B): 256x256x32 tile, 8 wavefronts (2 x 4), four 32 KiB LDS stages,
 //     128 FLOP per byte staged, one workgroup per CU;
-//   X = a X + B X: 128x256x32 tile, 4 wavefronts (1 x 4), two 24 KiB stages. Its epilogue moves
-//     12 bytes of HBM traffic per element (fp32 X read and written, two bf16 copies written)
-//     and is the longer phase; the small LDS footprint lets several workgroups share a CU, so
-//     the epilogue of one runs under the MFMAs of another.
+//   X = a X + B X: 128x256x32 tile, 4 wavefronts (1 x 4), three 24 KiB stages, two workgroups
+//     per CU. Its epilogue moves 8 bytes of HBM traffic per element (the bf16 pair of the
+//     iterate read and written) and runs at the HBM rate.
 //
 // Data path. Operand tiles go from HBM/L2 straight into LDS with global_load_lds_dwordx4 (no
 // register staging): one instruction moves 1 KiB, a lane writes 16 bytes at lds_base + 16*lane.
-// LDS rows are TK*2 bytes with no padding; bank conflicts are avoided by an XOR swizzle of the
-// 16-byte chunk index with row bits (bits 1..3 for 128-byte rows, bits 2..3 for 64-byte rows),
-// applied when choosing which global chunk a lane fetches and undone when a fragment is read:
-// 16 consecutive rows then cover all 64 banks once. The two stages live in two distinct
-// __shared__ arrays so that the compiler can tell a DMA write to one from a fragment read of
-// the other.
+// "NT" operand tiles ([row][k], TK*2-byte rows, no padding) avoid bank conflicts by an XOR
+// swizzle of the 16-byte chunk index with row bits (bits 1..3 for 128-byte rows, bits 2..3 for
+// 64-byte rows), applied when choosing which global chunk a lane fetches and undone when a
+// fragment is read: 16 consecutive rows then cover all 64 banks once. The B operand of
+// X = a X + B X is the iterate itself, (k, n) row-major: its tile is [k][256 columns], fetched
+// as whole 512-byte rows, and its fragments come from transposing LDS reads
+// (ds_read_b64_tr_b16), so no transposed copy of the iterate exists anywhere.
 //
-// Schedule per K tile: start the DMA of the next tile, run the k-steps of 8 MFMAs with the
-// fragments of the following k-step already in flight, wait for the DMA and synchronise before
-// the last k-step so that the first fragments of the next tile load under its MFMAs.
+// Stage ring. Tile k of the K loop lives in stage k % NS, each stage a __shared__ array of its
+// own. The DMA of tile k+NS-1 starts at the top of tile k; before the last k-step of tile k a
+// wavefront waits (s_waitcnt vmcnt) only for its own DMA of tile k+1, then the workgroup
+// synchronises with a barrier that orders LDS traffic only. The DMA instructions and these
+// waits are inline assembly: left to itself the compiler drains every outstanding LDS-DMA
+// load before an LDS read it cannot prove disjoint, and at __syncthreads().
 //
-// Epilogue. fp32 operands (A32, X32) are read and written straight from the accumulator
-// layout (128-byte row segments), all loads of a 32-row slab issued before its arithmetic;
-// every bf16 output passes through LDS so that rows and mirrored/transposed rows leave as
-// 16-byte stores.
+// Epilogue. fp32 operands (A32) are read straight into the accumulator layout (128-byte row
+// segments), all loads of a 32-row slab issued before its arithmetic; the bf16 pair of the
+// iterate that X = a X + B X needs at the output position arrives by LDS-DMA two slabs ahead;
+// every bf16 output passes through LDS so that rows and mirrored rows leave as 16-byte
+// stores. Epilogue loads and stores are nontemporal.
 //
 // Accumulation order per output element is the same in every tile configuration and in the
 // 128x128 kernel of ns.hip (terms in order, k ascending, one accumulator).
@@ -182,14 +186,25 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   };
 
   const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
-  const int tiles_per = p.lower ? p.tiles_m * (p.tiles_m + 1) / 2 : p.tiles_m * p.tiles_n;
+  // Symmetric outputs: only tiles that reach the diagonal or lie below it. Row tm of TM-row
+  // tiles has tm/R + 1 of them (R = TN/TM); a tile entirely below the diagonal is mirrored.
+  constexpr int R = TN / TM;
+  static_assert(TN % TM == 0, "tile ratio");
+  int tiles_per;
+  if (p.lower) {
+    const int q = p.tiles_m / R, r = p.tiles_m % R;          // sum over tm of (tm/R + 1)
+    tiles_per = R * q * (q + 1) / 2 + r * (q + 1);
+  } else {
+    tiles_per = p.tiles_m * p.tiles_n;
+  }
   const int e = L / tiles_per;
   const int t = L % tiles_per;
   int tm, tn;
   if (p.lower) {
     tm = 0;
-    while ((tm + 1) * (tm + 2) / 2 <= t) ++tm;
-    tn = t - tm * (tm + 1) / 2;
+    int left = t;
+    while (left >= tm / R + 1) { left -= tm / R + 1; ++tm; }
+    tn = left;
   } else {
     tm = t / p.tiles_n;
     tn = t % p.tiles_n;
@@ -316,7 +331,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
   unsigned char *region = st(wave / WPS) + (wave % WPS) * kStageRegion;
   const int gi0w = tm * TM + wm * 128, gj0w = tn * TN + wn * 64;
-  const bool mirror = (EPI != EPI_BX) && (tm != tn);
+  const bool mirror = (EPI != EPI_BX) && (TN * (tn + 1) <= TM * tm);
 
   // X = a X + B X reads the iterate at the output position (the bf16 pair Xh, Xl). A 32x64 slab
   // of each is 32 rows of 128 bytes: 4 DMA instructions (8 rows each, lane -> row lane/8, chunk
@@ -463,9 +478,11 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 
 template <int EPI>
 int launch_sym(const NsGemm &p, int64_t E, hipStream_t s) {
-  const int64_t grid = E * ((int64_t)p.tiles_m * (p.tiles_m + 1) / 2);
+  NsGemm q = p;
+  q.tiles_m = q.tiles_n = p.M / 256;
+  const int64_t grid = E * ((int64_t)q.tiles_m * (q.tiles_m + 1) / 2);
   ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
-  hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 32, 4, 1>), dim3((unsigned)grid), dim3(512), 0, s, p);
+  hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 32, 4, 1>), dim3((unsigned)grid), dim3(512), 0, s, q);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
