@@ -17,11 +17,15 @@ constexpr int kThreads = 256;
 constexpr int kBlockElems = 4096;
 constexpr int kTile = 64;
 
+constexpr int kPair = 2;     // internal u type: bf16 pair (hi at u, lo at u_lo), see k_mom_multi_pair
+
 struct MomArgs {
   float *buf;
   const void *g;
   void *u;
   int K, N;
+  void *u_lo;        // kPair only
+  double *fro;       // kPair only: this block's sum of u*u
 };
 struct UpdArgs {
   float *p32;
@@ -52,7 +56,7 @@ __device__ __forceinline__ anc_f32x4 load4(const void *p, int64_t e) {
 }
 template <int UD>
 __device__ __forceinline__ void store4(void *p, int64_t e, const float x[4]) {
-  if (UD == ANC_BF16) {
+  if (UD == ANC_BF16 || UD == kPair) {
     const uint32_t b0 = anc_bf16_rne_bits(x[0]), b1 = anc_bf16_rne_bits(x[1]);
     const uint32_t b2 = anc_bf16_rne_bits(x[2]), b3 = anc_bf16_rne_bits(x[3]);
     anc_u32x2 o = {(b0 & 0xFFFFu) | (b1 << 16), (b2 & 0xFFFFu) | (b3 << 16)};
@@ -61,6 +65,25 @@ __device__ __forceinline__ void store4(void *p, int64_t e, const float x[4]) {
     anc_f32x4 o = {x[0], x[1], x[2], x[3]};
     anc_st_stream((anc_f32x4 *)((float *)p + e), o);
   }
+}
+
+// The bf16 pair of x: hi = bf16(x) to `hi`, lo = bf16(x - hi) to `lo`.
+__device__ __forceinline__ void store4_pair(void *hi, void *lo, int64_t e, const float x[4]) {
+  store4<kPair>(hi, e, x);
+  float r[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) r[k] = x[k] - anc_bf16_bits_to_f32(anc_bf16_rne_bits(x[k]));
+  store4<kPair>(lo, e, r);
+}
+
+// Sum over the block of each lane's `v`, fixed order: xor butterfly inside a wavefront, then
+// the 4 wavefront sums left to right. Lane 0 writes the result.
+__device__ __forceinline__ void block_sum_to(double v, double *out) {
+  __shared__ double wsum[4];
+  v = anc_wave_sum_f64(v);
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) *out = ((wsum[0] + wsum[1]) + wsum[2]) + wsum[3];
 }
 
 // buf = mom*buf + g';  u = nesterov ? g' + mom*buf : buf     (g' = g*clip)
@@ -77,6 +100,7 @@ __device__ __forceinline__ void mom_flat(const MomArgs &a, int64_t blk, float mo
                                          float clip) {
   const int64_t base = blk * kBlockElems + (int64_t)threadIdx.x * 4;
   anc_f32x4 g4[4], b4[4];
+  double ss = 0.0;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int64_t e = base + j * 1024;
@@ -93,8 +117,15 @@ __device__ __forceinline__ void mom_flat(const MomArgs &a, int64_t blk, float mo
     for (int k = 0; k < 4; ++k) uu[k] = mom_elem(gg[k], bb[k], mom, nesterov, clip);
     anc_f32x4 bo = {bb[0], bb[1], bb[2], bb[3]};
     anc_st_stream((anc_f32x4 *)(a.buf + e), bo);
-    store4<UD>(a.u, e, uu);
+    if (UD == kPair) {
+      store4_pair(a.u, a.u_lo, e, uu);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) ss += (double)uu[k] * (double)uu[k];
+    } else {
+      store4<UD>(a.u, e, uu);
+    }
   }
+  if (UD == kPair) block_sum_to(ss, a.fro);
 }
 
 // ---- momentum, transposed store: 64x64 tile through LDS ------------------------
@@ -120,6 +151,7 @@ __device__ __forceinline__ void mom_tile_t(const MomArgs &a, int64_t tile, float
   }
   __syncthreads();
   // u^T is (N,K): row tc*64 + r, columns tr*64 + c4 ..
+  double ss = 0.0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = r0 + 16 * i;
@@ -127,8 +159,15 @@ __device__ __forceinline__ void mom_tile_t(const MomArgs &a, int64_t tile, float
 #pragma unroll
     for (int k = 0; k < 4; ++k) uu[k] = lds[c4 + k][r];
     const int64_t e = (int64_t)(tc * kTile + r) * a.K + tr * kTile + c4;
-    store4<UD>(a.u, e, uu);
+    if (UD == kPair) {
+      store4_pair(a.u, a.u_lo, e, uu);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) ss += (double)uu[k] * (double)uu[k];
+    } else {
+      store4<UD>(a.u, e, uu);
+    }
   }
+  if (UD == kPair) block_sum_to(ss, a.fro);
 }
 
 // ---- update: p32 -= lr_scale*O; p16 = bf16(p32) ----------------------------------
@@ -240,6 +279,32 @@ k_mom_multi(const anc_muon_desc_t *__restrict__ table, int n_weights, float mom,
   } else {
     if (d.g_dtype == ANC_BF16) mom_flat<ANC_BF16, UD>(a, local, mom, nesterov, clip);
     else                       mom_flat<ANC_F32, UD>(a, local, mom, nesterov, clip);
+  }
+}
+
+// Momentum straight into the Newton-Schulz input format. d.u is the weight's slice of the
+// packed batch counted in fp32 elements from `base` (where the chain's fp32 result will land);
+// the bf16 pair of u goes to the same element offset in two bf16 arrays, hi at `base`, lo
+// `lo_off` bytes further (together the same 4 bytes per element). Block b also leaves the sum
+// of its 4096 u*u in fro[b], so that the Frobenius norm needs no further pass over the data:
+// a weight's blocks are consecutive, K*N/4096 of them.
+__global__ void __launch_bounds__(kThreads)
+k_mom_multi_pair(const anc_muon_desc_t *__restrict__ table, int n_weights, float mom, int nesterov,
+                 uint64_t base, int64_t lo_off, double *__restrict__ fro,
+                 const anc_step_ctl_t *__restrict__ ctl) {
+  float clip;
+  if (!load_ctl(ctl, clip)) return;
+  const anc_muon_desc_t d = find_weight(table, n_weights, (int64_t)blockIdx.x);
+  const int64_t local = (int64_t)blockIdx.x - d.tile0;
+  const uint64_t hi = base + (d.u - base) / 2;
+  MomArgs a{(float *)d.buf, (const void *)d.g, (void *)hi, d.K, d.N, (void *)(hi + (uint64_t)lo_off),
+            fro + blockIdx.x};
+  if (d.transpose) {
+    if (d.g_dtype == ANC_BF16) mom_tile_t<ANC_BF16, kPair>(a, local, mom, nesterov, clip);
+    else                       mom_tile_t<ANC_F32, kPair>(a, local, mom, nesterov, clip);
+  } else {
+    if (d.g_dtype == ANC_BF16) mom_flat<ANC_BF16, kPair>(a, local, mom, nesterov, clip);
+    else                       mom_flat<ANC_F32, kPair>(a, local, mom, nesterov, clip);
   }
 }
 
@@ -382,6 +447,23 @@ extern "C" int anc_muon_momentum_multi(uint64_t desc_table, int32_t n_weights, i
   else
     hipLaunchKernelGGL(k_mom_multi<ANC_F32>, grid, block, 0, anc_stream(stream), tab, (int)n_weights,
                        mom, nesterov, c);
+  ANC_LAUNCH_CHECK();
+  return ANC_OK;
+}
+
+extern "C" int anc_muon_momentum_multi_pair(uint64_t desc_table, int32_t n_weights, int64_t total_tiles,
+                                            float mom, int nesterov, uint64_t pair_base,
+                                            int64_t lo_offset_bytes, uint64_t fro_partials,
+                                            uint64_t ctl, uint64_t stream) {
+  ANC_REQUIRE(desc_table != 0 && n_weights > 0, "anc_muon_momentum_multi_pair: empty descriptor table");
+  ANC_REQUIRE(total_tiles > 0 && total_tiles < (1ll << 31), "anc_muon_momentum_multi_pair: bad total_tiles");
+  ANC_REQUIRE(pair_base != 0 && (pair_base & 15) == 0 && lo_offset_bytes > 0 && (lo_offset_bytes & 15) == 0,
+              "anc_muon_momentum_multi_pair: pair buffer must be 16-byte aligned");
+  ANC_REQUIRE(fro_partials != 0 && (fro_partials & 7) == 0, "anc_muon_momentum_multi_pair: null partials");
+  AncProfScope prof(ANC_PROF_MUON_MOM, anc_stream(stream));
+  hipLaunchKernelGGL(k_mom_multi_pair, dim3((unsigned)total_tiles), dim3(kThreads), 0, anc_stream(stream),
+                     (const anc_muon_desc_t *)desc_table, (int)n_weights, mom, nesterov, pair_base,
+                     lo_offset_bytes, (double *)fro_partials, (const anc_step_ctl_t *)ctl);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }

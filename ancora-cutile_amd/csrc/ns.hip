@@ -142,6 +142,9 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
   //      row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 block.
   const int M = p.M, N = p.N;
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
+  float sc = 1.0f;
+  if (EPI != EPI_BMAT && p.scale != nullptr) sc = p.scale[e];
+  const float acc_scale = (EPI == EPI_GRAM) ? sc * sc : sc;
 #pragma unroll
   for (int bi = 0; bi < 2; ++bi) {
 #pragma unroll
@@ -150,7 +153,7 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
       for (int r = 0; r < 16; ++r) {
         const int gi = tm * BM + wm * 64 + bi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         const int gj = tn * BN + wn * 64 + bj * 32 + (lane & 31);
-        const float v = acc[bi][bj][r];
+        const float v = (EPI == EPI_BMAT) ? acc[bi][bj][r] : acc[bi][bj][r] * acc_scale;
         if (EPI == EPI_GRAM) {
           const bool diag = gi == gj;
           const uint16_t fh = diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v);
@@ -189,7 +192,7 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
           }
         } else {
           const int64_t o = mn + (int64_t)gi * N + gj;
-          const float x = anc_bf16_bits_to_f32(p.Xh[o]) + anc_bf16_bits_to_f32(p.Xl[o]);
+          const float x = (anc_bf16_bits_to_f32(p.Xh[o]) + anc_bf16_bits_to_f32(p.Xl[o])) * sc;
           const float y = (p.ca + p.dB[mv + gi]) * x + v;
           if (p.X32 != nullptr) p.X32[o] = y;
           if (p.Yh != nullptr) {
@@ -454,6 +457,83 @@ int check_shape(int64_t E, int64_t M, int64_t N, int mode, const char *who) {
   return ANC_OK;
 }
 
+// steps x { A = X X^T; B = b A + c A A; X = a X + B X } on the bf16 pair (inH, inL). The first
+// step's output goes to pair `nxt` of the plan, later steps ping-pong; the last step writes the
+// fp32 result X32 (which may overlay the input pair when steps >= 2). `scale0`, if given, is the
+// per-matrix factor the first step applies to its unnormalised input.
+int run_bf16_chain(const Plan &pl, const uint16_t *inH, const uint16_t *inL, int nxt, const float *scale0,
+                   float *X32, int64_t E, int64_t M, int64_t N, int steps, const float *coef,
+                   bool force_small, hipStream_t s) {
+  const int64_t mn = M * N;
+  const int split_from = pl.sp.x_from;   // first iteration with X residual terms
+  const bool big = !force_small && (M % 256 == 0) && (N % 256 == 0);   // 256x256 tiles, same bits
+  const int tile = big ? 256 : BM;
+  const int tM = (int)(M / tile), tN = (int)(N / tile);
+  const unsigned g_sym = (unsigned)(E * tM * (tM + 1) / 2), g_mn = (unsigned)(E * tM * tN);
+  const uint16_t *curH = inH, *curL = inL;
+  for (int k = 0; k < steps; ++k) {
+    const bool split = k >= split_from;
+    const bool split_fb = k >= pl.sp.fb_from;
+    const bool last = k + 1 == steps;
+    NsGemm g{};
+    g.M = (int)M; g.N = (int)N;
+    g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB;
+    g.Fl = split_fb ? pl.Fl : nullptr;
+    g.Bl = split_fb ? pl.Bl : nullptr;
+    g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
+    g.scale = (k == 0) ? scale0 : nullptr;
+    // A = X X^T
+    NsGemm ga = g;
+    ga.A[0] = curH; ga.B[0] = curH; ga.nterms = 1;
+    if (split) {
+      ga.A[1] = curH; ga.B[1] = curL;
+      ga.A[2] = curL; ga.B[2] = curH;
+      ga.nterms = 3;
+    }
+    ga.K = (int)N; ga.strideA = mn; ga.strideB = mn; ga.tiles_m = tM; ga.tiles_n = tM; ga.lower = 1;
+    {
+      AncProfScope prof(ANC_PROF_NS_GRAM, s);
+      if (big) { if (int rc = anc_ns_gemm_big(EPI_GRAM, ga, E, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga);
+    }
+    ANC_LAUNCH_CHECK();
+    // B = b A + c A A
+    NsGemm gb = g;
+    gb.A[0] = pl.Fh; gb.B[0] = pl.Fh; gb.nterms = 1;
+    if (split_fb) {
+      gb.A[1] = pl.Fh; gb.B[1] = pl.Fl;
+      gb.A[2] = pl.Fl; gb.B[2] = pl.Fh;
+      gb.nterms = 3;
+    }
+    gb.K = (int)M; gb.strideA = M * M; gb.strideB = M * M; gb.tiles_m = tM; gb.tiles_n = tM; gb.lower = 1;
+    {
+      AncProfScope prof(ANC_PROF_NS_BMAT, s);
+      if (big) { if (int rc = anc_ns_gemm_big(EPI_BMAT, gb, E, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb);
+    }
+    ANC_LAUNCH_CHECK();
+    // X = a X + B X
+    NsGemm gx = g;
+    gx.A[0] = pl.Bh; gx.B[0] = curH; gx.nterms = 1;
+    if (split) { gx.A[gx.nterms] = pl.Bh; gx.B[gx.nterms] = curL; ++gx.nterms; }
+    if (split_fb) { gx.A[gx.nterms] = pl.Bl; gx.B[gx.nterms] = curH; ++gx.nterms; }
+    gx.K = (int)M; gx.strideA = M * M; gx.strideB = mn; gx.tiles_m = tM; gx.tiles_n = tN; gx.lower = 0;
+    gx.Xh = curH; gx.Xl = curL;
+    gx.Yh = last ? nullptr : pl.Xh[nxt];
+    gx.Yl = last ? nullptr : pl.Xl[nxt];
+    gx.X32 = last ? X32 : nullptr;
+    {
+      AncProfScope prof(ANC_PROF_NS_BX, s);
+      if (big) { if (int rc = anc_ns_gemm_big(EPI_BX, gx, E, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx);
+    }
+    ANC_LAUNCH_CHECK();
+    curH = pl.Xh[nxt]; curL = pl.Xl[nxt];
+    nxt ^= 1;
+  }
+  return ANC_OK;
+}
+
 }  // namespace
 
 extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode) {
@@ -513,7 +593,6 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
   ANC_LAUNCH_CHECK();
   const int64_t total8 = E * mn / 8;
   const unsigned prep_grid = (unsigned)((total8 + kThreads - 1) / kThreads);
-  const int split_from = pl.sp.x_from;   // first iteration with X residual terms
 
   if (mode == ANC_NS_FP32) {
     { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, mn, total8,
@@ -555,68 +634,34 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
   { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, mn, total8,
                      pl.Xh[0], pl.Xl[0]); }
   ANC_LAUNCH_CHECK();
-  const bool big = !force_small && (M % 256 == 0) && (N % 256 == 0);   // 256x256 tiles, same bits
-  const int tile = big ? 256 : BM;
-  const int tM = (int)(M / tile), tN = (int)(N / tile);
-  const unsigned g_sym = (unsigned)(E * tM * (tM + 1) / 2), g_mn = (unsigned)(E * tM * tN);
-  int cur = 0;
-  for (int k = 0; k < steps; ++k) {
-    const bool split = k >= split_from;
-    const bool split_fb = k >= pl.sp.fb_from;
-    const bool last = k + 1 == steps;
-    NsGemm g{};
-    g.M = (int)M; g.N = (int)N;
-    g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB;
-    g.Fl = split_fb ? pl.Fl : nullptr;
-    g.Bl = split_fb ? pl.Bl : nullptr;
-    g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
-    // A = X X^T
-    NsGemm ga = g;
-    ga.A[0] = pl.Xh[cur]; ga.B[0] = pl.Xh[cur]; ga.nterms = 1;
-    if (split) {
-      ga.A[1] = pl.Xh[cur]; ga.B[1] = pl.Xl[cur];
-      ga.A[2] = pl.Xl[cur]; ga.B[2] = pl.Xh[cur];
-      ga.nterms = 3;
-    }
-    ga.K = (int)N; ga.strideA = mn; ga.strideB = mn; ga.tiles_m = tM; ga.tiles_n = tM; ga.lower = 1;
-    {
-      AncProfScope prof(ANC_PROF_NS_GRAM, s);
-      if (big) { if (int rc = anc_ns_gemm_big(EPI_GRAM, ga, E, s)) return rc; }
-      else hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga);
-    }
-    ANC_LAUNCH_CHECK();
-    // B = b A + c A A
-    NsGemm gb = g;
-    gb.A[0] = pl.Fh; gb.B[0] = pl.Fh; gb.nterms = 1;
-    if (split_fb) {
-      gb.A[1] = pl.Fh; gb.B[1] = pl.Fl;
-      gb.A[2] = pl.Fl; gb.B[2] = pl.Fh;
-      gb.nterms = 3;
-    }
-    gb.K = (int)M; gb.strideA = M * M; gb.strideB = M * M; gb.tiles_m = tM; gb.tiles_n = tM; gb.lower = 1;
-    {
-      AncProfScope prof(ANC_PROF_NS_BMAT, s);
-      if (big) { if (int rc = anc_ns_gemm_big(EPI_BMAT, gb, E, s)) return rc; }
-      else hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb);
-    }
-    ANC_LAUNCH_CHECK();
-    // X = a X + B X
-    NsGemm gx = g;
-    gx.A[0] = pl.Bh; gx.B[0] = pl.Xh[cur]; gx.nterms = 1;
-    if (split) { gx.A[gx.nterms] = pl.Bh; gx.B[gx.nterms] = pl.Xl[cur]; ++gx.nterms; }
-    if (split_fb) { gx.A[gx.nterms] = pl.Bl; gx.B[gx.nterms] = pl.Xh[cur]; ++gx.nterms; }
-    gx.K = (int)M; gx.strideA = M * M; gx.strideB = mn; gx.tiles_m = tM; gx.tiles_n = tN; gx.lower = 0;
-    gx.Xh = pl.Xh[cur]; gx.Xl = pl.Xl[cur];
-    gx.Yh = last ? nullptr : pl.Xh[cur ^ 1];
-    gx.Yl = last ? nullptr : pl.Xl[cur ^ 1];
-    gx.X32 = last ? X32 : nullptr;
-    {
-      AncProfScope prof(ANC_PROF_NS_BX, s);
-      if (big) { if (int rc = anc_ns_gemm_big(EPI_BX, gx, E, s)) return rc; }
-      else hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx);
-    }
-    ANC_LAUNCH_CHECK();
-    cur ^= 1;
-  }
-  return ANC_OK;
+  return run_bf16_chain(pl, pl.Xh[0], pl.Xl[0], 1, nullptr, X32, E, M, N, steps, coef, force_small, s);
+}
+
+// The chain on an unnormalised bf16 pair (what anc_muon_momentum_multi_pair leaves) with the
+// Frobenius partial sums already known: X0 = U / (||U|| + eps) is never materialised, the first
+// step folds the scale into its epilogues.
+extern "C" int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partials, int64_t n_partials,
+                                   uint64_t X32_out, int64_t E, int64_t M, int64_t N, int steps,
+                                   const float *coef, float eps, int mode, uint64_t workspace,
+                                   int64_t workspace_bytes, uint64_t stream) {
+  const bool force_small = (mode & ANC_NS_TILE128) != 0;
+  mode &= ~ANC_NS_TILE128;
+  if (int rc = check_shape(E, M, N, mode, "anc_ns_batched_pair")) return rc;
+  ANC_REQUIRE(mode != ANC_NS_FP32, "anc_ns_batched_pair: the fp32 chain takes fp32 input (anc_ns_batched)");
+  ANC_REQUIRE(Uh != 0 && Ul != 0 && ((Uh | Ul) & 15) == 0 && X32_out != 0 && (X32_out & 15) == 0,
+              "anc_ns_batched_pair: pointers must be 16-byte aligned and non-null");
+  ANC_REQUIRE(fro_partials != 0 && n_partials > 0 && n_partials < (1 << 30),
+              "anc_ns_batched_pair: need the Frobenius partial sums (n_partials per matrix)");
+  ANC_REQUIRE(steps >= 2 && steps <= 64 && coef != nullptr,
+              "anc_ns_batched_pair: steps=%d: needs at least 2 steps (the fp32 result may overlay the input pair)", steps);
+  ANC_REQUIRE(workspace != 0 && (workspace & 255) == 0, "anc_ns_batched_pair: workspace must be 256-byte aligned");
+  const Plan pl = make_plan(workspace, E, M, N, mode, steps);
+  ANC_REQUIRE(workspace_bytes >= pl.bytes, "anc_ns_batched_pair: workspace holds %lld bytes, %lld needed",
+              (long long)workspace_bytes, (long long)pl.bytes);
+  hipStream_t s = anc_stream(stream);
+  { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s,
+                     (const double *)fro_partials, (int)n_partials, eps, pl.recip); }
+  ANC_LAUNCH_CHECK();
+  return run_bf16_chain(pl, (const uint16_t *)Uh, (const uint16_t *)Ul, 0, pl.recip, (float *)X32_out, E, M, N,
+                        steps, coef, force_small, s);
 }

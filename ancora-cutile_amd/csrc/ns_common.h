@@ -56,6 +56,9 @@ struct NsGemm {
   const uint16_t *Xh, *Xl;   // (E,M,N) current iterate as a bf16 pair, X = Xh + Xl   BX in
   uint16_t *Yh, *Yl;         // (E,M,N) next iterate as a bf16 pair   BX out, null on the last step
   float *X32;                // (E,M,N) fp32 result                   BX out on the last step, else null
+  const float *scale;        // (E) or null. The operands are an unnormalised iterate U and the step
+                             // acts on X = scale*U: GRAM multiplies its accumulator by scale^2, BX
+                             // multiplies the accumulator and the epilogue's X by scale.
 };
 
 

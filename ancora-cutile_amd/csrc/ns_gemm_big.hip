@@ -332,6 +332,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   unsigned char *region = st(wave / WPS) + (wave % WPS) * kStageRegion;
   const int gi0w = tm * TM + wm * 128, gj0w = tn * TN + wn * 64;
   const bool mirror = (EPI != EPI_BX) && (TN * (tn + 1) <= TM * tm);
+  float sc = 1.0f;
+  if (EPI != EPI_BMAT && p.scale != nullptr) sc = p.scale[e];
+  const float acc_scale = (EPI == EPI_GRAM) ? sc * sc : sc;
 
   // X = a X + B X reads the iterate at the output position (the bf16 pair Xh, Xl). A 32x64 slab
   // of each is 32 rows of 128 bytes: 4 DMA instructions (8 rows each, lane -> row lane/8, chunk
@@ -396,7 +399,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           const int ro = (8 * (r >> 2) + (r & 3)) * 128;
           const uint16_t xh = *(const uint16_t *)(b + in_lane[bj] + ro);
           const uint16_t xl = *(const uint16_t *)(b + 4096 + in_lane[bj] + ro);
-          in[bj][r] = anc_bf16_bits_to_f32(xh) + anc_bf16_bits_to_f32(xl);
+          in[bj][r] = (anc_bf16_bits_to_f32(xh) + anc_bf16_bits_to_f32(xl)) * sc;
         }
       region = const_cast<unsigned char *>(b);
     }
@@ -415,7 +418,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       for (int r = 0; r < 16; ++r) {
         const int gi = gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         const int gj = gj0w + bj * 32 + (lane & 31);
-        const float v = acc[bi][bj][r];
+        const float v = (EPI == EPI_BMAT) ? acc[bi][bj][r] : acc[bi][bj][r] * acc_scale;
         if (EPI == EPI_GRAM) {
           const bool diag = gi == gj;
           const uint16_t fh = diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v);

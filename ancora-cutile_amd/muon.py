@@ -58,6 +58,7 @@ class _Batch:
         self.table = None
         self.key = None
         self.total_blocks = 0
+        self.fro = None              # per-block sums of u*u left by the pair momentum kernel
 
     def build(self, U, scale_index):
         key = tuple((w["G"].ptr, w["G"].dtype.str, w["p32"].ptr, w["p16"].ptr if w["p16"] is not None else 0,
@@ -82,6 +83,9 @@ class _Batch:
         if self.table is not None:
             self.table.free()
             self.table = None
+        if self.fro is not None:
+            self.fro.free()
+            self.fro = None
 
 
 class MuonEngine:
@@ -100,6 +104,11 @@ class MuonEngine:
         self.mom, self.ns, self.nesterov = float(momentum), int(ns_steps), bool(nesterov)
         self.mode, self.sr, self.seed = mode, bool(sr), int(seed)
         self.t = 0
+        # Fused prologue: the momentum kernel writes the chain's bf16-pair input and the partial
+        # sums of the Frobenius norm, and the first Newton-Schulz step applies the scale, so the
+        # norm and scaling passes over the batch do not exist. Needs a bf16 mode and >= 2 steps
+        # (the fp32 result overlays the pair); otherwise the fp32 hand-off is used.
+        self.fused_prologue = mode != "fp32" and self.ns >= 2
         groups = {}
         scales = []
         for idx, w in enumerate(weights):
@@ -179,11 +188,22 @@ class MuonEngine:
                 if i < len(self._streams):
                     self._fork.wait_on(st)
             b.build(b.U, self.scale_index)
-            api.anc_muon_momentum_multi(b.table.ptr, b.E, b.total_blocks, self.mom,
-                                        int(self.nesterov), F32, ctl, int(st))
             buf = b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self.mode))
-            api.anc_ns_batched(b.U.ptr, b.E, b.M, b.Nn, self.ns, coef, 1e-7,
-                               muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(st))
+            if self.fused_prologue:
+                if b.fro is None:
+                    b.fro = DevBuf.empty((b.total_blocks,), np.float64)
+                n_el = b.E * b.M * b.Nn
+                api.anc_muon_momentum_multi_pair(b.table.ptr, b.E, b.total_blocks, self.mom,
+                                                 int(self.nesterov), b.U.ptr, n_el * 2, b.fro.ptr,
+                                                 ctl, int(st))
+                api.anc_ns_batched_pair(b.U.ptr, b.U.ptr + n_el * 2, b.fro.ptr,
+                                        b.total_blocks // b.E, b.U.ptr, b.E, b.M, b.Nn, self.ns, coef,
+                                        1e-7, muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(st))
+            else:
+                api.anc_muon_momentum_multi(b.table.ptr, b.E, b.total_blocks, self.mom,
+                                            int(self.nesterov), F32, ctl, int(st))
+                api.anc_ns_batched(b.U.ptr, b.E, b.M, b.Nn, self.ns, coef, 1e-7,
+                                   muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(st))
             api.anc_muon_update_multi(b.table.ptr, b.E, b.total_blocks, lr_scales, F32,
                                       int(self.sr), seed_base, ctl, int(st))
             if forked:

@@ -130,6 +130,25 @@ def ns_batched(X32, E, M, N, si, steps=5, eps=1e-7, schedule=_KELLER, mode="bf16
 ns_fp32_batched = ns_batched
 
 
+def ns_batched_pair(U, fro_partials, n_partials, E, M, N, si, steps=5, eps=1e-7, schedule=_KELLER,
+                    mode="bf16", workspace=None):
+    """The chain on what `anc_muon_momentum_multi_pair` leaves in the packed buffer U (an
+    E*M*N fp32-sized DevBuf holding the bf16 pair of the unnormalised input: hi in its first
+    half, lo in its second) and the per-block sums of squares in `fro_partials`; U is
+    overwritten with the fp32 result. No norm pass, no scaling pass."""
+    schedule = _resolve(schedule)
+    if U.dtype != np.float32 or U.size < E * M * N:
+        raise ValueError(f"ns_batched_pair: U must hold {E}x{M}x{N} float32, has {U.size} {U.dtype}")
+    if mode == "fp32" or steps < 2:
+        raise ValueError("ns_batched_pair: bf16 modes and steps >= 2 only")
+    ws = _SHARED_WS if workspace is None else workspace
+    buf = ws.ensure(ns_workspace_bytes(E, M, N, mode))
+    coef = coef_array(schedule, steps)
+    api.anc_ns_batched_pair(U.ptr, U.ptr + E * M * N * 2, fro_partials.ptr, int(n_partials), U.ptr,
+                            E, M, N, int(steps), coef, float(eps), MODES[mode], buf.ptr, buf.nbytes,
+                            int(si))
+
+
 def _run_bf16(gX, E, M, N, si, steps, eps, schedule, mode, workspace):
     if gX.dtype != np.uint16 or gX.size < E * M * N:
         raise ValueError("newton_schulz_resident: gX must hold the packed bf16 (uint16) batch")

@@ -260,6 +260,16 @@ typedef struct {
 int anc_muon_momentum_multi(uint64_t desc_table, int32_t n_weights, int64_t total_tiles,
                             float mom, int nesterov, int u_dtype,
                             uint64_t ctl, uint64_t stream);
+/* Momentum straight into the Newton-Schulz input format (replaces `_muon_mom`/`_muon_mom_t`
+ * plus the norm pass `_fro`, ancora/kernels/muon_ns.py:156-186, 206-217). desc.u is each
+ * weight's fp32 slice of the packed batch that starts at pair_base; the bf16 pair of u is
+ * written at the same element offset into two bf16 arrays, hi at pair_base, lo
+ * lo_offset_bytes behind it, and block b leaves the sum of its 4096 u*u (fp64, fixed
+ * order) in fro_partials[b]: K*N/4096 consecutive partials per weight. */
+int anc_muon_momentum_multi_pair(uint64_t desc_table, int32_t n_weights, int64_t total_tiles,
+                                 float mom, int nesterov, uint64_t pair_base,
+                                 int64_t lo_offset_bytes, uint64_t fro_partials,
+                                 uint64_t ctl, uint64_t stream);
 /* lr_scales: host array of ANC_MUON_MAX_SCALES values lr * sqrt(max(1, K/N))
  * (ancora/optim/muon.py:308), one per distinct weight shape class; the table itself
  * holds nothing that changes from step to step. */
@@ -306,6 +316,20 @@ int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N,
                    int steps, const float *coef /* host, 3*steps */, float eps,
                    int mode, uint64_t workspace, int64_t workspace_bytes,
                    uint64_t stream);
+
+/* The same chain fed by anc_muon_momentum_multi_pair: the momentum kernel leaves the
+ * unnormalised input U as a bf16 pair (Uh = bf16(u), Ul = bf16(u - Uh), both (E,M,N)) and
+ * n_partials sums of u*u per matrix; the reference's separate norm and scale passes
+ * (`_fro` + `_scale_e`, ancora/kernels/muon_ns.py:156-174, 387-406) disappear: the scale
+ * 1/(||U||_F + eps) is applied inside the first step's epilogues (A = s^2 U U^T,
+ * X1 = s (a U + B U)). The fp32 result goes to X32_out, which may overlay the input pair
+ * (Uh at X32_out, Ul right behind it: the same 4 bytes per element); steps >= 2. bf16
+ * modes only. Results differ from anc_ns_batched on the same data only by where the bf16
+ * rounding of the first operand falls (before instead of after the scaling). */
+int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partials, int64_t n_partials,
+                        uint64_t X32_out, int64_t E, int64_t M, int64_t N,
+                        int steps, const float *coef, float eps, int mode,
+                        uint64_t workspace, int64_t workspace_bytes, uint64_t stream);
 
 /* Matrix-core FLOPs of one anc_ns_batched call: `executed` counts the tiles and terms the
  * kernels really multiply (lower-triangle tiles of the symmetric products, residual terms),

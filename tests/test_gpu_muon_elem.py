@@ -105,3 +105,42 @@ def test_shape_checks(gpu):
     with pytest.raises(_lib.AncoraError):
         api.anc_muon_update(0, 0, b.ptr, 128, 128, 0.1, 0, _lib.F32, 0, 0, 0, 0)
     b.free()
+
+
+@pytest.mark.parametrize("K,N", [(128, 256), (256, 128)])
+def test_momentum_pair_output_and_frobenius_partials(gpu, K, N):
+    """The pair momentum kernel: momentum buffer bit-exact, u leaves as hi = bf16(u) and
+    lo = bf16(u - hi) in the chain's orientation, and the per-block sums of u*u add up to the
+    fp64 sum of squares (each block sums 4096 fp32 values in fp64: exact to ~1e-15 relative)."""
+    from ancora_cutile_amd import DevBuf, _lib
+    from ancora_cutile_amd._lib import api, MuonDesc
+    from ancora_cutile_amd.devbuf import upload_table
+    rng = np.random.default_rng(K + N)
+    E = 3
+    M, Nn = min(K, N), max(K, N)
+    tr = int(K > N)
+    bufs0 = [rng.standard_normal((K, N)).astype(np.float32) for _ in range(E)]
+    gs = [rng.standard_normal((K, N)).astype(np.float32) for _ in range(E)]
+    U = DevBuf.zeros((E * M * Nn,), np.float32)
+    fro = DevBuf.zeros((E * K * N // 4096,), np.float64)
+    bd = [DevBuf(b) for b in bufs0]
+    gd = [DevBuf(g) for g in gs]
+    descs, blk0 = [], 0
+    for i in range(E):
+        descs.append(MuonDesc(bd[i].ptr, gd[i].ptr, 0, 0, U.ptr + i * M * Nn * 4, K, N, tr, _lib.F32, 0, i, blk0))
+        blk0 += K * N // 4096
+    table = upload_table(descs)
+    api.anc_muon_momentum_multi_pair(table.ptr, E, blk0, 0.95, 1, U.ptr, E * M * Nn * 2, fro.ptr, 0, 0)
+    pair = U.view((2, E, M, Nn), np.uint16).to_numpy()
+    parts = fro.to_numpy().reshape(E, -1)
+    for i in range(E):
+        wb, wu = muon_momentum(bufs0[i], gs[i], 0.95, True)
+        assert bits_equal(bd[i].to_numpy(), wb)
+        wu = np.ascontiguousarray(wu.T) if tr else wu
+        hi = bf16_rne_bits(wu).reshape(M, Nn)
+        lo = bf16_rne_bits(wu - bits_to_f32(hi).reshape(M, Nn)).reshape(M, Nn)
+        assert bits_equal(pair[0, i], hi) and bits_equal(pair[1, i], lo)
+        want = float(np.sum(wu.astype(np.float64) ** 2))
+        assert abs(parts[i].sum() - want) <= 1e-12 * want
+    for b in bd + gd + [U, fro, table]:
+        b.free()

@@ -149,3 +149,32 @@ def test_shape_errors(gpu):
     with pytest.raises(_lib.AncoraError):
         ns_batched(d, 1, 64, 512, 0)             # not 128-aligned
     d.free()
+
+
+@pytest.mark.parametrize("M,N,mode", [(128, 384, "bf16"), (256, 512, "bf16_fast"), (1024, 1024, "bf16"),
+                                      (1024, 2048, "bf16_fast")])
+def test_pair_entry_folds_the_normalisation(gpu, M, N, mode):
+    """anc_ns_batched_pair: unnormalised bf16-pair input + sums of squares, scale applied inside
+    the first step. Same bar against the fp32 oracle as the fp32-input entry (3e-3 for the
+    mode without residual terms, which carries no bar of its own), and as close to that entry's
+    result as two independent roundings of the first operand allow. The input scale (1e-3
+    here) must not matter."""
+    from ancora_cutile_amd import DevBuf
+    from ancora_cutile_amd.muon_ns import ns_batched_pair
+    rng = np.random.default_rng(M + 5 * N)
+    E = 2
+    X = (1e-3 * rng.standard_normal((E, M, N))).astype(np.float32)
+    hi = bf16_rne_bits(X).reshape(E, M, N)
+    lo = bf16_rne_bits(X - bits_to_f32(hi).reshape(E, M, N)).reshape(E, M, N)
+    U = DevBuf(np.concatenate([hi.reshape(-1), lo.reshape(-1)]).view(np.float32))
+    nper = 4
+    parts = (X.astype(np.float64) ** 2).reshape(E, nper, -1).sum(axis=2)
+    fro = DevBuf(np.ascontiguousarray(parts))
+    ns_batched_pair(U, fro, nper, E, M, N, 0, steps=5, schedule=PE_SCHEDULE, mode=mode)
+    got = U.to_numpy().reshape(E, M, N)
+    ref = run_ns(X, mode=mode)
+    tol = TOL_BF16 if mode == "bf16" else 3e-3
+    for e in range(E):
+        assert rel_fro(got[e], host_ns(X[e], PE_SCHEDULE, 5)) < tol
+        assert rel_fro(got[e], ref[e]) < 3e-3
+    U.free(); fro.free()
