@@ -10,7 +10,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libancora_optim.so")
+# ANCORA_OPTIM_LIB names another build of the same library (an ablation variant, see build.py)
+LIB_PATH = os.environ.get("ANCORA_OPTIM_LIB") or os.path.join(_HERE, "csrc", "libancora_optim.so")
 
 F32, BF16 = 0, 1                  # ANC_F32 / ANC_BF16
 FORM_DIV, FORM_IBC = 0, 1         # ANC_ADAMW_FORM_*

@@ -1,6 +1,12 @@
 """Compile the HIP sources under csrc/ into csrc/libancora_optim.so for gfx950.
 
     python -m ancora_cutile_amd.build
+    python -m ancora_cutile_amd.build --define ANC_DBG_NOEPI --out /tmp/noepi.so
+
+The second form builds an ablation variant somewhere else (objects in a temporary directory,
+the product library untouched); `ANCORA_OPTIM_LIB=/tmp/noepi.so` makes the host layer load it.
+Ablation switches of csrc/ns_gemm_big.hip: ANC_DBG_NOEPI (no epilogue), ANC_DBG_NODMA (operand
+tiles fetched for the first K tiles only), ANC_DBG_NOMFMA (matrix instructions replaced by an add).
 
 hipcc cross-compiles without a GPU. Flags: no FMA contraction (the AdamW kernel must
 reproduce a numpy fp32 evaluation operation by operation), correctly rounded fp32
@@ -10,6 +16,7 @@ import glob
 import os
 import subprocess
 import sys
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -21,16 +28,18 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
          "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
 
 
-def build(verbose=True):
+def build(verbose=True, defines=(), out=None):
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     if not srcs:
         raise RuntimeError(f"no HIP sources under {CSRC}")
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    target = out or OUT
+    objdir = CSRC if target == OUT else tempfile.mkdtemp(prefix="ancora_build_")
     objs = []
     procs = []
     for s in srcs:
-        o = s[:-4] + ".o"
-        cmd = [hipcc, *[f for f in FLAGS if f != "-shared"], "-c", s, "-o", o]
+        o = os.path.join(objdir, os.path.basename(s)[:-4] + ".o")
+        cmd = [hipcc, *[f for f in FLAGS if f != "-shared"], *[f"-D{d}" for d in defines], "-c", s, "-o", o]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((s, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
@@ -46,12 +55,17 @@ def build(verbose=True):
             failed = True
     if failed:
         raise RuntimeError("hipcc failed")
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", OUT]
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", target]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    return OUT
+    return target
 
 
 if __name__ == "__main__":
-    print(build())
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--define", action="append", default=[], help="extra -D for every source")
+    ap.add_argument("--out", default=None, help="output library (default: csrc/libancora_optim.so)")
+    a = ap.parse_args()
+    print(build(defines=a.define, out=a.out))

@@ -1,7 +1,9 @@
 """Single-kernel profiling targets for rocprofv3 (the role of the reference's Nsight Compute
 targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
 
-    python3 -m ancora_cutile_amd.prof_target ns M N E [mode] [calls]     Newton-Schulz chain
+    python3 -m ancora_cutile_amd.prof_target ns M N E [mode] [calls] [times]   Newton-Schulz chain
+                                      (a last word `times` adds one call under the library's
+                                      per-launch event timer and prints ms per kernel kind)
     python3 -m ancora_cutile_amd.prof_target adamw NUMEL [calls]         fused AdamW, bf16 grads, SR
     python3 -m ancora_cutile_amd.prof_target gradnorm NUMEL [calls]      grad-norm partials + finalize
 
@@ -30,6 +32,13 @@ def main(argv):
             X.at_pos(e * M).upload(one)
         for _ in range(calls):
             ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
+        if len(argv) > 6 and argv[6] == "times":
+            _lib.stream_sync(0)
+            _lib.profile_enable(True)
+            ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
+            pr = _lib.profile_read()
+            _lib.profile_enable(False)
+            print("  ".join(f"{k}={v[0]:.3f}ms/{v[1]}" for k, v in pr.items() if v[1]))
     elif what == "adamw":
         n = int(argv[1]) // 64 * 64
         calls = int(argv[2]) if len(argv) > 2 else 3
