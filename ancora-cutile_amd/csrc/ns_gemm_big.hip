@@ -41,6 +41,14 @@
 #define ANC_DBG_EPI 0
 #endif
 
+#ifdef ANC_DBG_TRACE
+// Debug build only: per-workgroup timestamps (100 MHz wall clock) of the last launch of each kind.
+__device__ unsigned long long anc_dbg_ts[3][16384][4];
+extern "C" int anc_dbg_trace_read(void *host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(anc_dbg_ts), sizeof(unsigned long long) * 3 * 16384 * 4);
+}
+#endif
+
 namespace {
 
 #define LDS3(p) ((__attribute__((address_space(3))) void *)(p))
@@ -185,6 +193,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     return i == 0 ? stage0 : i == 1 ? stage1 : i == 2 ? stage2 : stage3;
   };
 
+#ifdef ANC_DBG_TRACE
+  const unsigned long long dbg_t0 = wall_clock64();
+#endif
   const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
   // Symmetric outputs: only tiles that reach the diagonal or lie below it. Row tm of TM-row
   // tiles has tm/R + 1 of them (R = TN/TM); a tile entirely below the diagonal is mirrored.
@@ -324,6 +335,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   __syncthreads();
 
   // ---- epilogue
+#ifdef ANC_DBG_TRACE
+  const unsigned long long dbg_t1 = wall_clock64();
+#endif
 #ifdef ANC_DBG_NOEPI
   if (acc[0][0][0] + acc[3][1][7] != 12345.678f) return;
 #endif
@@ -343,7 +357,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // 16-byte chunk index is XORed with 4*((row>>2)&1): the two half-wavefronts, which read rows
   // 4 apart, then use different banks. The same buffer stages the slab's bf16 outputs.
   constexpr int kInBuf = 8192, kBufPerStage = kStage / kInBuf;
-  static_assert(EPI != EPI_BX || (kBufPerStage * NS >= 2 * NWAVES && kInBuf >= kStageRegion), "epilogue buffers");
+  static_assert(EPI != EPI_BX || (kBufPerStage * NS >= 2 * NWAVES + 1 && kInBuf >= kStageRegion &&
+                                  NWAVES * 1024 <= kInBuf && TM == 128), "epilogue buffers");
   auto inbuf = [&](int bi) -> unsigned char * {
     const int q = wave * 2 + (bi & 1);
     return st(q / kBufPerStage) + (q % kBufPerStage) * kInBuf;
@@ -360,10 +375,16 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     }
   };
   int in_lane[2] = {0, 0};
+  unsigned char *dvec_lds = st((2 * NWAVES) / kBufPerStage) + ((2 * NWAVES) % kBufPerStage) * kInBuf + wave * 1024;
   if (EPI == EPI_BX) {
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj)
       in_lane[bj] = 4 * (lane >> 5) * 128 + (((bj * 4 + ((lane & 31) >> 3)) ^ ((lane >> 5) << 2)) * 16) + (lane & 7) * 2;
+    asm volatile("" : "+v"(sc));      // the scale has arrived before the first DMA is issued
+    // dB of the tile's 128 rows, one private copy per wavefront (lanes 32..63 repeat lanes 0..31),
+    // fetched first: any ordinary load issued after the slab fetches would, completing in
+    // order, wait for them.
+    dma16((const char *)(p.dB + mv + gi0w) + (lane & 31) * 16, lds_addr(dvec_lds));
     fetch_in(0);
     fetch_in(1);
   }
@@ -389,8 +410,16 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         }
     }
     if (EPI == EPI_BX) {
+      // Wait for this slab's DMA only. Vector memory operations complete in issue order, and
+      // after the fetch of slab bi this wavefront issued: the fetch of slab bi+1 (8 DMA, at the
+      // end of slab bi-1, or up front for slab 1) and before it the stores of slab bi-1 (32
+      // dword stores of the fp32 result on the last step, else 2 x 4 stores of the pair).
+      // Nothing else in this epilogue is a vector memory operation.
+      const bool fp32_out = p.X32 != nullptr;
+      if (bi == 0) wait_vm<8>();
+      else if (bi == 3) { if (fp32_out) wait_vm<32>(); else wait_vm<8>(); }
+      else { if (fp32_out) wait_vm<40>(); else wait_vm<16>(); }
       // X = Xh + Xl is exact in fp32 (8 + 8 significant bits)
-      wait_vm<0>();
       const unsigned char *b = inbuf(bi);
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj)
@@ -403,14 +432,19 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         }
       region = const_cast<unsigned char *>(b);
     }
-    if (EPI != EPI_GRAM) {
-      const float *dvec = (EPI == EPI_BMAT) ? p.dA + mv : p.dB + mv;
+    if (EPI == EPI_BX) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const anc_f32x4 d4 = *(const anc_f32x4 *)(dvec_lds + (bi * 32 + 8 * q + 4 * (lane >> 5)) * 4);
+        drow[4 * q] = d4.x; drow[4 * q + 1] = d4.y; drow[4 * q + 2] = d4.z; drow[4 * q + 3] = d4.w;
+      }
+    }
+    if (EPI == EPI_BMAT) {
+      const float *dvec = p.dA + mv;
 #pragma unroll
       for (int r = 0; r < 16; ++r) drow[r] = dvec[gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
-      if (EPI == EPI_BMAT) {
 #pragma unroll
-        for (int bj = 0; bj < 2; ++bj) dcol[bj] = dvec[gj0w + bj * 32 + (lane & 31)];
-      }
+      for (int bj = 0; bj < 2; ++bj) dcol[bj] = dvec[gj0w + bj * 32 + (lane & 31)];
     }
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj) {
@@ -477,6 +511,18 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       if (bi + 2 < 4) fetch_in(bi + 2);
     }
   }
+#ifdef ANC_DBG_TRACE
+  if (threadIdx.x == 0 && blockIdx.x < 16384) {
+    unsigned int hwid;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+    unsigned int xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    anc_dbg_ts[EPI][blockIdx.x][0] = dbg_t0;
+    anc_dbg_ts[EPI][blockIdx.x][1] = dbg_t1;
+    anc_dbg_ts[EPI][blockIdx.x][2] = wall_clock64();
+    anc_dbg_ts[EPI][blockIdx.x][3] = ((unsigned long long)xcc << 32) | hwid;
+  }
+#endif
 }
 
 template <int EPI>
