@@ -45,6 +45,9 @@ namespace {
 
 using namespace anc_reduce;
 
+// bf16 (round to nearest even) by the hardware conversion, as in the 256-tile kernel
+__device__ __forceinline__ uint32_t hw_bf16(float x) { return anc_pk_bf16(x, 0.0f) & 0xFFFFu; }
+
 template <int EPI>
 __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
   __shared__ __attribute__((aligned(16))) uint16_t sA[BM * PITCH];
@@ -156,7 +159,7 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
         const float v = (EPI == EPI_BMAT) ? acc[bi][bj][r] : acc[bi][bj][r] * acc_scale;
         if (EPI == EPI_GRAM) {
           const bool diag = gi == gj;
-          const uint16_t fh = diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v);
+          const uint16_t fh = diag ? (uint16_t)0 : (uint16_t)hw_bf16(v);
           p.A32[mm + (int64_t)gi * M + gj] = v;
           p.Fh[mm + (int64_t)gi * M + gj] = fh;
           if (tm != tn) {
@@ -165,7 +168,7 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
           }
           if (p.Fl != nullptr) {
             const uint16_t fl =
-                diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v - anc_bf16_bits_to_f32(fh));
+                diag ? (uint16_t)0 : (uint16_t)hw_bf16(v - anc_bf16_bits_to_f32(fh));
             p.Fl[mm + (int64_t)gi * M + gj] = fl;
             if (tm != tn) p.Fl[mm + (int64_t)gj * M + gi] = fl;
           }
@@ -177,8 +180,8 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
           if (gi != gj) {
             const float a2 = v + (di * a + a * dj);   // symmetric in (i,j)
             const float bv = p.cb * a + p.cc * a2;
-            bh = (uint16_t)anc_bf16_rne_bits(bv);
-            bl = (uint16_t)anc_bf16_rne_bits(bv - anc_bf16_bits_to_f32(bh));
+            bh = (uint16_t)hw_bf16(bv);
+            bl = (uint16_t)hw_bf16(bv - anc_bf16_bits_to_f32(bh));
           } else {
             const float a2 = v + di * di;
             p.dB[mv + gi] = p.cb * di + p.cc * a2;
@@ -196,9 +199,9 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
           const float y = (p.ca + p.dB[mv + gi]) * x + v;
           if (p.X32 != nullptr) p.X32[o] = y;
           if (p.Yh != nullptr) {
-            const uint32_t yh = anc_bf16_rne_bits(y);
+            const uint32_t yh = hw_bf16(y);
             p.Yh[o] = (uint16_t)yh;
-            p.Yl[o] = (uint16_t)anc_bf16_rne_bits(y - anc_bf16_bits_to_f32(yh));
+            p.Yl[o] = (uint16_t)hw_bf16(y - anc_bf16_bits_to_f32(yh));
           }
         }
       }

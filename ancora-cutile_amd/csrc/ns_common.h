@@ -21,6 +21,19 @@ __device__ __forceinline__ bf16x8 anc_lds_tr_frag(const void *p0, const void *p1
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// Two fp32 -> one dword of two bf16 (round to nearest even, v_cvt_pk_bf16_f32): a in the low half.
+typedef __bf16 anc_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float anc_f32x2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t anc_pk_bf16(float a, float b) {
+  const anc_f32x2v v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, anc_bf16x2));
+}
+// The bf16 pair of two values: hi = bf16(x), lo = bf16(x - hi), each packed as above.
+__device__ __forceinline__ void anc_pk_pair(float a, float b, uint32_t &hi, uint32_t &lo) {
+  hi = anc_pk_bf16(a, b);
+  lo = anc_pk_bf16(a - __uint_as_float(hi << 16), b - __uint_as_float(hi & 0xFFFF0000u));
+}
+
 constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int PITCH = BK + 8;            // bf16 elements per LDS row: 144 bytes
 constexpr int kGemmThreads = 256;

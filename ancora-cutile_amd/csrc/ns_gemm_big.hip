@@ -96,43 +96,57 @@ __device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
 #endif
 }
 
-// bf16 tile staging through LDS. `v` holds, for the wavefront's 32-row slab, the 16-bit values
-// of its 2 column blocks in accumulator layout (row 8*(r/4) + 4*(lane/32) + r%4, column
-// bj*32 + lane%32). Row-major output: out[row*ld + col]; transposed: outT[col*ldT + row].
-__device__ __forceinline__ void stage_rows(unsigned char *region, const uint16_t (&v)[2][16], int lane,
+// bf16 tile staging through LDS. `v` holds, for the wavefront's 32-row slab, the bf16 values of
+// its 2 column blocks in accumulator layout (element r: row 8*(r/4) + 4*(lane/32) + r%4, column
+// bj*32 + lane%32), packed two per dword: v[bj][i] = elements r = 2i (low half), 2i+1 (high).
+// Row-major output: out[row*ld + col]; transposed: outT[col*ldT + row].
+__device__ __forceinline__ void stage_rows(unsigned char *region, const uint32_t (&v)[2][8], int lane,
                                            uint16_t *out, int64_t ld) {
   uint16_t *t = (uint16_t *)region;                 // [32][72]
 #pragma unroll
   for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
     for (int r = 0; r < 16; ++r)
-      t[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 72 + bj * 32 + (lane & 31)] = v[bj][r];
+      t[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 72 + bj * 32 + (lane & 31)] =
+          (uint16_t)((r & 1) ? (v[bj][r >> 1] >> 16) : (v[bj][r >> 1] & 0xFFFFu));
   __builtin_amdgcn_s_waitcnt(0xC07F);               // lgkmcnt(0): this wavefront's LDS writes landed
   __builtin_amdgcn_wave_barrier();
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, row = idx >> 3, c8 = (idx & 7) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + row * 72 + c8);
+#ifdef ANC_DBG_NOSTORE
+    if (q.x == 0x12345678u) anc_st_stream((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
+#else
     anc_st_stream((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
+#endif
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
 }
-__device__ __forceinline__ void stage_cols(unsigned char *region, const uint16_t (&v)[2][16], int lane,
+// Transposed: a lane's 4 consecutive rows are 4 consecutive elements of an output row, so they
+// go to LDS as one 8-byte write.
+__device__ __forceinline__ void stage_cols(unsigned char *region, const uint32_t (&v)[2][8], int lane,
                                            uint16_t *outT, int64_t ldT) {
   uint16_t *t = (uint16_t *)region;                 // [64][40]
 #pragma unroll
   for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-    for (int r = 0; r < 16; ++r)
-      t[(bj * 32 + (lane & 31)) * 40 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)] = v[bj][r];
+    for (int q = 0; q < 4; ++q) {
+      const anc_u32x2 w = {v[bj][2 * q], v[bj][2 * q + 1]};
+      *(anc_u32x2 *)(t + (bj * 32 + (lane & 31)) * 40 + 8 * q + 4 * (lane >> 5)) = w;
+    }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, col = idx >> 2, r8 = (idx & 3) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + col * 40 + r8);
+#ifdef ANC_DBG_NOSTORE
+    if (q.x == 0x12345678u) anc_st_stream((anc_u32x4 *)(outT + (int64_t)col * ldT + r8), q);
+#else
     anc_st_stream((anc_u32x4 *)(outT + (int64_t)col * ldT + r8), q);
+#endif
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
@@ -192,6 +206,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   auto st = [&](int i) -> unsigned char * {
     return i == 0 ? stage0 : i == 1 ? stage1 : i == 2 ? stage2 : stage3;
   };
+  // B = b A + c A A: per-wavefront copy of the dA entries of its 128 rows and 64 columns
+  __shared__ __attribute__((aligned(1024))) unsigned char aux[EPI == EPI_BMAT ? NWAVES * 1024 : 16];
 
 #ifdef ANC_DBG_TRACE
   const unsigned long long dbg_t0 = wall_clock64();
@@ -357,6 +373,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // 16-byte chunk index is XORed with 4*((row>>2)&1): the two half-wavefronts, which read rows
   // 4 apart, then use different banks. The same buffer stages the slab's bf16 outputs.
   constexpr int kInBuf = 8192, kBufPerStage = kStage / kInBuf;
+  static_assert(EPI != EPI_BMAT || kBufPerStage * NS >= 2 * NWAVES, "epilogue buffers");
   static_assert(EPI != EPI_BX || (kBufPerStage * NS >= 2 * NWAVES + 1 && kInBuf >= kStageRegion &&
                                   NWAVES * 1024 <= kInBuf && TM == 128), "epilogue buffers");
   auto inbuf = [&](int bi) -> unsigned char * {
@@ -374,7 +391,30 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       dma16((const char *)p.Xl + ub + ro + vo_in, lds_addr(b + 4096 + j * 1024));
     }
   };
+  // B = b A + c A A reads A32 at the output position the same way: a 32x64 fp32 slab is 32 rows
+  // of 256 bytes, 8 DMA instructions (4 rows each, lane -> row lane/16, chunk lane%16), chunk
+  // index XORed with 8*((row>>2)&1).
+  const uint32_t vo_a0 = (uint32_t)((lane >> 4) * M * 4 + ((lane & 15) * 16));
+  const uint32_t vo_a1 = (uint32_t)((lane >> 4) * M * 4 + (((lane & 15) ^ 8) * 16));
+  auto fetch_a32 = [&](int bi) {
+    const int64_t ub = (mm + (int64_t)(gi0w + bi * 32) * M + gj0w) * 4;
+    unsigned char *b = inbuf(bi);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      dma16((const char *)p.A32 + ub + (int64_t)(4 * j) * M * 4 + ((j & 1) ? vo_a1 : vo_a0), lds_addr(b + j * 1024));
+  };
   int in_lane[2] = {0, 0};
+  unsigned char *aux_w = aux + (EPI == EPI_BMAT ? wave * 1024 : 0);
+  if (EPI == EPI_BMAT) {
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+      in_lane[bj] = 4 * (lane >> 5) * 256 + (((bj * 8 + ((lane & 31) >> 2)) ^ ((lane >> 5) << 3)) * 16) + (lane & 3) * 4;
+    // dA of the wavefront's rows (lanes 0..31) and columns (lanes 32..47, repeated by 48..63)
+    const float *dsrc = (lane < 32) ? p.dA + mv + gi0w + lane * 4 : p.dA + mv + gj0w + (lane & 15) * 4;
+    dma16(dsrc, lds_addr(aux_w));
+    fetch_a32(0);
+    fetch_a32(1);
+  }
   unsigned char *dvec_lds = st((2 * NWAVES) / kBufPerStage) + ((2 * NWAVES) % kBufPerStage) * kInBuf + wave * 1024;
   if (EPI == EPI_BX) {
 #pragma unroll
@@ -390,24 +430,31 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   }
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi) {
-    uint16_t hv[2][16], lv[2][16];
     const int gi0 = gi0w + bi * 32;
     // operands of the epilogue first (all loads in flight together), arithmetic after
     float in[2][16], drow[16], dcol[2];
     if (EPI == EPI_BMAT) {
-      const float *src = p.A32 + mm;
+      // Wait for this slab's DMA only (see the X = a X + B X branch). Stores of a slab: 4 per
+      // staged bf16 block (Bh, its mirror, and the same for Bl); the conditional dB stores of
+      // diagonal tiles only add to what may stay outstanding, so leaving them out is safe.
+      const int nst = 4 * ((mirror ? 2 : 1) * (p.Bl != nullptr ? 2 : 1));
+      if (bi == 0) wait_vm<8>();
+      else if (bi == 3) { if (nst == 4) wait_vm<4>(); else if (nst == 8) wait_vm<8>(); else wait_vm<16>(); }
+      else { if (nst == 4) wait_vm<12>(); else if (nst == 8) wait_vm<16>(); else wait_vm<24>(); }
+      const unsigned char *b = inbuf(bi);
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int gi = gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-          const int gj = gj0w + bj * 32 + (lane & 31);
-#if (ANC_DBG_EPI & 1)
-          in[bj][r] = 1.0f;
-#else
-          in[bj][r] = anc_ld_stream(src + (int64_t)gi * M + gj);
-#endif
-        }
+        for (int r = 0; r < 16; ++r)
+          in[bj][r] = *(const float *)(b + in_lane[bj] + (8 * (r >> 2) + (r & 3)) * 256);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const anc_f32x4 d4 = *(const anc_f32x4 *)(aux_w + (bi * 32 + 8 * q + 4 * (lane >> 5)) * 4);
+        drow[4 * q] = d4.x; drow[4 * q + 1] = d4.y; drow[4 * q + 2] = d4.z; drow[4 * q + 3] = d4.w;
+      }
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj) dcol[bj] = *(const float *)(aux_w + 512 + (bj * 32 + (lane & 31)) * 4);
+      region = const_cast<unsigned char *>(b);
     }
     if (EPI == EPI_BX) {
       // Wait for this slab's DMA only. Vector memory operations complete in issue order, and
@@ -439,13 +486,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         drow[4 * q] = d4.x; drow[4 * q + 1] = d4.y; drow[4 * q + 2] = d4.z; drow[4 * q + 3] = d4.w;
       }
     }
-    if (EPI == EPI_BMAT) {
-      const float *dvec = p.dA + mv;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) drow[r] = dvec[gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
-#pragma unroll
-      for (int bj = 0; bj < 2; ++bj) dcol[bj] = dvec[gj0w + bj * 32 + (lane & 31)];
-    }
+
+    float ov[2][16];          // the values that leave as bf16 (pairs)
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj) {
 #pragma unroll
@@ -455,36 +497,36 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         const float v = (EPI == EPI_BMAT) ? acc[bi][bj][r] : acc[bi][bj][r] * acc_scale;
         if (EPI == EPI_GRAM) {
           const bool diag = gi == gj;
-          const uint16_t fh = diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v);
+#ifdef ANC_DBG_NOSTORE
+          if (v == 12345.678f) p.A32[mm + (int64_t)gi * M + gj] = v;
+#else
           p.A32[mm + (int64_t)gi * M + gj] = v;
-          hv[bj][r] = fh;
-          lv[bj][r] = diag ? (uint16_t)0 : (uint16_t)anc_bf16_rne_bits(v - anc_bf16_bits_to_f32(fh));
+#endif
+          ov[bj][r] = diag ? 0.0f : v;
           if (diag) p.dA[mv + gi] = v;
         } else if (EPI == EPI_BMAT) {
           const float a = in[bj][r];
           const float di = drow[r], dj = dcol[bj];
-          uint16_t bh, bl = 0;
           if (gi != gj) {
             const float a2 = v + (di * a + a * dj);   // symmetric in (i,j)
-            const float bv = p.cb * a + p.cc * a2;
-            bh = (uint16_t)anc_bf16_rne_bits(bv);
-            bl = (uint16_t)anc_bf16_rne_bits(bv - anc_bf16_bits_to_f32(bh));
+            ov[bj][r] = p.cb * a + p.cc * a2;
           } else {
             const float a2 = v + di * di;
             p.dB[mv + gi] = p.cb * di + p.cc * a2;
-            bh = 0;
+            ov[bj][r] = 0.0f;
           }
-          hv[bj][r] = bh;
-          lv[bj][r] = bl;
         } else {
           const float y = (p.ca + drow[r]) * in[bj][r] + v;
           if (p.X32 != nullptr) anc_st_stream(p.X32 + mn + (int64_t)gi * N + gj, y);
-          const uint32_t yh = anc_bf16_rne_bits(y);
-          hv[bj][r] = (uint16_t)yh;
-          lv[bj][r] = (uint16_t)anc_bf16_rne_bits(y - anc_bf16_bits_to_f32(yh));
+          ov[bj][r] = y;
         }
       }
     }
+    uint32_t hv[2][8], lv[2][8];
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) anc_pk_pair(ov[bj][2 * i], ov[bj][2 * i + 1], hv[bj][i], lv[bj][i]);
     if (EPI == EPI_GRAM) {
       stage_rows(region, hv, lane, p.Fh + mm + (int64_t)gi0 * M + gj0w, M);
       if (mirror) stage_cols(region, hv, lane, p.Fh + mm + (int64_t)gj0w * M + gi0, M);
@@ -499,6 +541,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         stage_rows(region, lv, lane, p.Bl + mm + (int64_t)gi0 * M + gj0w, M);
         if (mirror) stage_cols(region, lv, lane, p.Bl + mm + (int64_t)gj0w * M + gi0, M);
       }
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      asm volatile("" ::: "memory");
+      if (bi + 2 < 4) fetch_a32(bi + 2);
     } else {
       if (p.Yh != nullptr) {
         stage_rows(region, hv, lane, p.Yh + mn + (int64_t)gi0 * N + gj0w, N);
