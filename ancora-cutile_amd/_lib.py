@@ -60,6 +60,12 @@ class MuonDesc(C.Structure):
                 ("seed", u32), ("tile0", i64)]
 
 
+class NsProblem(C.Structure):
+    """anc_ns_problem_t: one batch of the multi-batch chain entry."""
+    _fields_ = [("Uh", u64), ("Ul", u64), ("fro_partials", u64), ("X32_out", u64), ("workspace", u64),
+                ("n_partials", i64), ("E", i64), ("M", i64), ("N", i64), ("workspace_bytes", i64)]
+
+
 # name -> (restype, argtypes); restype None means "int status, checked".
 _PROTOS = {
     "anc_last_error": (C.c_char_p, []),
@@ -111,6 +117,8 @@ _PROTOS = {
                               u64]),
     "anc_ns_batched_pair": (None, [u64, u64, u64, i64, u64, i64, i64, i64, C.c_int, C.POINTER(f32), f32,
                                    C.c_int, u64, i64, u64]),
+    "anc_ns_batched_pair_multi": (None, [C.POINTER(NsProblem), i32, C.c_int, C.POINTER(f32), f32, C.c_int,
+                                         u64]),
     "anc_ns_flops": (None, [i64, i64, i64, C.c_int, C.c_int, C.POINTER(C.c_double),
                             C.POINTER(C.c_double)]),
     "anc_bf16_to_f32": (None, [u64, u64, i64, u64]),

@@ -460,79 +460,99 @@ int check_shape(int64_t E, int64_t M, int64_t N, int mode, const char *who) {
   return ANC_OK;
 }
 
-// steps x { A = X X^T; B = b A + c A A; X = a X + B X } on the bf16 pair (inH, inL). The first
-// step's output goes to pair `nxt` of the plan, later steps ping-pong; the last step writes the
-// fp32 result X32 (which may overlay the input pair when steps >= 2). `scale0`, if given, is the
-// per-matrix factor the first step applies to its unnormalised input.
-int run_bf16_chain(const Plan &pl, const uint16_t *inH, const uint16_t *inL, int nxt, const float *scale0,
-                   float *X32, int64_t E, int64_t M, int64_t N, int steps, const float *coef,
-                   bool force_small, hipStream_t s) {
-  const int64_t mn = M * N;
-  const int split_from = pl.sp.x_from;   // first iteration with X residual terms
-  const bool big = !force_small && (M % 256 == 0) && (N % 256 == 0);   // 256x256 tiles, same bits
-  const int tile = big ? 256 : BM;
-  const int tM = (int)(M / tile), tN = (int)(N / tile);
-  const unsigned g_sym = (unsigned)(E * tM * (tM + 1) / 2), g_mn = (unsigned)(E * tM * tN);
-  const uint16_t *curH = inH, *curL = inL;
+// One problem of a chain launch: a batch of E (M,N) matrices with its workspace plan.
+struct ChainProb {
+  Plan pl;
+  const uint16_t *inH, *inL;   // the input bf16 pair
+  int nxt;                     // which pair of the plan receives the first step's output
+  const float *scale0;         // per-matrix factor the first step applies to its input, or null
+  float *X32;                  // fp32 result (may overlay the input pair when steps >= 2)
+  int64_t E, M, N;
+};
+
+// steps x { A = X X^T; B = b A + c A A; X = a X + B X } on n problems side by side: every
+// product of a step is ONE launch over all problems (problems in the order given; put the
+// longest K first). First step's output goes to pair `nxt` of each plan, later steps ping-pong;
+// the last step writes the fp32 results. With n == 1 and a shape that is not a multiple of 256
+// (or force_small) the 128x128-tile kernel runs instead.
+int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool force_small, hipStream_t s) {
+  bool big = !force_small;
+  for (int q = 0; q < n; ++q) big = big && (cp[q].M % 256 == 0) && (cp[q].N % 256 == 0);
+  ANC_REQUIRE(big || n == 1, "Newton-Schulz chain: several problems per launch need dims that are multiples of 256");
+  const uint16_t *curH[kMaxGroups], *curL[kMaxGroups];
+  int nxt[kMaxGroups];
+  int64_t Es[kMaxGroups];
+  for (int q = 0; q < n; ++q) { curH[q] = cp[q].inH; curL[q] = cp[q].inL; nxt[q] = cp[q].nxt; Es[q] = cp[q].E; }
   for (int k = 0; k < steps; ++k) {
-    const bool split = k >= split_from;
-    const bool split_fb = k >= pl.sp.fb_from;
     const bool last = k + 1 == steps;
-    NsGemm g{};
-    g.M = (int)M; g.N = (int)N;
-    g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB;
-    g.Fl = split_fb ? pl.Fl : nullptr;
-    g.Bl = split_fb ? pl.Bl : nullptr;
-    g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
-    g.scale = (k == 0) ? scale0 : nullptr;
-    // A = X X^T
-    NsGemm ga = g;
-    ga.A[0] = curH; ga.B[0] = curH; ga.nterms = 1;
-    if (split) {
-      ga.A[1] = curH; ga.B[1] = curL;
-      ga.A[2] = curL; ga.B[2] = curH;
-      ga.nterms = 3;
+    NsGemm ga[kMaxGroups], gb[kMaxGroups], gx[kMaxGroups];
+    for (int q = 0; q < n; ++q) {
+      const Plan &pl = cp[q].pl;
+      const int64_t M = cp[q].M, N = cp[q].N, mn = M * N;
+      const bool split = k >= pl.sp.x_from;        // X residual terms
+      const bool split_fb = k >= pl.sp.fb_from;    // F and Boff residual terms
+      const int tile = big ? 256 : BM;
+      const int tM = (int)(M / tile), tN = (int)(N / tile);
+      NsGemm g{};
+      g.M = (int)M; g.N = (int)N;
+      g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB;
+      g.Fl = split_fb ? pl.Fl : nullptr;
+      g.Bl = split_fb ? pl.Bl : nullptr;
+      g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
+      g.scale = (k == 0) ? cp[q].scale0 : nullptr;
+      // A = X X^T
+      ga[q] = g;
+      ga[q].A[0] = curH[q]; ga[q].B[0] = curH[q]; ga[q].nterms = 1;
+      if (split) {
+        ga[q].A[1] = curH[q]; ga[q].B[1] = curL[q];
+        ga[q].A[2] = curL[q]; ga[q].B[2] = curH[q];
+        ga[q].nterms = 3;
+      }
+      ga[q].K = (int)N; ga[q].strideA = mn; ga[q].strideB = mn; ga[q].tiles_m = tM; ga[q].tiles_n = tM; ga[q].lower = 1;
+      // B = b A + c A A
+      gb[q] = g;
+      gb[q].A[0] = pl.Fh; gb[q].B[0] = pl.Fh; gb[q].nterms = 1;
+      if (split_fb) {
+        gb[q].A[1] = pl.Fh; gb[q].B[1] = pl.Fl;
+        gb[q].A[2] = pl.Fl; gb[q].B[2] = pl.Fh;
+        gb[q].nterms = 3;
+      }
+      gb[q].K = (int)M; gb[q].strideA = M * M; gb[q].strideB = M * M; gb[q].tiles_m = tM; gb[q].tiles_n = tM; gb[q].lower = 1;
+      // X = a X + B X
+      gx[q] = g;
+      gx[q].A[0] = pl.Bh; gx[q].B[0] = curH[q]; gx[q].nterms = 1;
+      if (split) { gx[q].A[gx[q].nterms] = pl.Bh; gx[q].B[gx[q].nterms] = curL[q]; ++gx[q].nterms; }
+      if (split_fb) { gx[q].A[gx[q].nterms] = pl.Bl; gx[q].B[gx[q].nterms] = curH[q]; ++gx[q].nterms; }
+      gx[q].K = (int)M; gx[q].strideA = M * M; gx[q].strideB = mn; gx[q].tiles_m = tM; gx[q].tiles_n = tN; gx[q].lower = 0;
+      gx[q].Xh = curH[q]; gx[q].Xl = curL[q];
+      gx[q].Yh = last ? nullptr : pl.Xh[nxt[q]];
+      gx[q].Yl = last ? nullptr : pl.Xl[nxt[q]];
+      gx[q].X32 = last ? cp[q].X32 : nullptr;
     }
-    ga.K = (int)N; ga.strideA = mn; ga.strideB = mn; ga.tiles_m = tM; ga.tiles_n = tM; ga.lower = 1;
+    const int tM0 = (int)(cp[0].M / BM), tN0 = (int)(cp[0].N / BN);
+    const unsigned g_sym = (unsigned)(cp[0].E * tM0 * (tM0 + 1) / 2), g_mn = (unsigned)(cp[0].E * tM0 * tN0);
     {
       AncProfScope prof(ANC_PROF_NS_GRAM, s);
-      if (big) { if (int rc = anc_ns_gemm_big(EPI_GRAM, ga, E, s)) return rc; }
-      else hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga);
+      if (big) { if (int rc = anc_ns_gemm_big_multi(EPI_GRAM, ga, Es, n, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga[0]);
     }
     ANC_LAUNCH_CHECK();
-    // B = b A + c A A
-    NsGemm gb = g;
-    gb.A[0] = pl.Fh; gb.B[0] = pl.Fh; gb.nterms = 1;
-    if (split_fb) {
-      gb.A[1] = pl.Fh; gb.B[1] = pl.Fl;
-      gb.A[2] = pl.Fl; gb.B[2] = pl.Fh;
-      gb.nterms = 3;
-    }
-    gb.K = (int)M; gb.strideA = M * M; gb.strideB = M * M; gb.tiles_m = tM; gb.tiles_n = tM; gb.lower = 1;
     {
       AncProfScope prof(ANC_PROF_NS_BMAT, s);
-      if (big) { if (int rc = anc_ns_gemm_big(EPI_BMAT, gb, E, s)) return rc; }
-      else hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb);
+      if (big) { if (int rc = anc_ns_gemm_big_multi(EPI_BMAT, gb, Es, n, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_BMAT>, dim3(g_sym), dim3(kGemmThreads), 0, s, gb[0]);
     }
     ANC_LAUNCH_CHECK();
-    // X = a X + B X
-    NsGemm gx = g;
-    gx.A[0] = pl.Bh; gx.B[0] = curH; gx.nterms = 1;
-    if (split) { gx.A[gx.nterms] = pl.Bh; gx.B[gx.nterms] = curL; ++gx.nterms; }
-    if (split_fb) { gx.A[gx.nterms] = pl.Bl; gx.B[gx.nterms] = curH; ++gx.nterms; }
-    gx.K = (int)M; gx.strideA = M * M; gx.strideB = mn; gx.tiles_m = tM; gx.tiles_n = tN; gx.lower = 0;
-    gx.Xh = curH; gx.Xl = curL;
-    gx.Yh = last ? nullptr : pl.Xh[nxt];
-    gx.Yl = last ? nullptr : pl.Xl[nxt];
-    gx.X32 = last ? X32 : nullptr;
     {
       AncProfScope prof(ANC_PROF_NS_BX, s);
-      if (big) { if (int rc = anc_ns_gemm_big(EPI_BX, gx, E, s)) return rc; }
-      else hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx);
+      if (big) { if (int rc = anc_ns_gemm_big_multi(EPI_BX, gx, Es, n, s)) return rc; }
+      else hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx[0]);
     }
     ANC_LAUNCH_CHECK();
-    curH = pl.Xh[nxt]; curL = pl.Xl[nxt];
-    nxt ^= 1;
+    for (int q = 0; q < n; ++q) {
+      curH[q] = cp[q].pl.Xh[nxt[q]]; curL[q] = cp[q].pl.Xl[nxt[q]];
+      nxt[q] ^= 1;
+    }
   }
   return ANC_OK;
 }
@@ -637,7 +657,8 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
   { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, mn, total8,
                      pl.Xh[0], pl.Xl[0]); }
   ANC_LAUNCH_CHECK();
-  return run_bf16_chain(pl, pl.Xh[0], pl.Xl[0], 1, nullptr, X32, E, M, N, steps, coef, force_small, s);
+  ChainProb cp{pl, pl.Xh[0], pl.Xl[0], 1, nullptr, X32, E, M, N};
+  return run_bf16_chain(&cp, 1, steps, coef, force_small, s);
 }
 
 // The chain on an unnormalised bf16 pair (what anc_muon_momentum_multi_pair leaves) with the
@@ -665,6 +686,49 @@ extern "C" int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partia
   { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s,
                      (const double *)fro_partials, (int)n_partials, eps, pl.recip); }
   ANC_LAUNCH_CHECK();
-  return run_bf16_chain(pl, (const uint16_t *)Uh, (const uint16_t *)Ul, 0, pl.recip, (float *)X32_out, E, M, N,
-                        steps, coef, force_small, s);
+  ChainProb cp{pl, (const uint16_t *)Uh, (const uint16_t *)Ul, 0, pl.recip, (float *)X32_out, E, M, N};
+  return run_bf16_chain(&cp, 1, steps, coef, force_small, s);
+}
+
+// n_probs <= 4 independent batches (the shape groups of one optimizer step) through the chain
+// side by side: each product of each step is one launch over all of them, which keeps the
+// CUs busy where per-batch launches would each end in a partly filled last wave. Same
+// results, bit for bit, as anc_ns_batched_pair on each batch. All dims multiples of 256.
+extern "C" int anc_ns_batched_pair_multi(const anc_ns_problem_t *probs, int32_t n_probs, int steps,
+                                         const float *coef, float eps, int mode, uint64_t stream) {
+  ANC_REQUIRE(probs != nullptr && n_probs >= 1 && n_probs <= kMaxGroups,
+              "anc_ns_batched_pair_multi: 1..%d problems", kMaxGroups);
+  ANC_REQUIRE(mode == ANC_NS_BF16 || mode == ANC_NS_BF16_FAST, "anc_ns_batched_pair_multi: bf16 modes only");
+  ANC_REQUIRE(steps >= 2 && steps <= 64 && coef != nullptr, "anc_ns_batched_pair_multi: steps=%d: 2..64", steps);
+  hipStream_t s = anc_stream(stream);
+  ChainProb cp[kMaxGroups];
+  int order[kMaxGroups];
+  for (int q = 0; q < n_probs; ++q) {
+    const anc_ns_problem_t &b = probs[q];
+    if (int rc = check_shape(b.E, b.M, b.N, mode, "anc_ns_batched_pair_multi")) return rc;
+    ANC_REQUIRE(b.M % 256 == 0 && b.N % 256 == 0, "anc_ns_batched_pair_multi: dims must be multiples of 256");
+    ANC_REQUIRE(b.Uh != 0 && b.Ul != 0 && ((b.Uh | b.Ul | b.X32_out) & 15) == 0 && b.X32_out != 0,
+                "anc_ns_batched_pair_multi: pointers must be 16-byte aligned and non-null");
+    ANC_REQUIRE(b.fro_partials != 0 && b.n_partials > 0 && b.n_partials < (1 << 30),
+                "anc_ns_batched_pair_multi: need the Frobenius partial sums");
+    ANC_REQUIRE(b.workspace != 0 && (b.workspace & 255) == 0, "anc_ns_batched_pair_multi: workspace must be 256-byte aligned");
+    order[q] = q;
+  }
+  // longest tiles first: by N (the Gram product's K), then by M
+  for (int a = 0; a < n_probs; ++a)
+    for (int c = a + 1; c < n_probs; ++c) {
+      const anc_ns_problem_t &x = probs[order[a]], &y = probs[order[c]];
+      if (y.N > x.N || (y.N == x.N && y.M > x.M)) { const int t = order[a]; order[a] = order[c]; order[c] = t; }
+    }
+  for (int q = 0; q < n_probs; ++q) {
+    const anc_ns_problem_t &b = probs[order[q]];
+    const Plan pl = make_plan(b.workspace, b.E, b.M, b.N, mode, steps);
+    ANC_REQUIRE(b.workspace_bytes >= pl.bytes, "anc_ns_batched_pair_multi: workspace holds %lld bytes, %lld needed",
+                (long long)b.workspace_bytes, (long long)pl.bytes);
+    { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)b.E), dim3(kThreads), 0, s,
+                       (const double *)b.fro_partials, (int)b.n_partials, eps, pl.recip); }
+    ANC_LAUNCH_CHECK();
+    cp[q] = ChainProb{pl, (const uint16_t *)b.Uh, (const uint16_t *)b.Ul, 0, pl.recip, (float *)b.X32_out, b.E, b.M, b.N};
+  }
+  return run_bf16_chain(cp, n_probs, steps, coef, false, s);
 }

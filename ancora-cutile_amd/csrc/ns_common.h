@@ -75,6 +75,41 @@ struct NsGemm {
 };
 
 
+// Up to 4 independent problems of the same kind (the same product of different shape groups)
+// in one launch: tiles[k] workgroups belong to problem k. One launch over all groups keeps the
+// CUs busy where separate launches would each end in a partly filled last wave.
+constexpr int kMaxGroups = 4;
+struct NsGemmMulti {
+  int n;
+  int tiles[kMaxGroups];
+  NsGemm g[kMaxGroups];
+};
+
+// Workgroup id -> (problem, tile index inside the problem). The logical tile sequence is cut
+// into 8 segments, one per XCD (xcd_remap hands XCD x a contiguous range that coincides with
+// segment x up to a few tiles); segment x holds the x-th eighth of every problem's tiles,
+// problems in the order given (longest tiles first), so that every XCD gets the same mix and a
+// problem's consecutive tiles -- the tiles of one matrix -- stay on one XCD.
+__device__ __forceinline__ void anc_group_tile(const NsGemmMulti &pm, int bid, int grid, int &g, int &L) {
+  int pos = xcd_remap(bid, grid);
+  g = 0;
+  L = pos;
+  if (pm.n == 1) return;
+  for (int x = 0; x < kXcds; ++x)
+    for (int k = 0; k < pm.n; ++k) {
+      const int T = pm.tiles[k], base = T / kXcds, rem = T % kXcds;
+      const int c = base + (x < rem ? 1 : 0);
+      if (pos < c) {
+        g = k;
+        L = x * base + (x < rem ? x : rem) + pos;
+        return;
+      }
+      pos -= c;
+    }
+}
+
 // 256x256-tile kernel (ns_gemm_big.hip): same products, same accumulation order and
 // therefore the same bits as the 128x128 kernel; used when M and N are multiples of 256.
 int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s);
+// The same for n <= kMaxGroups problems in one launch (ps[k] with batch size Es[k]).
+int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s);

@@ -185,7 +185,7 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS>
-__global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemm p) {
+__global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemmMulti pm) {
   constexpr int NWN = TN / 64, NWAVES = (TM / 128) * NWN;
   constexpr int ROWB = TK * 2;                      // bytes per LDS row
   constexpr int CPR = TK / 8;                       // 16-byte chunks per row
@@ -212,7 +212,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #ifdef ANC_DBG_TRACE
   const unsigned long long dbg_t0 = wall_clock64();
 #endif
-  const int L = xcd_remap((int)blockIdx.x, (int)gridDim.x);
+  int gsel, L;
+  anc_group_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
+  const NsGemm &p = pm.g[gsel];
   // Symmetric outputs: only tiles that reach the diagonal or lie below it. Row tm of TM-row
   // tiles has tm/R + 1 of them (R = TN/TM); a tile entirely below the diagonal is mirrored.
   constexpr int R = TN / TM;
@@ -571,32 +573,54 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 }
 
 template <int EPI>
-int launch_sym(const NsGemm &p, int64_t E, hipStream_t s) {
-  NsGemm q = p;
-  q.tiles_m = q.tiles_n = p.M / 256;
-  const int64_t grid = E * ((int64_t)q.tiles_m * (q.tiles_m + 1) / 2);
-  ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
-  hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 32, 4, 1>), dim3((unsigned)grid), dim3(512), 0, s, q);
+int launch_sym(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
+  NsGemmMulti pm{};
+  pm.n = n;
+  int64_t grid = 0;
+  for (int k = 0; k < n; ++k) {
+    pm.g[k] = ps[k];
+    pm.g[k].tiles_m = pm.g[k].tiles_n = ps[k].M / 256;
+    const int64_t t = Es[k] * ((int64_t)pm.g[k].tiles_m * (pm.g[k].tiles_m + 1) / 2);
+    ANC_REQUIRE(t > 0 && t < (1ll << 30), "anc_ns_gemm_big: grid out of range");
+    pm.tiles[k] = (int)t;
+    grid += t;
+  }
+  ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
+  hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 32, 4, 1>), dim3((unsigned)grid), dim3(512), 0, s, pm);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
 
 }  // namespace
 
-// Symmetric products run on 256x256 tiles (p.tiles_m = p.tiles_n = M/256, lower triangle);
-// X = a X + B X runs on 128x256 tiles (the tile counts of p are recomputed here).
-int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
-  ANC_REQUIRE(p.M % 256 == 0 && p.N % 256 == 0 && p.K % 32 == 0,
-              "anc_ns_gemm_big: dims must be multiples of 256");
-  if (epi == EPI_GRAM) return launch_sym<EPI_GRAM>(p, E, s);
-  if (epi == EPI_BMAT) return launch_sym<EPI_BMAT>(p, E, s);
-  NsGemm q = p;
-  q.tiles_m = p.M / 128;
-  q.tiles_n = p.N / 256;
-  q.lower = 0;
-  const int64_t grid = E * (int64_t)q.tiles_m * q.tiles_n;
-  ANC_REQUIRE(grid > 0 && grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
-  hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, q);
+// Symmetric products run on 256x256 tiles (lower triangle); X = a X + B X runs on 128x256 tiles
+// (the tile counts of the problems are recomputed here).
+int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
+  ANC_REQUIRE(n >= 1 && n <= kMaxGroups, "anc_ns_gemm_big: 1..%d problems per launch", kMaxGroups);
+  for (int k = 0; k < n; ++k)
+    ANC_REQUIRE(ps[k].M % 256 == 0 && ps[k].N % 256 == 0 && ps[k].K % 32 == 0,
+                "anc_ns_gemm_big: dims must be multiples of 256");
+  if (epi == EPI_GRAM) return launch_sym<EPI_GRAM>(ps, Es, n, s);
+  if (epi == EPI_BMAT) return launch_sym<EPI_BMAT>(ps, Es, n, s);
+  NsGemmMulti pm{};
+  pm.n = n;
+  int64_t grid = 0;
+  for (int k = 0; k < n; ++k) {
+    pm.g[k] = ps[k];
+    pm.g[k].tiles_m = ps[k].M / 128;
+    pm.g[k].tiles_n = ps[k].N / 256;
+    pm.g[k].lower = 0;
+    const int64_t t = Es[k] * (int64_t)pm.g[k].tiles_m * pm.g[k].tiles_n;
+    ANC_REQUIRE(t > 0 && t < (1ll << 30), "anc_ns_gemm_big: grid out of range");
+    pm.tiles[k] = (int)t;
+    grid += t;
+  }
+  ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
+  hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
+}
+
+int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
+  return anc_ns_gemm_big_multi(epi, &p, &E, 1, s);
 }

@@ -109,6 +109,11 @@ class MuonEngine:
         # norm and scaling passes over the batch do not exist. Needs a bf16 mode and >= 2 steps
         # (the fp32 result overlays the pair); otherwise the fp32 hand-off is used.
         self.fused_prologue = mode != "fp32" and self.ns >= 2
+        # Grouped launches: the chains of up to 4 shape groups advance together, each product of
+        # each Newton-Schulz step being one launch over all of them (no partly filled last wave
+        # of workgroups per group). Needs the fused prologue, private buffers per batch and
+        # dims that are multiples of 256; other batches run one by one.
+        self.grouped = True
         groups = {}
         scales = []
         for idx, w in enumerate(weights):
@@ -140,6 +145,7 @@ class MuonEngine:
         self.concurrent = bool(concurrent) and self._own_ws and len(self.batches) > 1
         self.serial = False          # True: keep the private buffers but launch everything on `si`
         self._forked = False
+        self._n_forked = 0
         self._streams, self._fork, self._join = [], None, []
         if self.concurrent:
             for b in self.batches:
@@ -178,10 +184,18 @@ class MuonEngine:
         lr_scales = (ctypes.c_float * MUON_MAX_SCALES)(*[lr * s for s in self.scales])
         seed_base = ((self.seed + 1000003 * self.t) & 0xFFFFFFFF) if self.sr else 0
         coef = muon_ns.coef_array(schedule, self.ns)
-        forked = self.concurrent and not self.serial
+        together = [b for b in self.batches
+                    if self.grouped and self.fused_prologue and self.concurrent
+                    and b.M % 256 == 0 and b.Nn % 256 == 0]
+        if len(together) < 2:
+            together = []
+        alone = [b for b in self.batches if b not in together]
+        for i0 in range(0, len(together), 4):
+            self._step_grouped(together[i0:i0 + 4], si, ctl, coef, lr_scales, seed_base)
+        forked = self.concurrent and not self.serial and len(alone) > 1
         if forked:
             self._fork.record(si)
-        for i, b in enumerate(self.batches):
+        for i, b in enumerate(alone):
             st = si
             if forked:
                 st = self._streams[i % len(self._streams)]
@@ -190,12 +204,8 @@ class MuonEngine:
             b.build(b.U, self.scale_index)
             buf = b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self.mode))
             if self.fused_prologue:
-                if b.fro is None:
-                    b.fro = DevBuf.empty((b.total_blocks,), np.float64)
+                self._momentum_pair(b, ctl, st)
                 n_el = b.E * b.M * b.Nn
-                api.anc_muon_momentum_multi_pair(b.table.ptr, b.E, b.total_blocks, self.mom,
-                                                 int(self.nesterov), b.U.ptr, n_el * 2, b.fro.ptr,
-                                                 ctl, int(st))
                 api.anc_ns_batched_pair(b.U.ptr, b.U.ptr + n_el * 2, b.fro.ptr,
                                         b.total_blocks // b.E, b.U.ptr, b.E, b.M, b.Nn, self.ns, coef,
                                         1e-7, muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(st))
@@ -209,13 +219,35 @@ class MuonEngine:
             if forked:
                 self._join[i].record(st)
         self._forked = forked
+        self._n_forked = len(alone) if forked else 0
         if forked and not defer_join:
             self.join(si)
+
+    def _momentum_pair(self, b, ctl, st):
+        if b.fro is None:
+            b.fro = DevBuf.empty((b.total_blocks,), np.float64)
+        api.anc_muon_momentum_multi_pair(b.table.ptr, b.E, b.total_blocks, self.mom, int(self.nesterov),
+                                         b.U.ptr, b.E * b.M * b.Nn * 2, b.fro.ptr, ctl, int(st))
+
+    def _step_grouped(self, group, si, ctl, coef, lr_scales, seed_base):
+        probs = (_lib.NsProblem * len(group))()
+        for k, b in enumerate(group):
+            b.build(b.U, self.scale_index)
+            buf = b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self.mode))
+            self._momentum_pair(b, ctl, si)
+            n_el = b.E * b.M * b.Nn
+            probs[k] = _lib.NsProblem(b.U.ptr, b.U.ptr + n_el * 2, b.fro.ptr, b.U.ptr, buf.ptr,
+                                      b.total_blocks // b.E, b.E, b.M, b.Nn, buf.nbytes)
+        api.anc_ns_batched_pair_multi(probs, len(group), self.ns, coef, 1e-7, muon_ns.MODES[self.mode],
+                                      int(si))
+        for b in group:
+            api.anc_muon_update_multi(b.table.ptr, b.E, b.total_blocks, lr_scales, F32,
+                                      int(self.sr), seed_base, ctl, int(si))
 
     def join(self, si):
         """Make stream `si` wait for the per-batch streams of the last step."""
         if self._forked:
-            for ev in self._join:
+            for ev in self._join[:self._n_forked]:
                 ev.wait_on(si)
 
     def unstep(self):

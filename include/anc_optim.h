@@ -331,6 +331,22 @@ int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partials, int64_t
                         int steps, const float *coef, float eps, int mode,
                         uint64_t workspace, int64_t workspace_bytes, uint64_t stream);
 
+/* Several batches (the shape groups of one optimizer step) through anc_ns_batched_pair side
+ * by side: each of the three products of each step is ONE launch over all batches, so the
+ * CUs stay busy where per-batch launches would each end in a partly filled last wave of
+ * workgroups. No reference counterpart (the reference runs its shape groups one after the
+ * other, ancora/optim/muon.py:257-277). Results equal anc_ns_batched_pair on each batch bit
+ * for bit. n_probs <= 4; every M and N a multiple of 256; steps >= 2; bf16 modes. */
+typedef struct {
+  uint64_t Uh, Ul;            /* input bf16 pair, (E,M,N) each                        */
+  uint64_t fro_partials;      /* n_partials sums of u*u per matrix                     */
+  uint64_t X32_out;           /* fp32 result (may overlay the pair)                    */
+  uint64_t workspace;         /* anc_ns_workspace_bytes(E,M,N,mode) bytes of its own   */
+  int64_t  n_partials, E, M, N, workspace_bytes;
+} anc_ns_problem_t;
+int anc_ns_batched_pair_multi(const anc_ns_problem_t *probs, int32_t n_probs, int steps,
+                              const float *coef, float eps, int mode, uint64_t stream);
+
 /* Matrix-core FLOPs of one anc_ns_batched call: `executed` counts the tiles and terms the
  * kernels really multiply (lower-triangle tiles of the symmetric products, residual terms),
  * `dense` is steps*(4 M^2 N + 2 M^3) per matrix. Roofline figures use `executed`. */

@@ -178,3 +178,41 @@ def test_pair_entry_folds_the_normalisation(gpu, M, N, mode):
         assert rel_fro(got[e], host_ns(X[e], PE_SCHEDULE, 5)) < tol
         assert rel_fro(got[e], ref[e]) < 3e-3
     U.free(); fro.free()
+
+
+def test_grouped_launch_equals_per_batch_bits(gpu):
+    """anc_ns_batched_pair_multi (one launch per product over several shape groups) gives each
+    batch the bits of anc_ns_batched_pair on that batch alone; batch order does not matter."""
+    from ancora_cutile_amd import DevBuf, _lib
+    from ancora_cutile_amd._lib import api
+    from ancora_cutile_amd.muon_ns import ns_batched_pair, ns_workspace_bytes, coef_array, MODES
+    rng = np.random.default_rng(11)
+    shapes = [(3, 256, 256), (2, 256, 768), (5, 512, 512)]
+    host, alone = [], []
+    for (E, M, N) in shapes:
+        X = (0.01 * rng.standard_normal((E, M, N))).astype(np.float32)
+        hi = bf16_rne_bits(X).reshape(E, M, N)
+        lo = bf16_rne_bits(X - bits_to_f32(hi).reshape(E, M, N)).reshape(E, M, N)
+        pair = np.concatenate([hi.reshape(-1), lo.reshape(-1)]).view(np.float32)
+        parts = np.ascontiguousarray((X.astype(np.float64) ** 2).reshape(E, 2, -1).sum(axis=2))
+        host.append((pair, parts))
+        U, fro = DevBuf(pair), DevBuf(parts)
+        ns_batched_pair(U, fro, 2, E, M, N, 0, steps=5, schedule=PE_SCHEDULE, mode="bf16")
+        alone.append(U.to_numpy())
+        U.free(); fro.free()
+    for order in ([0, 1, 2], [2, 0, 1]):
+        bufs, probs = [], (_lib.NsProblem * 3)()
+        for k, q in enumerate(order):
+            E, M, N = shapes[q]
+            U, fro = DevBuf(host[q][0]), DevBuf(host[q][1])
+            nb = ns_workspace_bytes(E, M, N, "bf16")
+            ws = DevBuf.empty((nb // 4 + 64,), np.float32)
+            wptr = (ws.ptr + 255) // 256 * 256
+            probs[k] = _lib.NsProblem(U.ptr, U.ptr + E * M * N * 2, fro.ptr, U.ptr, wptr, 2, E, M, N, nb)
+            bufs.append((U, fro, ws))
+        api.anc_ns_batched_pair_multi(probs, 3, 5, coef_array(PE_SCHEDULE, 5), 1e-7, MODES["bf16"], 0)
+        for k, q in enumerate(order):
+            assert bits_equal(bufs[k][0].to_numpy(), alone[q])
+        for t in bufs:
+            for b in t:
+                b.free()
