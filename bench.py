@@ -349,7 +349,7 @@ def main():
         "ns_mfma_util_pct": round(100 * achieved / PEAK_BF16_TFLOPS, 2),
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kind_ms.items()},
         "event_ms_per_step": round(ev_ms, 3), "wall_ms_per_step": round(wall_ms, 3),
-        "streams": "serial" if args.serial else "one per Newton-Schulz shape group",
+        "streams": "serial" if args.serial else "one: the Newton-Schulz chains of all shape groups advance together (grouped launches)",
         "copy_kernel_gbps": round(copy_gbps, 1),
         "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
         "device": {"name": info["name"], "arch": info["arch"], "cus": info["cu_count"],
