@@ -206,8 +206,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   auto st = [&](int i) -> unsigned char * {
     return i == 0 ? stage0 : i == 1 ? stage1 : i == 2 ? stage2 : stage3;
   };
-  // B = b A + c A A: per-wavefront copy of the dA entries of its 128 rows and 64 columns
-  __shared__ __attribute__((aligned(1024))) unsigned char aux[EPI == EPI_BMAT ? NWAVES * 1024 : 16];
+  // B = b A + c A A: per-wavefront copy of the dA entries of its 128 rows and 64 columns;
+  // X = a X + B X: of the dB entries of its 128 rows
+  __shared__ __attribute__((aligned(1024))) unsigned char aux[EPI != EPI_GRAM ? NWAVES * 1024 : 16];
 
 #ifdef ANC_DBG_TRACE
   const unsigned long long dbg_t0 = wall_clock64();
@@ -376,8 +377,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // 4 apart, then use different banks. The same buffer stages the slab's bf16 outputs.
   constexpr int kInBuf = 8192, kBufPerStage = kStage / kInBuf;
   static_assert(EPI != EPI_BMAT || kBufPerStage * NS >= 2 * NWAVES, "epilogue buffers");
-  static_assert(EPI != EPI_BX || (kBufPerStage * NS >= 2 * NWAVES + 1 && kInBuf >= kStageRegion &&
-                                  NWAVES * 1024 <= kInBuf && TM == 128), "epilogue buffers");
+  static_assert(EPI != EPI_BX || (kBufPerStage * NS >= 2 * NWAVES && kInBuf >= kStageRegion), "epilogue buffers");
   auto inbuf = [&](int bi) -> unsigned char * {
     const int q = wave * 2 + (bi & 1);
     return st(q / kBufPerStage) + (q % kBufPerStage) * kInBuf;
@@ -406,7 +406,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       dma16((const char *)p.A32 + ub + (int64_t)(4 * j) * M * 4 + ((j & 1) ? vo_a1 : vo_a0), lds_addr(b + j * 1024));
   };
   int in_lane[2] = {0, 0};
-  unsigned char *aux_w = aux + (EPI == EPI_BMAT ? wave * 1024 : 0);
+  unsigned char *aux_w = aux + (EPI != EPI_GRAM ? wave * 1024 : 0);
   if (EPI == EPI_BMAT) {
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj)
@@ -417,7 +417,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     fetch_a32(0);
     fetch_a32(1);
   }
-  unsigned char *dvec_lds = st((2 * NWAVES) / kBufPerStage) + ((2 * NWAVES) % kBufPerStage) * kInBuf + wave * 1024;
+  unsigned char *dvec_lds = aux_w;
   if (EPI == EPI_BX) {
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj)
