@@ -84,13 +84,20 @@ __device__ __forceinline__ void load_frags_bt(const unsigned char *st, int a_bas
     f.b[i] = anc_lds_tr_frag(st + tb[i] + kk * (16 * 512), st + tb[i] + kk * (16 * 512) + 4 * 512);
 }
 
+// SWAP = false: accumulator block (bi,bj) holds C[32 bi + row][32 bj + col] with col = lane%32
+// and element r = row 8*(r/4) + 4*(lane/32) + r%4. SWAP = true computes the transposed block
+// (operands exchanged, same products, same order of summation): row = lane%32 and element
+// r = col 8*(r/4) + 4*(lane/32) + r%4, i.e. a lane holds runs of 4 consecutive columns of one
+// output row, which is what a row-major epilogue wants.
+template <bool SWAP>
 __device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi)
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj)
 #ifndef ANC_DBG_NOMFMA
-      acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[bi], f.b[bj], acc[bi][bj], 0, 0, 0);
+      acc[bi][bj] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[bj], f.a[bi], acc[bi][bj], 0, 0, 0)
+                         : __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[bi], f.b[bj], acc[bi][bj], 0, 0, 0);
 #else
       acc[bi][bj][0] += (float)f.a[bi][0] + (float)f.b[bj][0];
 #endif
@@ -339,12 +346,12 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #pragma unroll
     for (int kk = 0; kk < KSTEPS - 1; ++kk) {
       frags(cur, kk + 1, f[(kk + 1) & 1]);
-      mfma8(f[kk & 1], acc);
+      mfma8<BT>(f[kk & 1], acc);
     }
     if (refill) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
     lds_barrier();
     if (more) frags(nxt, 0, f[0]);
-    mfma8(f[(KSTEPS - 1) & 1], acc);
+    mfma8<BT>(f[(KSTEPS - 1) & 1], acc);
   };
   for (int step = 0; step < total; step += NS) {
 #pragma unroll
@@ -373,8 +380,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // of each is 32 rows of 128 bytes: 4 DMA instructions (8 rows each, lane -> row lane/8, chunk
   // lane%8) put it into a buffer private to the wavefront, two slabs ahead of the arithmetic, so
   // that full cache lines are requested and the latency runs under the previous slabs. The
-  // 16-byte chunk index is XORed with 4*((row>>2)&1): the two half-wavefronts, which read rows
-  // 4 apart, then use different banks. The same buffer stages the slab's bf16 outputs.
+  // 16-byte chunk index is XORed with (row&7) ^ ((row>>3)&1) (see the epilogue). The same
+  // buffer stages the slab's outputs.
   constexpr int kInBuf = 8192, kBufPerStage = kStage / kInBuf;
   static_assert(EPI != EPI_BMAT || kBufPerStage * NS >= 2 * NWAVES, "epilogue buffers");
   static_assert(EPI != EPI_BX || (kBufPerStage * NS >= 2 * NWAVES && kInBuf >= kStageRegion), "epilogue buffers");
@@ -382,15 +389,17 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     const int q = wave * 2 + (bi & 1);
     return st(q / kBufPerStage) + (q % kBufPerStage) * kInBuf;
   };
-  const uint32_t vo_in = (uint32_t)((lane >> 3) * N * 2 + (((lane & 7) ^ ((lane >> 5) << 2)) * 16));
+  const uint32_t vo_in0 = (uint32_t)((lane >> 3) * N * 2 + (((lane & 7) ^ (lane >> 3)) * 16));
+  const uint32_t vo_in1 = (uint32_t)((lane >> 3) * N * 2 + (((lane & 7) ^ (lane >> 3) ^ 1) * 16));
   auto fetch_in = [&](int bi) {
     const int64_t ub = (mn + (int64_t)(gi0w + bi * 32) * N + gj0w) * 2;
     unsigned char *b = inbuf(bi);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int64_t ro = (int64_t)(8 * j) * N * 2;
-      dma16((const char *)p.Xh + ub + ro + vo_in, lds_addr(b + j * 1024));
-      dma16((const char *)p.Xl + ub + ro + vo_in, lds_addr(b + 4096 + j * 1024));
+      const uint32_t vo = (j & 1) ? vo_in1 : vo_in0;
+      dma16((const char *)p.Xh + ub + ro + vo, lds_addr(b + j * 1024));
+      dma16((const char *)p.Xl + ub + ro + vo, lds_addr(b + 4096 + j * 1024));
     }
   };
   // B = b A + c A A reads A32 at the output position the same way: a 32x64 fp32 slab is 32 rows
@@ -419,9 +428,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   }
   unsigned char *dvec_lds = aux_w;
   if (EPI == EPI_BX) {
-#pragma unroll
-    for (int bj = 0; bj < 2; ++bj)
-      in_lane[bj] = 4 * (lane >> 5) * 128 + (((bj * 4 + ((lane & 31) >> 3)) ^ ((lane >> 5) << 2)) * 16) + (lane & 7) * 2;
     asm volatile("" : "+v"(sc));      // the scale has arrived before the first DMA is issued
     // dB of the tile's 128 rows, one private copy per wavefront (lanes 32..63 repeat lanes 0..31),
     // fetched first: any ordinary load issued after the slab fetches would, completing in
@@ -429,6 +435,109 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     dma16((const char *)(p.dB + mv + gi0w) + (lane & 31) * 16, lds_addr(dvec_lds));
     fetch_in(0);
     fetch_in(1);
+  }
+  if (EPI == EPI_BX) {
+    // Transposed accumulator layout (see mfma8): lane l holds row l%32 of the slab and, per
+    // column block bj and q = 0..3, the 4 consecutive columns bj*32 + 8q + 4*(l/32) .. +3.
+    // Inputs (the bf16 pair) are 8-byte LDS reads, outputs 8-byte (pair) or 16-byte (fp32
+    // result) LDS writes into the slab's own buffer, which then leaves as whole rows.
+    // Pair layout in the buffer: [32 rows][8 chunks of 16 B], chunk index XORed with
+    // (row&7) ^ ((row>>3)&1): the 32 rows a read touches spread over all banks.
+    const int rr = lane & 31, hh = lane >> 5;
+    const int key = (rr & 7) ^ ((rr >> 3) & 1);
+    const bool fp32_out = p.X32 != nullptr;
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi) {
+      const int gi0 = gi0w + bi * 32;
+      // Wait for this slab's DMA only. Vector memory operations complete in issue order; after
+      // the fetch of slab bi this wavefront issued the 8 row stores of slab bi-1 and the fetch
+      // of slab bi+1 (8 DMA); nothing else in this epilogue is a vector memory operation.
+      if (bi == 0 || bi == 3) wait_vm<8>(); else wait_vm<16>();
+      unsigned char *b = inbuf(bi);
+      const float dr = *(const float *)(dvec_lds + (bi * 32 + rr) * 4);
+      anc_u32x2 xh[2][4], xl[2][4];
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int off = rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8;
+          xh[bj][q] = *(const anc_u32x2 *)(b + off);
+          xl[bj][q] = *(const anc_u32x2 *)(b + 4096 + off);
+        }
+      float y[2][16];
+      const float cf = p.ca + dr;
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const uint32_t wh = (r & 2) ? xh[bj][r >> 2].y : xh[bj][r >> 2].x;
+          const uint32_t wl = (r & 2) ? xl[bj][r >> 2].y : xl[bj][r >> 2].x;
+          const float x = ((r & 1) ? __uint_as_float(wh & 0xFFFF0000u) : __uint_as_float(wh << 16)) +
+                          ((r & 1) ? __uint_as_float(wl & 0xFFFF0000u) : __uint_as_float(wl << 16));
+          y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
+        }
+      if (fp32_out) {
+        // fp32 result: [32 rows][16 chunks of 16 B], chunk XOR (row & 15)
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const anc_f32x4 v4 = {y[bj][4 * q], y[bj][4 * q + 1], y[bj][4 * q + 2], y[bj][4 * q + 3]};
+            *(anc_f32x4 *)(b + rr * 256 + (((bj * 8 + 2 * q + hh) ^ (rr & 15)) * 16)) = v4;
+          }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int pz = 0; pz < 8; ++pz) {
+          const int idx = pz * 64 + lane, row = idx >> 4, c = idx & 15;
+          const anc_f32x4 v4 = *(const anc_f32x4 *)(b + row * 256 + ((c ^ (row & 15)) * 16));
+          anc_st_stream((anc_f32x4 *)(p.X32 + mn + (int64_t)(gi0 + row) * N + gj0w + c * 4), v4);
+        }
+      } else {
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            uint32_t h0, l0, h1, l1;
+            anc_pk_pair(y[bj][4 * q], y[bj][4 * q + 1], h0, l0);
+            anc_pk_pair(y[bj][4 * q + 2], y[bj][4 * q + 3], h1, l1);
+            const anc_u32x2 wh = {h0, h1}, wl = {l0, l1};
+            const int off = rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8;
+            *(anc_u32x2 *)(b + off) = wh;
+            *(anc_u32x2 *)(b + 4096 + off) = wl;
+          }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int pz = 0; pz < 4; ++pz) {
+          const int idx = pz * 64 + lane, row = idx >> 3, c = idx & 7;
+          const int off = row * 128 + ((c ^ ((row & 7) ^ ((row >> 3) & 1))) * 16);
+          const anc_u32x4 qh = *(const anc_u32x4 *)(b + off);
+          anc_st_stream((anc_u32x4 *)(p.Yh + mn + (int64_t)(gi0 + row) * N + gj0w + c * 8), qh);
+        }
+#pragma unroll
+        for (int pz = 0; pz < 4; ++pz) {
+          const int idx = pz * 64 + lane, row = idx >> 3, c = idx & 7;
+          const int off = row * 128 + ((c ^ ((row & 7) ^ ((row >> 3) & 1))) * 16);
+          const anc_u32x4 ql = *(const anc_u32x4 *)(b + 4096 + off);
+          anc_st_stream((anc_u32x4 *)(p.Yl + mn + (int64_t)(gi0 + row) * N + gj0w + c * 8), ql);
+        }
+      }
+      // the buffer is free again once the staged rows have been read back
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_wave_barrier();
+      asm volatile("" ::: "memory");
+      if (bi + 2 < 4) fetch_in(bi + 2);
+    }
+#ifdef ANC_DBG_TRACE
+    if (threadIdx.x == 0 && blockIdx.x < 16384) {
+      anc_dbg_ts[EPI][blockIdx.x][0] = dbg_t0;
+      anc_dbg_ts[EPI][blockIdx.x][1] = dbg_t1;
+      anc_dbg_ts[EPI][blockIdx.x][2] = wall_clock64();
+      anc_dbg_ts[EPI][blockIdx.x][3] = 0;
+    }
+#endif
+    return;
   }
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi) {
@@ -458,37 +567,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       for (int bj = 0; bj < 2; ++bj) dcol[bj] = *(const float *)(aux_w + 512 + (bj * 32 + (lane & 31)) * 4);
       region = const_cast<unsigned char *>(b);
     }
-    if (EPI == EPI_BX) {
-      // Wait for this slab's DMA only. Vector memory operations complete in issue order, and
-      // after the fetch of slab bi this wavefront issued: the fetch of slab bi+1 (8 DMA, at the
-      // end of slab bi-1, or up front for slab 1) and before it the stores of slab bi-1 (32
-      // dword stores of the fp32 result on the last step, else 2 x 4 stores of the pair).
-      // Nothing else in this epilogue is a vector memory operation.
-      const bool fp32_out = p.X32 != nullptr;
-      if (bi == 0) wait_vm<8>();
-      else if (bi == 3) { if (fp32_out) wait_vm<32>(); else wait_vm<8>(); }
-      else { if (fp32_out) wait_vm<40>(); else wait_vm<16>(); }
-      // X = Xh + Xl is exact in fp32 (8 + 8 significant bits)
-      const unsigned char *b = inbuf(bi);
-#pragma unroll
-      for (int bj = 0; bj < 2; ++bj)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int ro = (8 * (r >> 2) + (r & 3)) * 128;
-          const uint16_t xh = *(const uint16_t *)(b + in_lane[bj] + ro);
-          const uint16_t xl = *(const uint16_t *)(b + 4096 + in_lane[bj] + ro);
-          in[bj][r] = (anc_bf16_bits_to_f32(xh) + anc_bf16_bits_to_f32(xl)) * sc;
-        }
-      region = const_cast<unsigned char *>(b);
-    }
-    if (EPI == EPI_BX) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const anc_f32x4 d4 = *(const anc_f32x4 *)(dvec_lds + (bi * 32 + 8 * q + 4 * (lane >> 5)) * 4);
-        drow[4 * q] = d4.x; drow[4 * q + 1] = d4.y; drow[4 * q + 2] = d4.z; drow[4 * q + 3] = d4.w;
-      }
-    }
-
     float ov[2][16];          // the values that leave as bf16 (pairs)
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj) {
@@ -517,10 +595,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
             p.dB[mv + gi] = p.cb * di + p.cc * a2;
             ov[bj][r] = 0.0f;
           }
-        } else {
-          const float y = (p.ca + drow[r]) * in[bj][r] + v;
-          if (p.X32 != nullptr) anc_st_stream(p.X32 + mn + (int64_t)gi * N + gj, y);
-          ov[bj][r] = y;
         }
       }
     }
@@ -546,16 +620,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       __builtin_amdgcn_s_waitcnt(0xC07F);
       asm volatile("" ::: "memory");
       if (bi + 2 < 4) fetch_a32(bi + 2);
-    } else {
-      if (p.Yh != nullptr) {
-        stage_rows(region, hv, lane, p.Yh + mn + (int64_t)gi0 * N + gj0w, N);
-        stage_rows(region, lv, lane, p.Yl + mn + (int64_t)gi0 * N + gj0w, N);
-      }
-      // this slab's buffer is free again (its inputs are in registers, its staged outputs
-      // were read back before stage_rows returned): fetch the slab after the next into it
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      asm volatile("" ::: "memory");
-      if (bi + 2 < 4) fetch_in(bi + 2);
     }
   }
 #ifdef ANC_DBG_TRACE
