@@ -274,11 +274,21 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const uint32_t voffB1 = (uint32_t)((lane >> 5) * ldn * 2 + (((lane & 31) ^ ((2 + (lane >> 5)) << 2)) * 16));
   const int64_t ubaseBT = ((int64_t)e * p.strideB + (int64_t)tn * TN + (int64_t)(wave * IB * 2) * ldn) * 2;
 
-  auto issue = [&](int step, unsigned char *stage) {
-    const int term = step / nk, kt = step - term * nk;
-    const char *Ag = (const char *)p.A[term] + ubaseA + (int64_t)kt * ROWB;
-    const char *Bg = BT ? (const char *)p.B[term] + ubaseBT + (int64_t)kt * TK * ldn * 2
-                        : (const char *)p.B[term] + ubaseB + (int64_t)kt * ROWB;
+  // Operand pointers of the three terms are fetched from the argument block once, here: a
+  // scalar load inside the K loop would have to be waited for with lgkmcnt(0), which also
+  // waits for the LDS fragment reads in flight. K tiles are issued strictly in order, so the
+  // running pointers just advance.
+  const char *Abase[3], *Bbase[3];
+#pragma unroll
+  for (int t3 = 0; t3 < 3; ++t3) {
+    Abase[t3] = (const char *)p.A[t3] + ubaseA;
+    Bbase[t3] = (const char *)p.B[t3] + (BT ? ubaseBT : ubaseB);
+  }
+  const int64_t advB = BT ? (int64_t)TK * ldn * 2 : (int64_t)ROWB;
+  const char *curA = Abase[0], *curB = Bbase[0];
+  int is_kt = 0, is_term = 0;
+  auto issue = [&](unsigned char *stage) {
+    const char *Ag = curA, *Bg = curB;
 #pragma unroll
     for (int i = 0; i < IA; ++i) {
       const int64_t ro = (int64_t)(i * RPI) * K * 2;
@@ -290,6 +300,14 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       const int64_t ro = BT ? (int64_t)(i * 2) * ldn * 2 : (int64_t)(i * RPI) * K * 2;
       const uint32_t vo = BT ? ((i & 1) ? voffB1 : voffB0) : ((i & 1) ? voff1 : voff0);
       dma16(Bg + ro + vo, lds_addr(stage + TM * ROWB + (wave * IB + i) * 1024));
+    }
+    curA += ROWB;
+    curB += advB;
+    if (++is_kt == nk) {
+      is_kt = 0;
+      ++is_term;
+      curA = is_term == 1 ? Abase[1] : Abase[2];
+      curB = is_term == 1 ? Bbase[1] : Bbase[2];
     }
   };
 
@@ -331,7 +349,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   Frags f[2];
 #pragma unroll
   for (int s0 = 0; s0 < NS - 1; ++s0)
-    if (s0 < total) issue(s0, st(s0));
+    if (s0 < total) issue(st(s0));
   if (total >= NS - 1) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
   lds_barrier();
   frags(stage0, 0, f[0]);
@@ -341,7 +359,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     const bool more = step + 1 < total;
     const bool refill = step + NS - 1 < total;
 #ifndef ANC_DBG_NODMA
-    if (refill) issue(step + NS - 1, fill);
+    if (refill) issue(fill);
 #endif
 #pragma unroll
     for (int kk = 0; kk < KSTEPS - 1; ++kk) {
