@@ -90,6 +90,16 @@ __device__ __forceinline__ void load_frags_bt(const unsigned char *st, int a_bas
 // r = col 8*(r/4) + 4*(lane/32) + r%4, i.e. a lane holds runs of 4 consecutive columns of one
 // output row, which is what a row-major epilogue wants.
 template <bool SWAP>
+__device__ __forceinline__ void mfma1(const Frags &f, f32x16 (&acc)[4][2], int idx) {
+  const int bi = idx >> 1, bj = idx & 1;
+#ifndef ANC_DBG_NOMFMA
+  acc[bi][bj] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[bj], f.a[bi], acc[bi][bj], 0, 0, 0)
+                     : __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[bi], f.b[bj], acc[bi][bj], 0, 0, 0);
+#else
+  acc[bi][bj][0] += (float)f.a[bi][0] + (float)f.b[bj][0];
+#endif
+}
+template <bool SWAP>
 __device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi)
@@ -287,20 +297,20 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const int64_t advB = BT ? (int64_t)TK * ldn * 2 : (int64_t)ROWB;
   const char *curA = Abase[0], *curB = Bbase[0];
   int is_kt = 0, is_term = 0;
-  auto issue = [&](unsigned char *stage) {
-    const char *Ag = curA, *Bg = curB;
-#pragma unroll
-    for (int i = 0; i < IA; ++i) {
+  // DMA instruction i of a stage (0 .. IPS-1: the A tile's IA, then the B tile's IB)
+  auto issue_piece = [&](int i, unsigned char *stage) {
+    if (i < IA) {
       const int64_t ro = (int64_t)(i * RPI) * K * 2;
       const uint32_t vo = (i & 1) ? voff1 : voff0;
-      dma16(Ag + ro + vo, lds_addr(stage + (wave * IA + i) * 1024));
+      dma16(curA + ro + vo, lds_addr(stage + (wave * IA + i) * 1024));
+    } else {
+      const int j = i - IA;
+      const int64_t ro = BT ? (int64_t)(j * 2) * ldn * 2 : (int64_t)(j * RPI) * K * 2;
+      const uint32_t vo = BT ? ((j & 1) ? voffB1 : voffB0) : ((j & 1) ? voff1 : voff0);
+      dma16(curB + ro + vo, lds_addr(stage + TM * ROWB + (wave * IB + j) * 1024));
     }
-#pragma unroll
-    for (int i = 0; i < IB; ++i) {
-      const int64_t ro = BT ? (int64_t)(i * 2) * ldn * 2 : (int64_t)(i * RPI) * K * 2;
-      const uint32_t vo = BT ? ((i & 1) ? voffB1 : voffB0) : ((i & 1) ? voff1 : voff0);
-      dma16(Bg + ro + vo, lds_addr(stage + TM * ROWB + (wave * IB + i) * 1024));
-    }
+  };
+  auto issue_advance = [&]() {
     curA += ROWB;
     curB += advB;
     if (++is_kt == nk) {
@@ -309,6 +319,11 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       curA = is_term == 1 ? Abase[1] : Abase[2];
       curB = is_term == 1 ? Bbase[1] : Bbase[2];
     }
+  };
+  auto issue = [&](unsigned char *stage) {
+#pragma unroll
+    for (int i = 0; i < IPS; ++i) issue_piece(i, stage);
+    issue_advance();
   };
 
   // ---- fragment addressing
@@ -346,7 +361,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // barrier inside tile k-1). Before the last k-step of tile k each wavefront waits until its
   // own DMA of tile k+1 has landed (NS-2 younger tiles may still be in flight), all
   // wavefronts synchronise, and the first fragments of tile k+1 load under the last MFMAs.
-  Frags f[2];
+Frags f[2];
 #pragma unroll
   for (int s0 = 0; s0 < NS - 1; ++s0)
     if (s0 < total) issue(st(s0));
@@ -359,12 +374,33 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     const bool more = step + 1 < total;
     const bool refill = step + NS - 1 < total;
 #ifndef ANC_DBG_NODMA
-    if (refill) issue(fill);
+    if (KSTEPS == 2) {
+      // The stage's DMA instructions go out between the MFMAs of the first k-step, one every
+      // 8/IPS matrix instructions, instead of as a burst during which the matrix pipe idles.
+      frags(cur, 1, f[1]);
+#pragma unroll
+      for (int idx = 0; idx < 8; ++idx) {
+        mfma1<BT>(f[0], acc, idx);
+#pragma unroll
+        for (int i = 0; i < IPS; ++i)
+          if (((i + 1) * 8 + IPS - 1) / IPS - 1 == idx) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (refill) issue_piece(i, fill);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+      }
+      if (refill) issue_advance();
+    } else
+#endif
+    {
+#ifndef ANC_DBG_NODMA
+      if (refill) issue(fill);
 #endif
 #pragma unroll
-    for (int kk = 0; kk < KSTEPS - 1; ++kk) {
-      frags(cur, kk + 1, f[(kk + 1) & 1]);
-      mfma8<BT>(f[kk & 1], acc);
+      for (int kk = 0; kk < KSTEPS - 1; ++kk) {
+        frags(cur, kk + 1, f[(kk + 1) & 1]);
+        mfma8<BT>(f[kk & 1], acc);
+      }
     }
     if (refill) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
     lds_barrier();

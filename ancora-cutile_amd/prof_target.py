@@ -6,6 +6,8 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
                                       per-launch event timer and prints ms per kernel kind)
     python3 -m ancora_cutile_amd.prof_target adamw NUMEL [calls]         fused AdamW, bf16 grads, SR
     python3 -m ancora_cutile_amd.prof_target gradnorm NUMEL [calls]      grad-norm partials + finalize
+    python3 -m ancora_cutile_amd.prof_target mfmamix                    matrix-instruction rate next to
+                                      unrelated LDS / LDS-DMA traffic (anc_probe_mfma_mix), a table
 
 Each target allocates its operands, runs the kernel(s) `calls` times on the null stream and
 synchronises; nothing is checked here (parity lives in tests/).
@@ -56,6 +58,19 @@ def main(argv):
         guard = StepGuard(1.0)
         for _ in range(calls):
             guard.compute([g], 0)
+    elif what == "mfmamix":
+        src = DevBuf.zeros((1 << 28,), np.float32)          # 1 GiB
+        sink = DevBuf.zeros((512,), np.float32)
+        print("16 MFMA per wavefront-iteration, 8 wavefronts per CU, 256 CUs")
+        tf, cyc = ctypes.c_double(0), ctypes.c_double(0)
+        _lib.api.anc_probe_mfma_mix(0, 0, 0, 100000, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf),
+                                    ctypes.byref(cyc))                     # clocks settle; discarded
+        for nread, ndma, hbm in ((0, 0, 0), (12, 0, 0), (0, 4, 0), (12, 4, 0), (24, 8, 0), (12, 4, 1),
+                                 (0, 0, 0)):
+            _lib.api.anc_probe_mfma_mix(nread, ndma, hbm, 50000, src.ptr, src.nbytes, sink.ptr,
+                                        ctypes.byref(tf), ctypes.byref(cyc))
+            print(f"  + {nread:2d} ds_read_b128 + {ndma} LDS-DMA KiB ({'HBM stream' if hbm else 'L2 resident'}): "
+                  f"{tf.value:7.1f} TFLOP/s = {tf.value / 25:.1f} % of 2.5 PFLOP/s")
     else:
         raise SystemExit(__doc__)
     _lib.api.anc_device_sync()

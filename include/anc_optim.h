@@ -353,6 +353,16 @@ int anc_ns_batched_pair_multi(const anc_ns_problem_t *probs, int32_t n_probs, in
 int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
                  double *executed, double *dense);
 
+/* Diagnostics, no reference counterpart: rate of the bf16 matrix instruction on register
+ * operands while the same wavefronts issue `nread` LDS fragment reads and `ndma` LDS-DMA loads
+ * of 1 KiB per 16 matrix instructions that nothing depends on (the proportions of the
+ * Newton-Schulz GEMM's K loop are 12 and 4), from an L2-resident source or, with hbm != 0,
+ * streaming through `span_bytes` of HBM. (nread, ndma) one of (0,0) (12,0) (0,4) (12,4)
+ * (24,8). `cycles_per_iter` is scaled so that the matrix instructions alone take 1024. */
+int anc_probe_mfma_mix(int nread, int ndma, int hbm, int iters, uint64_t src,
+                       int64_t span_bytes, uint64_t sink, double *tflops,
+                       double *cycles_per_iter);
+
 /* fp32 <-> bf16 conversion of packed batches (entry/exit of the bf16-typed
  * reference drivers): dst_f32 = float(src_bf16); dst_bf16 = RNE(src_f32). */
 int anc_bf16_to_f32(uint64_t src, uint64_t dst, int64_t n, uint64_t stream);
