@@ -361,7 +361,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // barrier inside tile k-1). Before the last k-step of tile k each wavefront waits until its
   // own DMA of tile k+1 has landed (NS-2 younger tiles may still be in flight), all
   // wavefronts synchronise, and the first fragments of tile k+1 load under the last MFMAs.
-Frags f[2];
+  Frags f[2];
 #pragma unroll
   for (int s0 = 0; s0 < NS - 1; ++s0)
     if (s0 < total) issue(st(s0));
