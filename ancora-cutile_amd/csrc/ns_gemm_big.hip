@@ -22,17 +22,21 @@
 // (ds_read_b64_tr_b16), so no transposed copy of the iterate exists anywhere.
 //
 // Stage ring. Tile k of the K loop lives in stage k % NS, each stage a __shared__ array of its
-// own. The DMA of tile k+NS-1 starts at the top of tile k; before the last k-step of tile k a
-// wavefront waits (s_waitcnt vmcnt) only for its own DMA of tile k+1, then the workgroup
-// synchronises with a barrier that orders LDS traffic only. The DMA instructions and these
+// own. The DMA instructions of tile k+NS-1 go out between the MFMAs of tile k's first k-step;
+// before the last k-step of tile k a wavefront waits (s_waitcnt vmcnt) only for its own DMA of
+// tile k+1, then the workgroup synchronises with a barrier that orders LDS traffic only. The DMA instructions and these
 // waits are inline assembly: left to itself the compiler drains every outstanding LDS-DMA
 // load before an LDS read it cannot prove disjoint, and at __syncthreads().
 //
-// Epilogue. fp32 operands (A32) are read straight into the accumulator layout (128-byte row
-// segments), all loads of a 32-row slab issued before its arithmetic; the bf16 pair of the
-// iterate that X = a X + B X needs at the output position arrives by LDS-DMA two slabs ahead;
-// every bf16 output passes through LDS so that rows and mirrored rows leave as 16-byte
-// stores. Epilogue loads and stores are nontemporal.
+// Epilogue. What an epilogue reads at the output position (fp32 A32 for B, the bf16 pair of the
+// iterate for X = a X + B X, the diagonal vectors) arrives by LDS-DMA in buffers private to the
+// wavefront, two 32-row slabs ahead; a slab waits with an exact vmcnt for its own fetch only.
+// bf16 outputs are converted with v_cvt_pk_bf16_f32 and pass through LDS so that rows and
+// mirrored rows leave as 16-byte nontemporal stores. X = a X + B X issues its MFMAs with the
+// operands exchanged (transposed accumulator layout: a lane holds runs of 4 consecutive columns
+// of one output row) and reads and writes LDS 8 or 16 bytes at a time.
+//
+// One launch covers up to 4 problems (the shape groups of an optimizer step), see NsGemmMulti.
 //
 // Accumulation order per output element is the same in every tile configuration and in the
 // 128x128 kernel of ns.hip (terms in order, k ascending, one accumulator).
