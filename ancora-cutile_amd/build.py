@@ -6,7 +6,8 @@
 The second form builds an ablation variant somewhere else (objects in a temporary directory,
 the product library untouched); `ANCORA_OPTIM_LIB=/tmp/noepi.so` makes the host layer load it.
 Ablation switches of csrc/ns_gemm_big.hip: ANC_DBG_NOEPI (no epilogue), ANC_DBG_NODMA (operand
-tiles fetched for the first K tiles only), ANC_DBG_NOMFMA (matrix instructions replaced by an add).
+tiles fetched for the first K tiles only), ANC_DBG_NOMFMA (matrix instructions replaced by an add),
+ANC_DBG_TRACE (per-workgroup timestamps of K loop and epilogue, read with anc_dbg_trace_read).
 
 hipcc cross-compiles without a GPU. Flags: no FMA contraction (the AdamW kernel must
 reproduce a numpy fp32 evaluation operation by operation), correctly rounded fp32

@@ -41,9 +41,6 @@
 // Accumulation order per output element is the same in every tile configuration and in the
 // 128x128 kernel of ns.hip (terms in order, k ascending, one accumulator).
 #include "ns_common.h"
-#ifndef ANC_DBG_EPI
-#define ANC_DBG_EPI 0
-#endif
 
 #ifdef ANC_DBG_TRACE
 // Debug build only: per-workgroup timestamps (100 MHz wall clock) of the last launch of each kind.
@@ -136,11 +133,7 @@ __device__ __forceinline__ void stage_rows(unsigned char *region, const uint32_t
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, row = idx >> 3, c8 = (idx & 7) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + row * 72 + c8);
-#ifdef ANC_DBG_NOSTORE
-    if (q.x == 0x12345678u) anc_st_stream((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
-#else
     anc_st_stream((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
-#endif
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
@@ -163,11 +156,7 @@ __device__ __forceinline__ void stage_cols(unsigned char *region, const uint32_t
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, col = idx >> 2, r8 = (idx & 3) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + col * 40 + r8);
-#ifdef ANC_DBG_NOSTORE
-    if (q.x == 0x12345678u) anc_st_stream((anc_u32x4 *)(outT + (int64_t)col * ldT + r8), q);
-#else
     anc_st_stream((anc_u32x4 *)(outT + (int64_t)col * ldT + r8), q);
-#endif
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
@@ -635,11 +624,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         const float v = (EPI == EPI_BMAT) ? acc[bi][bj][r] : acc[bi][bj][r] * acc_scale;
         if (EPI == EPI_GRAM) {
           const bool diag = gi == gj;
-#ifdef ANC_DBG_NOSTORE
-          if (v == 12345.678f) p.A32[mm + (int64_t)gi * M + gj] = v;
-#else
           p.A32[mm + (int64_t)gi * M + gj] = v;
-#endif
           ov[bj][r] = diag ? 0.0f : v;
           if (diag) p.dA[mv + gi] = v;
         } else if (EPI == EPI_BMAT) {
