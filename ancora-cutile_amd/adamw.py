@@ -178,6 +178,26 @@ class AdamW:
         """bf16-valued fp32 weights (what the forward consumes), per name."""
         return {n: _bits_f32(s["p16"].numpy()).reshape(s["shape"]) for n, s in self.st.items()}
 
+    def state_dict(self):
+        """Everything a resumed run needs, as host arrays: per tensor the fp32 master, both
+        moments and the bf16 weights, plus the step counter (it enters the bias corrections and
+        the stochastic-rounding seed). The reference has no optimizer checkpoint at all."""
+        out = {"t": np.int64(self.t)}
+        for n, s in self.st.items():
+            for k in ("p32", "m", "v", "p16"):
+                out[f"{n}/{k}"] = s[k].to_numpy()
+        return out
+
+    def load_state_dict(self, sd, stream_int=0):
+        for n, s in self.st.items():
+            for k in ("p32", "m", "v", "p16"):
+                a = np.asarray(sd[f"{n}/{k}"])
+                if a.size != s[k].size or a.dtype != s[k].dtype:
+                    raise ValueError(f"AdamW.load_state_dict: '{n}/{k}' is {a.dtype}[{a.size}], "
+                                     f"expected {s[k].dtype}[{s[k].size}]")
+                s[k].upload(a.reshape(s[k].shape), stream_int)
+        self.t = int(sd["t"])
+
     def master(self):
         return {n: s["p32"].numpy().reshape(s["shape"]) for n, s in self.st.items()}
 

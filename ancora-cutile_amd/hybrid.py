@@ -110,6 +110,26 @@ class HybridOptimizer:
             self.muon.unstep()
             self.adamw.unstep()
 
+    def state_dict(self):
+        """Optimizer state of both groups as one flat {key: ndarray} mapping."""
+        out = {f"muon/{k}": v for k, v in self.muon.state_dict().items()}
+        out.update({f"adamw/{k}": v for k, v in self.adamw.state_dict().items()})
+        return out
+
+    def load_state_dict(self, sd, stream_int=0):
+        self.muon.load_state_dict({k[5:]: v for k, v in sd.items() if k.startswith("muon/")}, stream_int)
+        self.adamw.load_state_dict({k[6:]: v for k, v in sd.items() if k.startswith("adamw/")}, stream_int)
+        _lib.stream_sync(stream_int)
+
+    def save(self, path):
+        """Checkpoint to one uncompressed .npz (plain arrays, no pickle): a run resumed with
+        `load` continues bit for bit. The reference keeps optimizer state in memory only."""
+        np.savez(path, **self.state_dict())
+
+    def load(self, path, stream_int=0):
+        with np.load(path, allow_pickle=False) as z:
+            self.load_state_dict({k: z[k] for k in z.files}, stream_int)
+
     def weights(self):
         return {**self.muon.weights(), **self.adamw.weights()}
 

@@ -470,6 +470,26 @@ class Muon:
             self.unstep()
             self.last_skipped = True
 
+    def state_dict(self):
+        """Host arrays for a resumed run: per weight the fp32 master, the momentum buffer and the
+        bf16 weights, plus the step counter (it seeds the stochastic rounding)."""
+        out = {"t": np.int64(self.engine.t if self.engine is not None else 0)}
+        for n, s in self.st.items():
+            for k in ("p32", "buf", "p16"):
+                out[f"{n}/{k}"] = s[k].to_numpy()
+        return out
+
+    def load_state_dict(self, sd, stream_int=0):
+        for n, s in self.st.items():
+            for k in ("p32", "buf", "p16"):
+                a = np.asarray(sd[f"{n}/{k}"])
+                if a.size != s[k].size or a.dtype != s[k].dtype:
+                    raise ValueError(f"Muon.load_state_dict: '{n}/{k}' is {a.dtype}[{a.size}], "
+                                     f"expected {s[k].dtype}[{s[k].size}]")
+                s[k].upload(a.reshape(s[k].shape), stream_int)
+        if self.engine is not None:
+            self.engine.t = int(sd["t"])
+
     def weights(self):
         """bf16-valued fp32 weights for the forward (ancora/optim/muon.py:311-312)."""
         return {n: _bf(s["p32"].to_numpy()).reshape(s["shape"]) for n, s in self.st.items()}

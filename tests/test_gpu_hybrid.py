@@ -154,3 +154,35 @@ def test_expert_optimizer(gpu):
     for b in list(Gd.values()) + [rgd]:
         b.free()
     opt.free()
+
+
+def test_checkpoint_resume_is_bitwise(gpu, tmp_path):
+    """save() after two steps, load() into a fresh optimizer, two more steps on both: masters,
+    moments, momentum and bf16 weights agree bit for bit (stochastic rounding included: the step
+    counters travel with the state)."""
+    from ancora_cutile_amd import HybridOptimizer, PE_SCHEDULE
+    rng = np.random.default_rng(5)
+    params = {"embed": (0.02 * rng.standard_normal((256, 128))).astype(np.float32),
+              "final_norm": np.ones(128, np.float32),
+              "layer0.q_proj": (0.02 * rng.standard_normal((128, 256))).astype(np.float32),
+              "layer0.down_proj": (0.02 * rng.standard_normal((384, 128))).astype(np.float32)}
+    grads = [{n: (1e-2 * rng.standard_normal(p.shape)).astype(np.float32) for n, p in params.items()}
+             for _ in range(4)]
+    kw = dict(muon_kw=dict(schedule=PE_SCHEDULE, sr=True, seed=3), max_grad_norm=1.0,
+              adamw_kw=dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.1, sr=True, seed=9))
+    a = HybridOptimizer(params, **kw)
+    for g in grads[:2]:
+        a.step(g, 0)
+    path = str(tmp_path / "opt.npz")
+    a.save(path)
+    for g in grads[2:]:
+        a.step(g, 0)
+    b = HybridOptimizer(params, **kw)
+    b.load(path)
+    for g in grads[2:]:
+        b.step(g, 0)
+    sa, sb = a.state_dict(), b.state_dict()
+    assert sa.keys() == sb.keys()
+    for k in sa:
+        assert np.atleast_1d(sa[k]).tobytes() == np.atleast_1d(sb[k]).tobytes(), k
+    a.free(); b.free()
