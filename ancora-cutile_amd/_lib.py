@@ -57,7 +57,7 @@ class GnDesc(C.Structure):
 class MuonDesc(C.Structure):
     _fields_ = [("buf", u64), ("g", u64), ("p32", u64), ("p16", u64), ("u", u64), ("K", i32),
                 ("N", i32), ("transpose", i32), ("g_dtype", i32), ("scale_idx", i32),
-                ("seed", u32), ("tile0", i64)]
+                ("seed", u32), ("tile0", i64), ("p16t", u64)]
 
 
 class NsProblem(C.Structure):

@@ -173,9 +173,8 @@ __device__ __forceinline__ void mom_tile_t(const MomArgs &a, int64_t tile, float
 // ---- update: p32 -= lr_scale*O; p16 = bf16(p32) ----------------------------------
 template <int SR>
 __device__ __forceinline__ void upd_store(const UpdArgs &a, int64_t e, const float o[4],
-                                          const anc_f32x4 &p) {
+                                          const anc_f32x4 &p, uint32_t (&hb)[4]) {
   float pp[4] = {p.x, p.y, p.z, p.w};
-  uint32_t hb[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     pp[k] = pp[k] - a.lr_scale * o[k];
@@ -189,6 +188,13 @@ __device__ __forceinline__ void upd_store(const UpdArgs &a, int64_t e, const flo
     anc_u32x2 ho = {(hb[0] & 0xFFFFu) | (hb[1] << 16), (hb[2] & 0xFFFFu) | (hb[3] << 16)};
     anc_st_stream((anc_u32x2 *)(a.p16 + e), ho);
   }
+}
+
+template <int SR>
+__device__ __forceinline__ void upd_store(const UpdArgs &a, int64_t e, const float o[4],
+                                          const anc_f32x4 &p) {
+  uint32_t hb[4];
+  upd_store<SR>(a, e, o, p, hb);
 }
 
 template <int OD, int SR>
@@ -208,31 +214,62 @@ __device__ __forceinline__ void upd_flat(const UpdArgs &a, int64_t blk) {
   }
 }
 
+// ---- update that also refreshes a transposed bf16 copy of the weight -------------------
+// p16t is (N,K): the copy the MoE backward reads (ancora/kernels/moe.py:370-377, 593-597 runs a
+// separate transpose kernel over p16 after the step). 64x64 tile of W per block in either
+// orientation of O; the new bf16 values cross LDS once more and leave as rows of p16t.
 template <int OD, int SR>
-__device__ __forceinline__ void upd_tile_t(const UpdArgs &a, int64_t tile) {
-  __shared__ float lds[kTile][kTile + 1];
+__device__ __forceinline__ void upd_tile_p16t(const UpdArgs &a, int64_t tile, bool o_transposed,
+                                              uint16_t *p16t) {
+  __shared__ float ldsO[kTile][kTile + 1];
+  __shared__ uint16_t ldsH[kTile][kTile + 2];
   const int tiles_n = a.N / kTile;
   const int tr = (int)(tile / tiles_n), tc = (int)(tile % tiles_n);
   const int c4 = (threadIdx.x & 15) * 4, r0 = threadIdx.x >> 4;
-  // O is (N,K): read rows tc*64 + r, columns tr*64 + c4 ..
+  if (o_transposed) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = r0 + 16 * i;
-    const int64_t e = (int64_t)(tc * kTile + r) * a.K + tr * kTile + c4;
-    const anc_f32x4 o = load4<OD>(a.O, e);
-    lds[r][c4] = o.x; lds[r][c4 + 1] = o.y; lds[r][c4 + 2] = o.z; lds[r][c4 + 3] = o.w;
+    for (int i = 0; i < 4; ++i) {
+      const int r = r0 + 16 * i;
+      const int64_t e = (int64_t)(tc * kTile + r) * a.K + tr * kTile + c4;
+      const anc_f32x4 o = load4<OD>(a.O, e);
+      ldsO[r][c4] = o.x; ldsO[r][c4 + 1] = o.y; ldsO[r][c4 + 2] = o.z; ldsO[r][c4 + 3] = o.w;
+    }
+    __syncthreads();
   }
-  __syncthreads();
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = r0 + 16 * i;
     const int64_t e = (int64_t)(tr * kTile + r) * a.N + tc * kTile + c4;
     const anc_f32x4 p = anc_ld_stream((const anc_f32x4 *)(a.p32 + e));
     float oo[4];
+    if (o_transposed) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) oo[k] = lds[c4 + k][r];
-    upd_store<SR>(a, e, oo, p);
+      for (int k = 0; k < 4; ++k) oo[k] = ldsO[c4 + k][r];
+    } else {
+      const anc_f32x4 o = load4<OD>(a.O, e);
+      oo[0] = o.x; oo[1] = o.y; oo[2] = o.z; oo[3] = o.w;
+    }
+    uint32_t hb[4];
+    upd_store<SR>(a, e, oo, p, hb);
+    if (p16t != nullptr) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) ldsH[r][c4 + k] = (uint16_t)hb[k];
+    }
   }
+  if (p16t == nullptr) return;        // uniform over the block
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + 16 * i;
+    const uint32_t h0 = ldsH[c4][r], h1 = ldsH[c4 + 1][r], h2 = ldsH[c4 + 2][r], h3 = ldsH[c4 + 3][r];
+    const anc_u32x2 ho = {h0 | (h1 << 16), h2 | (h3 << 16)};
+    anc_st_stream((anc_u32x2 *)(p16t + (int64_t)(tc * kTile + r) * a.K + tr * kTile + c4), ho);
+  }
+}
+
+template <int OD, int SR>
+__device__ __forceinline__ void upd_tile_t(const UpdArgs &a, int64_t tile) {
+  upd_tile_p16t<OD, SR>(a, tile, true, nullptr);
 }
 
 // ---- kernels -----------------------------------------------------------------------
@@ -320,8 +357,10 @@ k_upd_multi(const anc_muon_desc_t *__restrict__ table, int n_weights, LrScales s
   const int64_t local = (int64_t)blockIdx.x - d.tile0;
   UpdArgs a{(float *)d.p32, (uint16_t *)d.p16, (const void *)d.u, d.K, d.N,
             scales.v[d.scale_idx & (ANC_MUON_MAX_SCALES - 1)], seed_base + d.seed};
-  if (d.transpose) upd_tile_t<OD, SR>(a, local);
-  else             upd_flat<OD, SR>(a, local);
+  if (d.p16t != 0 || d.transpose)
+    upd_tile_p16t<OD, SR>(a, local, d.transpose != 0, (uint16_t *)d.p16t);
+  else
+    upd_flat<OD, SR>(a, local);
 }
 
 // bf16 transpose, batched: XT[e] (N,M) = X[e] (M,N)^T, 64x64 tiles through LDS.

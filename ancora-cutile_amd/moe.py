@@ -5,9 +5,9 @@ Mirror of the optimizer part of ancora/kernels/moe.py: `ExpertMuonScratch` (:404
 and backward are not part of this package) into `ExpertOptimizer`. Expert tensors are
 stacked [E, K, N]; with optimizer="muon" every expert slice is one matrix of a batched
 Newton-Schulz chain (fp32 master + one momentum buffer, no second moment), otherwise the
-flat tensor goes through AdamW. The router stays on AdamW (wd = 0, :603-604). After the
-update the transposed copies the backward reads are refreshed (`_transpose_e`, :370-377,
-593-597).
+flat tensor goes through AdamW. The router stays on AdamW (wd = 0, :603-604). The transposed
+copies the backward reads (`_transpose_e`, :370-377, 593-597) are refreshed by the Muon update
+kernel in the same pass; the AdamW variant runs the transpose kernel after the step.
 """
 import ctypes
 
@@ -85,7 +85,7 @@ class ExpertOptimizer:
                 for e in range(s["E"]):
                     recs.append(dict(buf=s["buf"].at_pos(e * s["K"]), p32=s["p32"].at_pos(e * s["K"]),
                                      p16=s["p16"].at_pos(e * s["K"]), G=g2.at_pos(e * s["K"]),
-                                     K=s["K"], N=s["N"]))
+                                     p16T=s["p16T"].at_pos(e * s["N"]), K=s["K"], N=s["N"]))
             ws = None if self._scratch is None else self._scratch.ws
             self._engine = MuonEngine(recs, self._mom, self._ns, True, None, None, self._mode,
                                       workspace=ws)
@@ -107,9 +107,10 @@ class ExpertOptimizer:
                 s = self.st[name]
                 _adamw(si, grads[name], s["m"], s["v"], s["p32"], s["p16"], 0, b1, b2, self._eps, lr,
                        self._wd, ibc1, ibc2, ctl)
-        for name in self.NAMES:                      # refresh the transposed backward weights
-            s = self.st[name]
-            api.anc_transpose_bf16(s["p16"].ptr, s["p16T"].ptr, s["E"], s["K"], s["N"], int(si))
+        if self.optimizer != "muon":                 # Muon's update kernel refreshes p16T itself
+            for name in self.NAMES:                  # the transposed backward weights
+                s = self.st[name]
+                api.anc_transpose_bf16(s["p16"].ptr, s["p16T"].ptr, s["E"], s["K"], s["N"], int(si))
         if self.router is not None and router_grad is not None:
             r = self.router
             _adamw(si, router_grad, r["m"], r["v"], r["p32"], r["p16"], r["otm"], b1, b2, self._eps,

@@ -62,7 +62,8 @@ class _Batch:
 
     def build(self, U, scale_index):
         key = tuple((w["G"].ptr, w["G"].dtype.str, w["p32"].ptr, w["p16"].ptr if w["p16"] is not None else 0,
-                     w["buf"].ptr) for w in self.weights) + (U.ptr,)
+                     w["buf"].ptr, w["p16T"].ptr if w.get("p16T") is not None else 0)
+                    for w in self.weights) + (U.ptr,)
         if key == self.key:
             return
         if self.table is not None:
@@ -73,7 +74,8 @@ class _Batch:
             descs.append(MuonDesc(w["buf"].ptr, w["G"].ptr, w["p32"].ptr,
                                   w["p16"].ptr if w["p16"] is not None else 0,
                                   U.ptr + i * self.M * self.Nn * 4, K, N, int(K > N),
-                                  _g_code(w["G"].dtype), scale_index[w["scale"]], w["seed"], blk0))
+                                  _g_code(w["G"].dtype), scale_index[w["scale"]], w["seed"], blk0,
+                                  w["p16T"].ptr if w.get("p16T") is not None else 0))
             blk0 += (K * N) // 4096
         self.total_blocks = blk0
         self.table = upload_table(descs)
@@ -92,7 +94,8 @@ class MuonEngine:
     """Shape-grouped, batched Muon over device-resident weights.
 
     weights: list of dicts {buf, p32, p16, G: DevBuf; K, N: int; lid: int (optional)} -- the
-    record of ancora/optim/muon.py:220. `chunk` caps the matrices per batch (None = the whole
+    record of ancora/optim/muon.py:220; an optional `p16T` DevBuf (N,K) is a transposed bf16
+    copy that the update refreshes in the same pass. `chunk` caps the matrices per batch (None = the whole
     shape group, which is what 288 GB of HBM is for); `scope=k` sub-groups by lid // k
     (ancora/optim/muon.py:221-222,235). Neither changes any result bit."""
 

@@ -253,6 +253,9 @@ typedef struct {
   int32_t  scale_idx;          /* which of the launch's lr_scale values applies   */
   uint32_t seed;               /* per-weight SR seed offset (added to seed_base)  */
   int64_t  tile0;              /* index of this weight's first 4096-element block */
+  uint64_t p16t;               /* 0, or a (N,K) bf16 copy of the weight that the update
+                                  refreshes in the same pass (replaces the `_transpose_e`
+                                  launch after the step, ancora/kernels/moe.py:593-597)   */
 } anc_muon_desc_t;
 #define ANC_MUON_MAX_SCALES 8
 /* All weights of a packed batch in ONE launch each (the reference launches once per

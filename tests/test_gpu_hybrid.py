@@ -122,34 +122,38 @@ def test_chunk_and_scope_are_bitwise_neutral(gpu):
                 assert bits_equal(x, y)
 
 
-def test_expert_optimizer(gpu):
+@pytest.mark.parametrize("Ie", [128, 256])
+def test_expert_optimizer(gpu, Ie):
     """Stacked [E,K,N] experts: Muon per slice, idle experts (zero grad) leave their weights
-    unchanged at step 1, router on AdamW with wd=0, transposed copies refreshed."""
+    unchanged at step 1, router on AdamW with wd=0, transposed copies refreshed (wide
+    gate/up and tall down projections when Ie != H)."""
     from ancora_cutile_amd import ExpertOptimizer, DevBuf, PE_SCHEDULE as PE
-    from oracle.muon_ref import muon_momentum, host_ns, muon_update
+    from oracle.muon_ref import muon_momentum, ns_any_shape, muon_update, shape_scale
     rng = np.random.default_rng(4)
     E, H = 4, 128
-    W = {n: (0.02 * rng.standard_normal((E, H, H))).astype(np.float32)
-         for n in ("gate_proj", "up_proj", "down_proj")}
+    shp = {"gate_proj": (H, Ie), "up_proj": (H, Ie), "down_proj": (Ie, H)}
+    W = {n: (0.02 * rng.standard_normal((E,) + kn)).astype(np.float32) for n, kn in shp.items()}
     router = (0.02 * rng.standard_normal((H, 16))).astype(np.float32)
-    G = {n: rng.standard_normal((E, H, H)).astype(np.float32) for n in W}
+    G = {n: rng.standard_normal(W[n].shape).astype(np.float32) for n in W}
     for n in G:
         G[n][2] = 0
-    Gd = {n: DevBuf(g.reshape(E * H, H)) for n, g in G.items()}
+    Gd = {n: DevBuf(g.reshape(E * shp[n][0], shp[n][1])) for n, g in G.items()}
     rg = rng.standard_normal((H, 16)).astype(np.float32)
     rgd = DevBuf(rg.reshape(-1, 64))
     opt = ExpertOptimizer(W, router)
     opt.step(Gd, 0, lr=1e-3, muon_lr=0.02, router_grad=rgd, schedule=PE)
     m = opt.master()
     for n in W:
+        K, N = shp[n]
         assert bits_equal(m[n][2], W[n][2])                       # idle expert untouched
-        _, u = muon_momentum(np.zeros((H, H), np.float32), G[n][0])
-        want = muon_update(W[n][0], host_ns(u, PE_SCHEDULE, 5), 0.02)
-        assert rel_fro((W[n][0] - m[n][0]) / 0.02, (W[n][0] - want) / 0.02) < 2.5e-3
+        _, u = muon_momentum(np.zeros((K, N), np.float32), G[n][0])
+        want = muon_update(W[n][0], ns_any_shape(u, PE_SCHEDULE, 5), 0.02)
+        step = 0.02 * shape_scale(K, N)
+        assert rel_fro((W[n][0] - m[n][0]) / step, (W[n][0] - want) / step) < 2.5e-3
         s = opt.st[n]
-        p16 = s["p16"].to_numpy().reshape(E, H, H)
-        assert np.array_equal(s["p16T"].to_numpy().reshape(E, H, H), p16.transpose(0, 2, 1))
-        assert bits_equal(p16, bf16_rne_bits(m[n]).reshape(E, H, H))
+        p16 = s["p16"].to_numpy().reshape(E, K, N)
+        assert np.array_equal(s["p16T"].to_numpy().reshape(E, N, K), p16.transpose(0, 2, 1))
+        assert bits_equal(p16, bf16_rne_bits(m[n]).reshape(E, K, N))
     assert not np.array_equal(m["router"], router)
     for b in list(Gd.values()) + [rgd]:
         b.free()

@@ -144,3 +144,43 @@ def test_momentum_pair_output_and_frobenius_partials(gpu, K, N):
         assert abs(parts[i].sum() - want) <= 1e-12 * want
     for b in bd + gd + [U, fro, table]:
         b.free()
+
+
+@pytest.mark.parametrize("K,N", [(128, 256), (256, 128), (192, 192)])
+@pytest.mark.parametrize("sr", [0, 1])
+def test_update_multi_refreshes_the_transposed_copy(gpu, K, N, sr):
+    """With `p16t` set in the descriptor, the update leaves p16t == p16^T bit for bit (what a
+    separate transpose launch after the step would leave), p32 and p16 exactly as without it;
+    a weight with p16t = 0 in the same table is untouched by the new path."""
+    import ctypes as C
+    from ancora_cutile_amd import DevBuf, _lib
+    from ancora_cutile_amd._lib import api, MuonDesc
+    from ancora_cutile_amd.devbuf import upload_table
+    rng = np.random.default_rng(7 * K + N + sr)
+    E = 3
+    M, Nn = min(K, N), max(K, N)
+    tr = int(K > N)
+    Ws = [(0.05 * rng.standard_normal((K, N))).astype(np.float32) for _ in range(E)]
+    Os = [rng.standard_normal((K, N)).astype(np.float32) for _ in range(E)]
+    U = DevBuf(np.stack([np.ascontiguousarray(o.T) if tr else o for o in Os]).reshape(E * M, Nn))
+    p32 = [DevBuf(w) for w in Ws]
+    p16 = [DevBuf.zeros((K, N), np.uint16) for _ in range(E)]
+    p16t = [DevBuf.zeros((N, K), np.uint16) for _ in range(E - 1)]
+    descs, blk0 = [], 0
+    for i in range(E):
+        descs.append(MuonDesc(0, 0, p32[i].ptr, p16[i].ptr, U.ptr + i * M * Nn * 4, K, N, tr, _lib.F32, 0,
+                              11 * i, blk0, p16t[i].ptr if i < E - 1 else 0))
+        blk0 += K * N // 4096
+    table = upload_table(descs)
+    lr, seed_base = 0.02, 1234
+    scales = (C.c_float * _lib.MUON_MAX_SCALES)(*([lr * shape_scale(K, N)] * _lib.MUON_MAX_SCALES))
+    api.anc_muon_update_multi(table.ptr, E, blk0, scales, _lib.F32, sr, seed_base, 0, 0)
+    for i in range(E):
+        want = muon_update(Ws[i], Os[i], lr)
+        assert bits_equal(p32[i].to_numpy(), want)
+        w16 = (bf16_sr_bits(want, seed_base + 11 * i) if sr else bf16_rne_bits(want)).reshape(K, N)
+        assert bits_equal(p16[i].to_numpy(), w16)
+        if i < E - 1:
+            assert np.array_equal(p16t[i].to_numpy(), w16.T)
+    for b in p32 + p16 + p16t + [U, table]:
+        b.free()

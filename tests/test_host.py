@@ -35,7 +35,7 @@ def test_struct_sizes_match_header():
     assert ctypes.sizeof(_lib.AdamWHyper) == 48
     assert ctypes.sizeof(_lib.AdamWDesc) == 72
     assert ctypes.sizeof(_lib.GnDesc) == 40
-    assert ctypes.sizeof(_lib.MuonDesc) == 72
+    assert ctypes.sizeof(_lib.MuonDesc) == 80
     assert ctypes.sizeof(_lib.DeviceInfo) == 24 + 16 + 128
 
 
