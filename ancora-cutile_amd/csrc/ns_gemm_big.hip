@@ -42,6 +42,15 @@
 // 128x128 kernel of ns.hip (terms in order, k ascending, one accumulator).
 #include "ns_common.h"
 
+// Epilogue store; the timing-only ablation ANC_DBG_EPI_NOST never executes it.
+template <typename T> __device__ __forceinline__ void epi_st(T *p, T v) {
+#if defined(ANC_DBG_EPI_NOST)
+  if (((uintptr_t)p & 1) != 0) *p = v;
+#else
+  anc_st_stream(p, v);
+#endif
+}
+
 #ifdef ANC_DBG_TRACE
 // Debug build only: per-workgroup timestamps (100 MHz wall clock) of the last launch of each kind.
 __device__ unsigned long long anc_dbg_ts[3][16384][4];
@@ -133,7 +142,7 @@ __device__ __forceinline__ void stage_rows(unsigned char *region, const uint32_t
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, row = idx >> 3, c8 = (idx & 7) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + row * 72 + c8);
-    anc_st_stream((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
+    epi_st((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
@@ -156,7 +165,7 @@ __device__ __forceinline__ void stage_cols(unsigned char *region, const uint32_t
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, col = idx >> 2, r8 = (idx & 3) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + col * 40 + r8);
-    anc_st_stream((anc_u32x4 *)(outT + (int64_t)col * ldT + r8), q);
+    epi_st((anc_u32x4 *)(outT + (int64_t)col * ldT + r8), q);
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
@@ -178,6 +187,13 @@ template <int N> __device__ __forceinline__ void wait_vm() {
 __device__ __forceinline__ void dma16(const void *g, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g)
                : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_epi(const void *g, uint32_t lds_base) {
+#if defined(ANC_DBG_EPI_NOLD)
+  (void)g; (void)lds_base;
+#else
+  dma16(g, lds_base);
+#endif
 }
 __device__ __forceinline__ uint32_t lds_addr(const void *p) {
   return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void *)p);
@@ -395,7 +411,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         mfma8<BT>(f[kk & 1], acc);
       }
     }
+#ifndef ANC_DBG_KNOWAIT
     if (refill) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
+#endif
     lds_barrier();
     if (more) frags(nxt, 0, f[0]);
     mfma8<BT>(f[(KSTEPS - 1) & 1], acc);
@@ -445,8 +463,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     for (int j = 0; j < 4; ++j) {
       const int64_t ro = (int64_t)(8 * j) * N * 2;
       const uint32_t vo = (j & 1) ? vo_in1 : vo_in0;
-      dma16((const char *)p.Xh + ub + ro + vo, lds_addr(b + j * 1024));
-      dma16((const char *)p.Xl + ub + ro + vo, lds_addr(b + 4096 + j * 1024));
+      dma16_epi((const char *)p.Xh + ub + ro + vo, lds_addr(b + j * 1024));
+      dma16_epi((const char *)p.Xl + ub + ro + vo, lds_addr(b + 4096 + j * 1024));
     }
   };
   // B = b A + c A A reads A32 at the output position the same way: a 32x64 fp32 slab is 32 rows
@@ -459,7 +477,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     unsigned char *b = inbuf(bi);
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      dma16((const char *)p.A32 + ub + (int64_t)(4 * j) * M * 4 + ((j & 1) ? vo_a1 : vo_a0), lds_addr(b + j * 1024));
+      dma16_epi((const char *)p.A32 + ub + (int64_t)(4 * j) * M * 4 + ((j & 1) ? vo_a1 : vo_a0), lds_addr(b + j * 1024));
   };
   int in_lane[2] = {0, 0};
   unsigned char *aux_w = aux + (EPI != EPI_GRAM ? wave * 1024 : 0);
@@ -538,7 +556,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         for (int pz = 0; pz < 8; ++pz) {
           const int idx = pz * 64 + lane, row = idx >> 4, c = idx & 15;
           const anc_f32x4 v4 = *(const anc_f32x4 *)(b + row * 256 + ((c ^ (row & 15)) * 16));
-          anc_st_stream((anc_f32x4 *)(p.X32 + mn + (int64_t)(gi0 + row) * N + gj0w + c * 4), v4);
+          epi_st((anc_f32x4 *)(p.X32 + mn + (int64_t)(gi0 + row) * N + gj0w + c * 4), v4);
         }
       } else {
 #pragma unroll
@@ -560,14 +578,14 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           const int idx = pz * 64 + lane, row = idx >> 3, c = idx & 7;
           const int off = row * 128 + ((c ^ ((row & 7) ^ ((row >> 3) & 1))) * 16);
           const anc_u32x4 qh = *(const anc_u32x4 *)(b + off);
-          anc_st_stream((anc_u32x4 *)(p.Yh + mn + (int64_t)(gi0 + row) * N + gj0w + c * 8), qh);
+          epi_st((anc_u32x4 *)(p.Yh + mn + (int64_t)(gi0 + row) * N + gj0w + c * 8), qh);
         }
 #pragma unroll
         for (int pz = 0; pz < 4; ++pz) {
           const int idx = pz * 64 + lane, row = idx >> 3, c = idx & 7;
           const int off = row * 128 + ((c ^ ((row & 7) ^ ((row >> 3) & 1))) * 16);
           const anc_u32x4 ql = *(const anc_u32x4 *)(b + 4096 + off);
-          anc_st_stream((anc_u32x4 *)(p.Yl + mn + (int64_t)(gi0 + row) * N + gj0w + c * 8), ql);
+          epi_st((anc_u32x4 *)(p.Yl + mn + (int64_t)(gi0 + row) * N + gj0w + c * 8), ql);
         }
       }
       // the buffer is free again once the staged rows have been read back
