@@ -14,3 +14,4 @@ from .muon import (Muon, DeviceMuon, MuonScratch, ResidentMuon, BatchedProjMuon,
                    newton_schulz5)
 from .moe import ExpertMuonScratch, ExpertOptimizer                          # noqa: F401
 from .hybrid import HybridOptimizer, default_is_muon, resident_is_muon       # noqa: F401
+from .quant import Mxfp8WeightCache, quant_mxfp8_w                          # noqa: F401

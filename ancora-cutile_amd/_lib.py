@@ -112,6 +112,7 @@ _PROTOS = {
     "anc_muon_update_multi": (None, [u64, i32, i64, C.POINTER(f32), C.c_int, C.c_int, u32, u64,
                                      u64]),
     "anc_transpose_bf16": (None, [u64, u64, i64, i64, i64, u64]),
+    "anc_quant_mxfp8_w": (None, [u64, u64, u64, i64, i64, i64, C.c_int, u64]),
     "anc_ns_workspace_bytes": (i64, [i64, i64, i64, C.c_int]),
     "anc_ns_batched": (None, [u64, i64, i64, i64, C.c_int, C.POINTER(f32), f32, C.c_int, u64, i64,
                               u64]),

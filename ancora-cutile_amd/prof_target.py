@@ -6,6 +6,8 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
                                       per-launch event timer and prints ms per kernel kind)
     python3 -m ancora_cutile_amd.prof_target adamw NUMEL [calls]         fused AdamW, bf16 grads, SR
     python3 -m ancora_cutile_amd.prof_target gradnorm NUMEL [calls]      grad-norm partials + finalize
+    python3 -m ancora_cutile_amd.prof_target quant K N E [cm] [calls]    MXFP8 weight re-quantisation
+                                      (prints GB/s from HIP events around the calls)
     python3 -m ancora_cutile_amd.prof_target mfmamix                    matrix-instruction rate next to
                                       unrelated LDS / LDS-DMA traffic (anc_probe_mfma_mix), a table
 
@@ -58,6 +60,28 @@ def main(argv):
         guard = StepGuard(1.0)
         for _ in range(calls):
             guard.compute([g], 0)
+    elif what == "quant":
+        K, N, E = int(argv[1]), int(argv[2]), int(argv[3])
+        cm = len(argv) > 4 and argv[4] == "cm"
+        calls = int(argv[5]) if len(argv) > 5 else 5
+        wb = (np.random.default_rng(0).standard_normal((K, N)) * 0.05).astype(np.float32)
+        wb = (wb.view(np.uint32) >> 16).astype(np.uint16)
+        w = DevBuf.empty((E * K, N), np.uint16)
+        for e in range(E):
+            w.at_pos(e * K).upload(wb)
+        f8 = DevBuf.zeros((E * K * N,), np.uint8)
+        sc = DevBuf.zeros((E * K * N // 32,), np.uint8)
+        t0, t1 = _lib.Event(), _lib.Event()
+        _lib.api.anc_quant_mxfp8_w(w.ptr, f8.ptr, sc.ptr, E, K, N, int(cm), 0)
+        t0.record(0)
+        for _ in range(calls):
+            _lib.api.anc_quant_mxfp8_w(w.ptr, f8.ptr, sc.ptr, E, K, N, int(cm), 0)
+        t1.record(0)
+        t1.sync()
+        ms = t0.elapsed_ms(t1) / calls
+        nbytes = E * K * N * (2 + 1 + 1 / 32)
+        print(f"quant_mxfp8_w {'column-major' if cm else 'row-major'} {E}x({K},{N}): {ms * 1e3:.1f} us per call, "
+              f"{nbytes / ms / 1e9:.2f} TB/s of {nbytes / 1e9:.3f} GB algorithmic")
     elif what == "mfmamix":
         src = DevBuf.zeros((1 << 28,), np.float32)          # 1 GiB
         sink = DevBuf.zeros((512,), np.float32)

@@ -286,6 +286,19 @@ int anc_muon_update_multi(uint64_t desc_table, int32_t n_weights, int64_t total_
 int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
                        uint64_t stream);
 
+/* MXFP8 re-quantisation of bf16 weights (E, K, N) after the step: per block of 32 consecutive K
+ * and per column one E8M0 scale byte = (biased fp32 exponent of the block's amax) - 7 (0 below
+ * 7), elements E4M3FN(w / 2^(byte-127)) rounded to nearest even. col_major = 0 writes
+ * fp8_out (E, K, N) and scale_out (E, K/32, N): replaces `_quant_mxfp8_w`
+ * (ancora/kernels/quant.py:60-73); col_major = 1 writes the transposed fp8_out (E, N, K) and
+ * scale_out (E, N, K/32): replaces `_quant_mxfp8_w_cm` (quant.py:84-100). The reference launches
+ * them per weight from the forward that follows a step (ancora/model/resident_train.py:190-199,
+ * dirty flags set by the step at :354-357). K and N must be multiples of 128 (the reference:
+ * K % 32, N % 128); w and fp8_out 16-byte, scale_out 8-byte aligned. bf16 subnormals count as
+ * zero, Inf/NaN elements become the E4M3 NaN byte. */
+int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int64_t E, int64_t K,
+                      int64_t N, int col_major, uint64_t stream);
+
 /* --------------------------------------------------------- Newton-Schulz ---
  * Replaces the chains `newton_schulz_resident` / `newton_schulz_resident_e`
  * (ancora/kernels/muon_ns.py:245-283, 430-468) and the kernels they launch

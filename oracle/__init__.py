@@ -25,5 +25,12 @@ How each function is pinned (see tests/test_oracle_*.py):
                                     (tests/kernels/_probe_polar_express_device.py:83)
   muon_step / hybrid routing        table-driven over the Qwen3 / MoE name lists, shape scale
                                     sqrt(max(1, rows/cols)) on square, wide and tall weights
-No function here is "parity unpinned".
+  quant_mxfp8_w / e4m3_rne          (quant_ref.py) format constants, midpoints and their neighbours,
+                                    an independent integer-bit formulation over every bf16 input
+                                    and every reachable scale, powers of two, zero blocks, the
+                                    format's error bound and the reference-held 8 % acceptance
+                                    (tests/kernels/test_gpu_quant.py:45-47,68)
+No function of the optimizer step is "parity unpinned". quant_mxfp8_w has three edge behaviours
+that no reference-held vector fixes (blocks with amax < 2**-120, bf16 subnormal inputs,
+non-finite inputs): they are parity unpinned and listed in the header of quant_ref.py.
 """
