@@ -120,8 +120,11 @@ _PROTOS = {
                                    C.c_int, u64, i64, u64]),
     "anc_ns_batched_pair_multi": (None, [C.POINTER(NsProblem), i32, C.c_int, C.POINTER(f32), f32, C.c_int,
                                          u64]),
+    "anc_muon_ns_update_multi": (None, [C.POINTER(NsProblem), i32, C.POINTER(u64), C.c_int, C.POINTER(f32), f32,
+                                        C.c_int, C.POINTER(f32), C.c_int, u32, u64, u64]),
     "anc_ns_flops": (None, [i64, i64, i64, C.c_int, C.c_int, C.POINTER(C.c_double),
                             C.POINTER(C.c_double)]),
+    "anc_ns_product_flops": (None, [i64, i64, i64, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "anc_probe_mfma_mix": (None, [C.c_int, C.c_int, C.c_int, C.c_int, u64, i64, u64,
                                   C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "anc_bf16_to_f32": (None, [u64, u64, i64, u64]),
@@ -204,7 +207,7 @@ def stream_sync(stream=0):
 
 PROF_KINDS = ("adamw", "gradnorm_partials", "gradnorm_finalize", "muon_momentum", "muon_update",
               "ns_fro", "ns_prep", "ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx", "ns_gemm_f32",
-              "misc", "copy")
+              "misc", "copy", "ns_gemm_bx_update")
 
 
 def profile_enable(on=True):

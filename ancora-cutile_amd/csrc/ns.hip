@@ -468,6 +468,7 @@ struct ChainProb {
   const float *scale0;         // per-matrix factor the first step applies to its input, or null
   float *X32;                  // fp32 result (may overlay the input pair when steps >= 2)
   int64_t E, M, N;
+  const anc_muon_desc_t *upd;  // or: the weights (E entries) the last step updates in its epilogue
 };
 
 // steps x { A = X X^T; B = b A + c A A; X = a X + B X } on n problems side by side: every
@@ -475,7 +476,8 @@ struct ChainProb {
 // longest K first). First step's output goes to pair `nxt` of each plan, later steps ping-pong;
 // the last step writes the fp32 results. With n == 1 and a shape that is not a multiple of 256
 // (or force_small) the 128x128-tile kernel runs instead.
-int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool force_small, hipStream_t s) {
+int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool force_small, hipStream_t s,
+                   const NsUpdate *upd = nullptr) {
   bool big = !force_small;
   for (int q = 0; q < n; ++q) big = big && (cp[q].M % 256 == 0) && (cp[q].N % 256 == 0);
   ANC_REQUIRE(big || n == 1, "Newton-Schulz chain: several problems per launch need dims that are multiples of 256");
@@ -527,7 +529,8 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       gx[q].Xh = curH[q]; gx[q].Xl = curL[q];
       gx[q].Yh = last ? nullptr : pl.Xh[nxt[q]];
       gx[q].Yl = last ? nullptr : pl.Xl[nxt[q]];
-      gx[q].X32 = last ? cp[q].X32 : nullptr;
+      gx[q].X32 = (last && cp[q].upd == nullptr) ? cp[q].X32 : nullptr;
+      gx[q].upd = last ? cp[q].upd : nullptr;
     }
     const int tM0 = (int)(cp[0].M / BM), tN0 = (int)(cp[0].N / BN);
     const unsigned g_sym = (unsigned)(cp[0].E * tM0 * (tM0 + 1) / 2), g_mn = (unsigned)(cp[0].E * tM0 * tN0);
@@ -544,8 +547,8 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
     }
     ANC_LAUNCH_CHECK();
     {
-      AncProfScope prof(ANC_PROF_NS_BX, s);
-      if (big) { if (int rc = anc_ns_gemm_big_multi(EPI_BX, gx, Es, n, s)) return rc; }
+      AncProfScope prof(last && upd != nullptr ? ANC_PROF_NS_BX_UPD : ANC_PROF_NS_BX, s);
+      if (big) { if (int rc = anc_ns_gemm_big_multi(EPI_BX, gx, Es, n, s, last ? upd : nullptr)) return rc; }
       else hipLaunchKernelGGL(k_ns_gemm<EPI_BX>, dim3(g_mn), dim3(kGemmThreads), 0, s, gx[0]);
     }
     ANC_LAUNCH_CHECK();
@@ -587,6 +590,28 @@ extern "C" int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode
     ex += tM * tN * (1 + (sx ? 1 : 0) + (sfb ? 1 : 0)) * tile * m;       // X = a X + B X
   }
   *executed = e * ex;
+  return ANC_OK;
+}
+
+extern "C" int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, int mode, int k, int product,
+                                    double *executed) {
+  mode &= ~ANC_NS_TILE128;
+  if (int rc = check_shape(E, M, N, mode, "anc_ns_product_flops")) return rc;
+  ANC_REQUIRE(executed != nullptr && steps > 0 && k >= 0 && k < steps && product >= 0 && product <= 2,
+              "anc_ns_product_flops: bad arguments");
+  const double m = (double)M, n = (double)N;
+  if (mode == ANC_NS_FP32) {
+    *executed = (double)E * (product == 1 ? 2.0 * m * m * m : 2.0 * m * m * n);
+    return ANC_OK;
+  }
+  const SplitPlan sp = split_plan(M, N, mode, steps);
+  const bool sx = k >= sp.x_from, sfb = k >= sp.fb_from;
+  const double tM = m / BM, tN = n / BN, tile = 2.0 * BM * BN;
+  double ex;
+  if (product == 0)      ex = tM * (tM + 1) / 2 * (sx ? 3 : 1) * tile * n;
+  else if (product == 1) ex = tM * (tM + 1) / 2 * (sfb ? 3 : 1) * tile * m;
+  else                   ex = tM * tN * (1 + (sx ? 1 : 0) + (sfb ? 1 : 0)) * tile * m;
+  *executed = (double)E * ex;
   return ANC_OK;
 }
 
@@ -694,24 +719,26 @@ extern "C" int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partia
 // side by side: each product of each step is one launch over all of them, which keeps the
 // CUs busy where per-batch launches would each end in a partly filled last wave. Same
 // results, bit for bit, as anc_ns_batched_pair on each batch. All dims multiples of 256.
-extern "C" int anc_ns_batched_pair_multi(const anc_ns_problem_t *probs, int32_t n_probs, int steps,
-                                         const float *coef, float eps, int mode, uint64_t stream) {
-  ANC_REQUIRE(probs != nullptr && n_probs >= 1 && n_probs <= kMaxGroups,
-              "anc_ns_batched_pair_multi: 1..%d problems", kMaxGroups);
-  ANC_REQUIRE(mode == ANC_NS_BF16 || mode == ANC_NS_BF16_FAST, "anc_ns_batched_pair_multi: bf16 modes only");
-  ANC_REQUIRE(steps >= 2 && steps <= 64 && coef != nullptr, "anc_ns_batched_pair_multi: steps=%d: 2..64", steps);
+static int pair_multi_impl(const char *who, const anc_ns_problem_t *probs, int32_t n_probs,
+                           const uint64_t *desc_tables, const NsUpdate *upd, int steps, const float *coef,
+                           float eps, int mode, uint64_t stream) {
+  ANC_REQUIRE(probs != nullptr && n_probs >= 1 && n_probs <= kMaxGroups, "%s: 1..%d problems", who, kMaxGroups);
+  ANC_REQUIRE(mode == ANC_NS_BF16 || mode == ANC_NS_BF16_FAST, "%s: bf16 modes only", who);
+  ANC_REQUIRE(steps >= 2 && steps <= 64 && coef != nullptr, "%s: steps=%d: 2..64", who, steps);
   hipStream_t s = anc_stream(stream);
   ChainProb cp[kMaxGroups];
   int order[kMaxGroups];
   for (int q = 0; q < n_probs; ++q) {
     const anc_ns_problem_t &b = probs[q];
-    if (int rc = check_shape(b.E, b.M, b.N, mode, "anc_ns_batched_pair_multi")) return rc;
-    ANC_REQUIRE(b.M % 256 == 0 && b.N % 256 == 0, "anc_ns_batched_pair_multi: dims must be multiples of 256");
-    ANC_REQUIRE(b.Uh != 0 && b.Ul != 0 && ((b.Uh | b.Ul | b.X32_out) & 15) == 0 && b.X32_out != 0,
-                "anc_ns_batched_pair_multi: pointers must be 16-byte aligned and non-null");
+    if (int rc = check_shape(b.E, b.M, b.N, mode, who)) return rc;
+    ANC_REQUIRE(b.M % 256 == 0 && b.N % 256 == 0, "%s: dims must be multiples of 256", who);
+    ANC_REQUIRE(b.Uh != 0 && b.Ul != 0 && ((b.Uh | b.Ul | b.X32_out) & 15) == 0,
+                "%s: pointers must be 16-byte aligned and non-null", who);
+    if (desc_tables == nullptr) ANC_REQUIRE(b.X32_out != 0, "%s: null X32_out", who);
+    else ANC_REQUIRE(desc_tables[q] != 0 && (desc_tables[q] & 7) == 0, "%s: null or misaligned descriptor table", who);
     ANC_REQUIRE(b.fro_partials != 0 && b.n_partials > 0 && b.n_partials < (1 << 30),
-                "anc_ns_batched_pair_multi: need the Frobenius partial sums");
-    ANC_REQUIRE(b.workspace != 0 && (b.workspace & 255) == 0, "anc_ns_batched_pair_multi: workspace must be 256-byte aligned");
+                "%s: need the Frobenius partial sums", who);
+    ANC_REQUIRE(b.workspace != 0 && (b.workspace & 255) == 0, "%s: workspace must be 256-byte aligned", who);
     order[q] = q;
   }
   // longest tiles first: by N (the Gram product's K), then by M
@@ -723,12 +750,35 @@ extern "C" int anc_ns_batched_pair_multi(const anc_ns_problem_t *probs, int32_t 
   for (int q = 0; q < n_probs; ++q) {
     const anc_ns_problem_t &b = probs[order[q]];
     const Plan pl = make_plan(b.workspace, b.E, b.M, b.N, mode, steps);
-    ANC_REQUIRE(b.workspace_bytes >= pl.bytes, "anc_ns_batched_pair_multi: workspace holds %lld bytes, %lld needed",
+    ANC_REQUIRE(b.workspace_bytes >= pl.bytes, "%s: workspace holds %lld bytes, %lld needed", who,
                 (long long)b.workspace_bytes, (long long)pl.bytes);
     { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)b.E), dim3(kThreads), 0, s,
                        (const double *)b.fro_partials, (int)b.n_partials, eps, pl.recip); }
     ANC_LAUNCH_CHECK();
-    cp[q] = ChainProb{pl, (const uint16_t *)b.Uh, (const uint16_t *)b.Ul, 0, pl.recip, (float *)b.X32_out, b.E, b.M, b.N};
+    cp[q] = ChainProb{pl, (const uint16_t *)b.Uh, (const uint16_t *)b.Ul, 0, pl.recip, (float *)b.X32_out, b.E, b.M, b.N,
+                      desc_tables ? (const anc_muon_desc_t *)desc_tables[order[q]] : nullptr};
   }
-  return run_bf16_chain(cp, n_probs, steps, coef, false, s);
+  return run_bf16_chain(cp, n_probs, steps, coef, false, s, upd);
+}
+
+extern "C" int anc_ns_batched_pair_multi(const anc_ns_problem_t *probs, int32_t n_probs, int steps,
+                                         const float *coef, float eps, int mode, uint64_t stream) {
+  return pair_multi_impl("anc_ns_batched_pair_multi", probs, n_probs, nullptr, nullptr, steps, coef, eps, mode, stream);
+}
+
+// The same chain with the Muon weight update applied by the last step's epilogue: problem q's
+// matrix e is the orthogonalised update of the weight desc_tables[q][e] (p32, p16, K, N,
+// transpose, scale_idx and seed are read; p16t must be 0). Same bits in p32 and p16 as the chain
+// followed by anc_muon_update_multi, without the fp32 hand-off in between.
+extern "C" int anc_muon_ns_update_multi(const anc_ns_problem_t *probs, int32_t n_probs,
+                                        const uint64_t *desc_tables, int steps, const float *coef, float eps,
+                                        int mode, const float *lr_scales, int sr, uint32_t seed_base,
+                                        uint64_t ctl, uint64_t stream) {
+  ANC_REQUIRE(desc_tables != nullptr && lr_scales != nullptr, "anc_muon_ns_update_multi: null descriptor tables or lr_scales");
+  NsUpdate u{};
+  for (int k = 0; k < ANC_MUON_MAX_SCALES; ++k) u.lr[k] = lr_scales[k];
+  u.sr = sr ? 1 : 0;
+  u.seed_base = seed_base;
+  u.ctl = (const anc_step_ctl_t *)ctl;
+  return pair_multi_impl("anc_muon_ns_update_multi", probs, n_probs, desc_tables, &u, steps, coef, eps, mode, stream);
 }

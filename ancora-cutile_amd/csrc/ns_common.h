@@ -69,6 +69,9 @@ struct NsGemm {
   const uint16_t *Xh, *Xl;   // (E,M,N) current iterate as a bf16 pair, X = Xh + Xl   BX in
   uint16_t *Yh, *Yl;         // (E,M,N) next iterate as a bf16 pair   BX out, null on the last step
   float *X32;                // (E,M,N) fp32 result                   BX out on the last step, else null
+  const anc_muon_desc_t *upd;  // BX, last step only: if set, matrix e is the Newton-Schulz result of the
+                             // weight upd[e] and the epilogue applies W -= lr*O to it (p32, p16) instead
+                             // of writing X32
   const float *scale;        // (E) or null. The operands are an unnormalised iterate U and the step
                              // acts on X = scale*U: GRAM multiplies its accumulator by scale^2, BX
                              // multiplies the accumulator and the epilogue's X by scale.
@@ -83,6 +86,18 @@ struct NsGemmMulti {
   int n;
   int tiles[kMaxGroups];
   NsGemm g[kMaxGroups];
+  // fused weight update (problems with `upd` set): lr*shape_scale by descriptor scale index,
+  // stochastic-rounding switch and seed, the step's control block (skip flag) or null
+  float lr[ANC_MUON_MAX_SCALES];
+  int sr;
+  uint32_t seed_base;
+  const anc_step_ctl_t *ctl;
+};
+struct NsUpdate {
+  float lr[ANC_MUON_MAX_SCALES];
+  int sr;
+  uint32_t seed_base;
+  const anc_step_ctl_t *ctl;
 };
 
 // Workgroup id -> (problem, tile index inside the problem). The logical tile sequence is cut
@@ -112,4 +127,6 @@ __device__ __forceinline__ void anc_group_tile(const NsGemmMulti &pm, int bid, i
 // therefore the same bits as the 128x128 kernel; used when M and N are multiples of 256.
 int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s);
 // The same for n <= kMaxGroups problems in one launch (ps[k] with batch size Es[k]).
-int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s);
+// `upd` (may be null) carries the scalars of the fused weight update for problems whose `upd` is set.
+int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s,
+                          const NsUpdate *upd = nullptr);

@@ -432,6 +432,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #ifdef ANC_DBG_NOEPI
   if (acc[0][0][0] + acc[3][1][7] != 12345.678f) return;
 #endif
+  if (EPI == EPI_BX && p.upd != nullptr && pm.ctl != nullptr && pm.ctl->skip != 0u) return;   // skipped step
   const int M = p.M, N = p.N;
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
   unsigned char *region = st(wave / WPS) + (wave % WPS) * kStageRegion;
@@ -511,13 +512,52 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     const int rr = lane & 31, hh = lane >> 5;
     const int key = (rr & 7) ^ ((rr >> 3) & 1);
     const bool fp32_out = p.X32 != nullptr;
+    // Fused weight update (last step): the slab is the Newton-Schulz result O of a 32x64 (or,
+    // for a tall weight whose chain ran on its transpose, 64x32) block of the weight W; the
+    // epilogue reads that block of the fp32 master, subtracts lr*O, writes it back together with
+    // its bf16 copy. The master block is requested (8 x 16 bytes per lane) before the wait for
+    // the slab's DMA, so that its latency runs under the wait and the arithmetic.
+    const bool fused = (p.upd != nullptr);
+    float *W32 = nullptr;
+    uint16_t *W16 = nullptr;
+    float wlr = 0.0f;
+    uint32_t wseed = 0;
+    int wN = 0;
+    bool wtr = false;
+    if (fused) {
+      const anc_muon_desc_t &d = p.upd[e];
+      W32 = (float *)d.p32;
+      W16 = (uint16_t *)d.p16;
+      wN = d.N;
+      wtr = d.transpose != 0;
+      wlr = pm.lr[d.scale_idx & (ANC_MUON_MAX_SCALES - 1)];
+      wseed = pm.seed_base + d.seed;
+    }
+    // element offset in W of the 4 values lane-piece pz handles
+    auto w_off = [&](int gi0, int pz) -> int64_t {
+      const int idx = pz * 64 + lane;
+      if (!wtr) return (int64_t)(gi0 + (idx >> 4)) * wN + gj0w + (idx & 15) * 4;
+      return (int64_t)(gj0w + (idx >> 3)) * wN + gi0 + (idx & 7) * 4;
+    };
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi) {
       const int gi0 = gi0w + bi * 32;
+      anc_f32x4 pv[8];
+      if (fused) {
+#pragma unroll
+        for (int pz = 0; pz < 8; ++pz) pv[pz] = anc_ld_stream((const anc_f32x4 *)(W32 + w_off(gi0, pz)));
+      }
       // Wait for this slab's DMA only. Vector memory operations complete in issue order; after
       // the fetch of slab bi this wavefront issued the 8 row stores of slab bi-1 and the fetch
-      // of slab bi+1 (8 DMA); nothing else in this epilogue is a vector memory operation.
-      if (bi == 0 || bi == 3) wait_vm<8>(); else wait_vm<16>();
+      // of slab bi+1 (8 DMA); in the fused update the stores of a slab are 8 (master) + 8 (bf16
+      // copy, if there is one) and the 8 master loads of slab bi are younger too.
+      if (!fused) {
+        if (bi == 0 || bi == 3) wait_vm<8>(); else wait_vm<16>();
+      } else if (W16 != nullptr) {
+        if (bi == 0) wait_vm<16>(); else if (bi == 3) wait_vm<24>(); else wait_vm<32>();
+      } else {
+        if (bi == 0) wait_vm<16>(); else if (bi == 3) wait_vm<16>(); else wait_vm<24>();
+      }
       unsigned char *b = inbuf(bi);
       const float dr = *(const float *)(dvec_lds + (bi * 32 + rr) * 4);
       anc_u32x2 xh[2][4], xl[2][4];
@@ -541,7 +581,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
                           ((r & 1) ? __uint_as_float(wl & 0xFFFF0000u) : __uint_as_float(wl << 16));
           y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
         }
-      if (fp32_out) {
+      if (fp32_out || fused) {
         // fp32 result: [32 rows][16 chunks of 16 B], chunk XOR (row & 15)
 #pragma unroll
         for (int bj = 0; bj < 2; ++bj)
@@ -552,11 +592,48 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           }
         __builtin_amdgcn_s_waitcnt(0xC07F);
         __builtin_amdgcn_wave_barrier();
+        if (!fused) {
 #pragma unroll
-        for (int pz = 0; pz < 8; ++pz) {
-          const int idx = pz * 64 + lane, row = idx >> 4, c = idx & 15;
-          const anc_f32x4 v4 = *(const anc_f32x4 *)(b + row * 256 + ((c ^ (row & 15)) * 16));
-          epi_st((anc_f32x4 *)(p.X32 + mn + (int64_t)(gi0 + row) * N + gj0w + c * 4), v4);
+          for (int pz = 0; pz < 8; ++pz) {
+            const int idx = pz * 64 + lane, row = idx >> 4, c = idx & 15;
+            const anc_f32x4 v4 = *(const anc_f32x4 *)(b + row * 256 + ((c ^ (row & 15)) * 16));
+            epi_st((anc_f32x4 *)(p.X32 + mn + (int64_t)(gi0 + row) * N + gj0w + c * 4), v4);
+          }
+        } else {
+#pragma unroll
+          for (int pz = 0; pz < 8; ++pz) {
+            const int idx = pz * 64 + lane;
+            float o[4];
+            if (!wtr) {
+              const int row = idx >> 4, c = idx & 15;
+              const anc_f32x4 v4 = *(const anc_f32x4 *)(b + row * 256 + ((c ^ (row & 15)) * 16));
+              o[0] = v4.x; o[1] = v4.y; o[2] = v4.z; o[3] = v4.w;
+            } else {
+              // W row = column `col` of the slab, W columns = slab rows 4c .. 4c+3
+              const int col = idx >> 3, c = idx & 7;
+#pragma unroll
+              for (int t4 = 0; t4 < 4; ++t4) {
+                const int row = 4 * c + t4;
+                o[t4] = *(const float *)(b + row * 256 + (((col >> 2) ^ (row & 15)) * 16) + (col & 3) * 4);
+              }
+            }
+            const int64_t we = w_off(gi0, pz);
+            float pp[4] = {pv[pz].x, pv[pz].y, pv[pz].z, pv[pz].w};
+            uint32_t hb[4];
+#pragma unroll
+            for (int k4 = 0; k4 < 4; ++k4) {
+              pp[k4] = pp[k4] - wlr * o[k4];
+              const uint64_t i = (uint64_t)(we + k4);
+              hb[k4] = pm.sr ? anc_bf16_sr_bits(pp[k4], (uint32_t)(i >> 6), (uint32_t)(i & 63u), wseed)
+                             : anc_bf16_rne_bits(pp[k4]);
+            }
+            const anc_f32x4 po = {pp[0], pp[1], pp[2], pp[3]};
+            epi_st((anc_f32x4 *)(W32 + we), po);
+            if (W16 != nullptr) {
+              const anc_u32x2 ho = {(hb[0] & 0xFFFFu) | (hb[1] << 16), (hb[2] & 0xFFFFu) | (hb[3] << 16)};
+              epi_st((anc_u32x2 *)(W16 + we), ho);
+            }
+          }
         }
       } else {
 #pragma unroll
@@ -720,7 +797,8 @@ int launch_sym(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
 
 // Symmetric products run on 256x256 tiles (lower triangle); X = a X + B X runs on 128x256 tiles
 // (the tile counts of the problems are recomputed here).
-int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
+int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s,
+                          const NsUpdate *upd) {
   ANC_REQUIRE(n >= 1 && n <= kMaxGroups, "anc_ns_gemm_big: 1..%d problems per launch", kMaxGroups);
   for (int k = 0; k < n; ++k)
     ANC_REQUIRE(ps[k].M % 256 == 0 && ps[k].N % 256 == 0 && ps[k].K % 32 == 0,
@@ -741,11 +819,19 @@ int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, h
     grid += t;
   }
   ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
+  if (upd != nullptr) {
+    for (int k = 0; k < ANC_MUON_MAX_SCALES; ++k) pm.lr[k] = upd->lr[k];
+    pm.sr = upd->sr;
+    pm.seed_base = upd->seed_base;
+    pm.ctl = upd->ctl;
+  } else {
+    for (int k = 0; k < n; ++k) ANC_REQUIRE(ps[k].upd == nullptr, "anc_ns_gemm_big: fused update without its scalars");
+  }
   hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
 
 int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s) {
-  return anc_ns_gemm_big_multi(epi, &p, &E, 1, s);
+  return anc_ns_gemm_big_multi(epi, &p, &E, 1, s, nullptr);
 }

@@ -117,6 +117,9 @@ class MuonEngine:
         # of workgroups per group). Needs the fused prologue, private buffers per batch and
         # dims that are multiples of 256; other batches run one by one.
         self.grouped = True
+        # Fused update: the epilogue of the chain's last product applies W -= lr*O itself (grouped
+        # path only; a weight with a transposed bf16 copy to refresh keeps the separate kernel).
+        self.fused_update = True
         groups = {}
         scales = []
         for idx, w in enumerate(weights):
@@ -188,13 +191,20 @@ class MuonEngine:
         seed_base = ((self.seed + 1000003 * self.t) & 0xFFFFFFFF) if self.sr else 0
         coef = muon_ns.coef_array(schedule, self.ns)
         together = [b for b in self.batches
-                    if self.grouped and self.fused_prologue and self.concurrent
-                    and b.M % 256 == 0 and b.Nn % 256 == 0]
-        if len(together) < 2:
-            together = []
+                    if self.grouped and self.fused_prologue and b.M % 256 == 0 and b.Nn % 256 == 0]
+        if not self.concurrent and len(self.batches) > 1:
+            # shared packed buffer and workspace: one batch per call, and only if that buys the
+            # fused update
+            per_call = 1
+            if not self.fused_update:
+                together = []
+        else:
+            per_call = 4
+            if len(together) < 2 and not self.fused_update:
+                together = []
         alone = [b for b in self.batches if b not in together]
-        for i0 in range(0, len(together), 4):
-            self._step_grouped(together[i0:i0 + 4], si, ctl, coef, lr_scales, seed_base)
+        for i0 in range(0, len(together), per_call):
+            self._step_grouped(together[i0:i0 + per_call], si, ctl, coef, lr_scales, seed_base)
         forked = self.concurrent and not self.serial and len(alone) > 1
         if forked:
             self._fork.record(si)
@@ -241,6 +251,12 @@ class MuonEngine:
             n_el = b.E * b.M * b.Nn
             probs[k] = _lib.NsProblem(b.U.ptr, b.U.ptr + n_el * 2, b.fro.ptr, b.U.ptr, buf.ptr,
                                       b.total_blocks // b.E, b.E, b.M, b.Nn, buf.nbytes)
+        if self.fused_update and not any(w.get("p16T") is not None for b in group for w in b.weights):
+            tables = (ctypes.c_uint64 * len(group))(*[b.table.ptr for b in group])
+            api.anc_muon_ns_update_multi(probs, len(group), tables, self.ns, coef, 1e-7,
+                                         muon_ns.MODES[self.mode], lr_scales, int(self.sr), seed_base, ctl,
+                                         int(si))
+            return
         api.anc_ns_batched_pair_multi(probs, len(group), self.ns, coef, 1e-7, muon_ns.MODES[self.mode],
                                       int(si))
         for b in group:

@@ -113,6 +113,15 @@ def ns_flops(E, M, N, steps=5, mode="bf16"):
     return ex.value, de.value
 
 
+def ns_product_flops(E, M, N, k, product, steps=5, mode="bf16"):
+    """Executed matrix-core FLOPs of product 0 (A = X X^T), 1 (B = b A + c A A) or 2
+    (X = a X + B X) of iteration k of a chain call."""
+    ex = ctypes.c_double(0)
+    api.anc_ns_product_flops(int(E), int(M), int(N), int(steps), MODES[mode], int(k), int(product),
+                             ctypes.byref(ex))
+    return ex.value
+
+
 def ns_batched(X32, E, M, N, si, steps=5, eps=1e-7, schedule=_KELLER, mode="bf16", workspace=None):
     """Native driver: X32 is a DevBuf of E packed (M,N) fp32 matrices, M <= N, both multiples of
     128; overwritten with the orthogonalised result."""

@@ -218,7 +218,7 @@ def main():
         return side_workload(args)
     from ancora_cutile_amd import HybridOptimizer, DevBuf, PE_SCHEDULE, _lib
     from ancora_cutile_amd.hybrid import resident_is_muon
-    from ancora_cutile_amd.muon_ns import ns_flops
+    from ancora_cutile_amd.muon_ns import ns_flops, ns_product_flops
     from ancora_cutile_amd.shapes import qwen3_shapes, moe_shapes
 
     _lib.init(0)
@@ -296,18 +296,30 @@ def main():
     kind_ms = {k: v[0] / prof_steps for k, v in prof.items() if v[1]}
     launches = {k: v[1] // prof_steps for k, v in prof.items() if v[1]}
 
-    executed = dense = 0.0
+    executed = dense = last_bx = 0.0
     for b in opt.muon.engine.batches:
         ex, de = ns_flops(b.E, b.M, b.Nn, 5, "bf16")
         executed += ex
         dense += de
-    gemm_ms = sum(kind_ms.get(k, 0.0) for k in ("ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx"))
-    gemm_launches = sum(launches.get(k, 0) for k in ("ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx"))
+        last_bx += ns_product_flops(b.E, b.M, b.Nn, 4, 2, 5, "bf16")
+    # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
+    # last X = a X + B X) also reads and writes the weights
+    gemm_kinds = ("ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx", "ns_gemm_bx_update")
+    gemm_ms = sum(kind_ms.get(k, 0.0) for k in gemm_kinds)
+    gemm_launches = sum(launches.get(k, 0) for k in gemm_kinds)
     achieved = executed / (gemm_ms * 1e-3) / 1e12 if gemm_ms else 0.0
+    pure_ms = gemm_ms - kind_ms.get("ns_gemm_bx_update", 0.0)
+    pure_launches = gemm_launches - launches.get("ns_gemm_bx_update", 0)
+    pure_flops = executed - (last_bx if "ns_gemm_bx_update" in kind_ms else 0.0)
+    pure_achieved = pure_flops / (pure_ms * 1e-3) / 1e12 if pure_ms else 0.0
     adamw_gbps = 28.0 * n_adam / (kind_ms["adamw"] * 1e-3) / 1e9
     gn_gbps = 2.0 * n_params / (kind_ms["gradnorm_partials"] * 1e-3) / 1e9
-    elem_ms = kind_ms["muon_momentum"] + kind_ms["muon_update"]
-    elem_gbps = 24.0 * n_muon / (elem_ms * 1e-3) / 1e9
+    # With the fused update the last X = a X + B X launch of the chain applies W -= lr*O itself:
+    # no update kernel exists and its traffic (10 B per parameter) is inside that GEMM launch.
+    upd_fused = "muon_update" not in kind_ms
+    elem_ms = kind_ms["muon_momentum"] + kind_ms.get("muon_update", 0.0)
+    elem_bytes = 12.0 if upd_fused else 24.0
+    elem_gbps = elem_bytes * n_muon / (elem_ms * 1e-3) / 1e9
 
     # HBM bytes per k_ns_gemm_big launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE on this
     # same workload (two counter runs scaled by the copy kernel; summary under profiles/)
@@ -332,8 +344,12 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
                      "kernel": "k_ns_gemm_big (gram, bmat, bx launches of the Newton-Schulz chain)",
-                     "timed": "HIP events around each launch, chains serialised on one stream",
+                     "timed": "HIP events around each launch, chains serialised on one stream"
+                              + ("; the last of the 15 launches also carries the fused weight update" if upd_fused else ""),
                      "launches_per_step": gemm_launches,
+                     "without_fused_update_launch": {"launches": pure_launches, "achieved": round(pure_achieved, 1),
+                                                     "frac": round(pure_achieved / PEAK_BF16_TFLOPS, 4),
+                                                     "avg_launch_ms": round(pure_ms / max(1, pure_launches), 4)},
                      "avg_launch_ms": round(gemm_ms / max(1, gemm_launches), 4),
                      "executed_tflop_per_step": round(executed / 1e12, 3),
                      "dense_tflop_per_step": round(dense / 1e12, 3)},
@@ -344,8 +360,10 @@ def main():
                          "frac": round(gn_gbps / PEAK_HBM_GBPS, 4), "bytes_per_elem": 2,
                          "ms": round(kind_ms["gradnorm_partials"], 4)},
         "muon_elementwise_hbm": {"achieved": round(elem_gbps, 1), "unit": "GB/s",
-                                 "frac": round(elem_gbps / PEAK_HBM_GBPS, 4), "bytes_per_param": 24,
-                                 "ms": round(elem_ms, 4)},
+                                 "frac": round(elem_gbps / PEAK_HBM_GBPS, 4), "bytes_per_param": int(elem_bytes),
+                                 "ms": round(elem_ms, 4),
+                                 "kernels": "momentum; the update runs in the epilogue of the chain's last GEMM"
+                                 if upd_fused else "momentum + update"},
         "ns_mfma_util_pct": round(100 * achieved / PEAK_BF16_TFLOPS, 2),
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kind_ms.items()},
         "event_ms_per_step": round(ev_ms, 3), "wall_ms_per_step": round(wall_ms, 3),

@@ -109,7 +109,8 @@ int anc_copy_kernel(uint64_t dst, uint64_t src, int64_t n_bytes, uint64_t stream
 #define ANC_PROF_NS_GEMM_F32 10   /* any GEMM of the fp32 validation chain        */
 #define ANC_PROF_MISC        11   /* casts, conversions, transposes, fill         */
 #define ANC_PROF_COPY        12
-#define ANC_PROF_KINDS       13
+#define ANC_PROF_NS_BX_UPD   13   /* X = a X + B X whose epilogue applies the weight update */
+#define ANC_PROF_KINDS       14
 int anc_profile_enable(int on);
 int anc_profile_read(float *ms /* [ANC_PROF_KINDS] */, int64_t *launches /* [ANC_PROF_KINDS] */);
 
@@ -365,11 +366,29 @@ typedef struct {
 int anc_ns_batched_pair_multi(const anc_ns_problem_t *probs, int32_t n_probs, int steps,
                               const float *coef, float eps, int mode, uint64_t stream);
 
+/* anc_ns_batched_pair_multi followed by the Muon weight update of every matrix, the update
+ * applied by the epilogue of the chain's last product instead of by a kernel of its own:
+ * W -= lr_scales[scale_idx] * O, bf16 copy by RNE or stochastic rounding (`_muon_update_cast[_t]`,
+ * ancora/kernels/muon_ns.py:189-242, launched after the chain at ancora/optim/muon.py:272-277).
+ * desc_tables[q] is a device array of problems[q].E anc_muon_desc_t, entry e describing the weight
+ * whose orthogonalised update is matrix e of the batch (fields read: p32, p16 (may be 0), K, N,
+ * transpose, scale_idx, seed; p16t must be 0). X32_out of the problems is not used. Results in
+ * p32 and p16 are bit-identical to the unfused sequence; the fp32 hand-off (8 bytes per parameter
+ * of HBM traffic) disappears. ctl: the step's control block or 0 (skip flag honoured). */
+int anc_muon_ns_update_multi(const anc_ns_problem_t *problems, int32_t n_problems,
+                             const uint64_t *desc_tables, int steps, const float *coef, float eps,
+                             int mode, const float *lr_scales /* [ANC_MUON_MAX_SCALES] */, int sr,
+                             uint32_t seed_base, uint64_t ctl, uint64_t stream);
+
 /* Matrix-core FLOPs of one anc_ns_batched call: `executed` counts the tiles and terms the
  * kernels really multiply (lower-triangle tiles of the symmetric products, residual terms),
  * `dense` is steps*(4 M^2 N + 2 M^3) per matrix. Roofline figures use `executed`. */
 int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
                  double *executed, double *dense);
+/* Executed matrix-core work of one product of one iteration of that chain: iteration k in
+ * 0..steps-1, product 0 (A = X X^T), 1 (B = b A + c A A) or 2 (X = a X + B X). */
+int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, int mode, int k, int product,
+                         double *executed);
 
 /* Diagnostics, no reference counterpart: rate of the bf16 matrix instruction on register
  * operands while the same wavefronts issue `nread` LDS fragment reads and `ndma` LDS-DMA loads

@@ -190,3 +190,59 @@ def test_checkpoint_resume_is_bitwise(gpu, tmp_path):
     for k in sa:
         assert np.atleast_1d(sa[k]).tobytes() == np.atleast_1d(sb[k]).tobytes(), k
     a.free(); b.free()
+
+
+@pytest.mark.parametrize("sr", [False, True])
+def test_fused_update_equals_separate_update_kernel(gpu, sr):
+    """The chain whose last epilogue applies W -= lr*O gives the bits of the chain followed by the
+    update kernel: square, wide and tall (transposed) weights, with and without a bf16 copy,
+    RNE and stochastic rounding, two steps, and a skipped step leaves everything untouched."""
+    from ancora_cutile_amd import BatchedProjMuon, DevBuf, StepGuard, PE_SCHEDULE as PE
+    rng = np.random.default_rng(21)
+    shapes = [(256, 256), (256, 512), (512, 256), (256, 256), (768, 256), (256, 512), (512, 256)]
+    W0 = [(0.02 * rng.standard_normal(s)).astype(np.float32) for s in shapes]
+    G = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+
+    def run(fused, skip_second=False):
+        ws = [dict(buf=DevBuf.zeros(s, np.float32), p32=DevBuf(w),
+                   p16=None if i == 3 else DevBuf.zeros(s, np.uint16),
+                   G=DevBuf(g), K=s[0], N=s[1], lid=i) for i, (s, w, g) in enumerate(zip(shapes, W0, G))]
+        opt = BatchedProjMuon(ws, chunk=None, sr=sr, seed=5)
+        opt.engine.fused_update = fused
+        guard = StepGuard(1e9)
+        grads = [w["G"] for w in ws]
+        for t in range(2):
+            if skip_second and t == 1:
+                bad = G[0].copy(); bad[3, 7] = np.inf
+                ws[0]["G"].upload(bad)
+            guard.compute(grads, 0)
+            opt.step(0, lr=0.02, schedule=PE, guard=guard)
+        out = [(w["p32"].to_numpy(), None if w["p16"] is None else w["p16"].to_numpy(), w["buf"].to_numpy())
+               for w in ws]
+        opt.free(); guard.free()
+        for w in ws:
+            for k in ("buf", "p32", "p16", "G"):
+                if w[k] is not None:
+                    w[k].free()
+        return out
+
+    for skip in (False, True):
+        a, b = run(True, skip), run(False, skip)
+        for x, y in zip(a, b):
+            for u, v in zip(x, y):
+                assert (u is None and v is None) or bits_equal(u, v)
+    one = run(True, True)
+    # the skipped second step changed nothing: equal to a single step
+    ws1 = None
+    from ancora_cutile_amd import BatchedProjMuon as BPM
+    ws = [dict(buf=DevBuf.zeros(s, np.float32), p32=DevBuf(w), p16=None if i == 3 else DevBuf.zeros(s, np.uint16),
+               G=DevBuf(g), K=s[0], N=s[1], lid=i) for i, (s, w, g) in enumerate(zip(shapes, W0, G))]
+    opt = BPM(ws, chunk=None, sr=sr, seed=5)
+    opt.step(0, lr=0.02, schedule=PE)
+    for w, o in zip(ws, one):
+        assert bits_equal(w["p32"].to_numpy(), o[0])
+    opt.free()
+    for w in ws:
+        for k in ("buf", "p32", "p16", "G"):
+            if w[k] is not None:
+                w[k].free()
