@@ -210,7 +210,9 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("" ::: "memory");
 }
 
-template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS>
+// FUSED (X = a X + B X only): the instantiation whose epilogue applies the weight update; kept
+// apart so that its extra registers do not weigh on the other launches.
+template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS, bool FUSED = false>
 __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemmMulti pm) {
   constexpr int NWN = TN / 64, NWAVES = (TM / 128) * NWN;
   constexpr int ROWB = TK * 2;                      // bytes per LDS row
@@ -432,7 +434,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #ifdef ANC_DBG_NOEPI
   if (acc[0][0][0] + acc[3][1][7] != 12345.678f) return;
 #endif
-  if (EPI == EPI_BX && p.upd != nullptr && pm.ctl != nullptr && pm.ctl->skip != 0u) return;   // skipped step
+  if (FUSED && pm.ctl != nullptr && pm.ctl->skip != 0u) return;   // skipped step
   const int M = p.M, N = p.N;
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
   unsigned char *region = st(wave / WPS) + (wave % WPS) * kStageRegion;
@@ -517,7 +519,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     // epilogue reads that block of the fp32 master, subtracts lr*O, writes it back together with
     // its bf16 copy. The master block is requested (8 x 16 bytes per lane) before the wait for
     // the slab's DMA, so that its latency runs under the wait and the arithmetic.
-    const bool fused = (p.upd != nullptr);
+    constexpr bool fused = FUSED;
     float *W32 = nullptr;
     uint16_t *W16 = nullptr;
     float wlr = 0.0f;
@@ -827,7 +829,13 @@ int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, h
   } else {
     for (int k = 0; k < n; ++k) ANC_REQUIRE(ps[k].upd == nullptr, "anc_ns_gemm_big: fused update without its scalars");
   }
-  hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+  bool any_upd = false, all_upd = true;
+  for (int k = 0; k < n; ++k) { any_upd = any_upd || ps[k].upd != nullptr; all_upd = all_upd && ps[k].upd != nullptr; }
+  ANC_REQUIRE(any_upd == all_upd, "anc_ns_gemm_big: the fused update applies to every problem of a launch or to none");
+  if (any_upd)
+    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, true>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+  else
+    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
