@@ -39,6 +39,39 @@ def test_struct_sizes_match_header():
     assert ctypes.sizeof(_lib.DeviceInfo) == 24 + 16 + 128
 
 
+def test_header_is_plain_c_and_layouts_match_ctypes(tmp_path):
+    """include/anc_optim.h compiles as C99 with gcc (no C++ in the boundary) and every struct has
+    the size and the field offsets the ctypes mirror assumes."""
+    import shutil
+    import subprocess
+    from ancora_cutile_amd import _lib
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    pairs = [("anc_step_ctl_t", _lib.StepCtl), ("anc_adamw_hyper_t", _lib.AdamWHyper),
+             ("anc_adamw_desc_t", _lib.AdamWDesc), ("anc_gn_desc_t", _lib.GnDesc),
+             ("anc_muon_desc_t", _lib.MuonDesc), ("anc_ns_problem_t", _lib.NsProblem),
+             ("anc_device_info_t", _lib.DeviceInfo)]
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "anc_optim.h"', 'int main(void) {']
+    for cname, ct in pairs:
+        lines.append(f'  printf("{cname} %zu", sizeof({cname}));')
+        for fname, _ in ct._fields_:
+            lines.append(f'  printf(" %zu", offsetof({cname}, {fname}));')
+        lines.append('  printf("\\n");')
+    lines += ['  return 0;', '}']
+    src = tmp_path / "abi.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "abi"
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    for (cname, ct), line in zip(pairs, out):
+        vals = line.split()
+        assert vals[0] == cname and int(vals[1]) == ctypes.sizeof(ct), line
+        for (fname, _), off in zip(ct._fields_, vals[2:]):
+            assert int(off) == getattr(ct, fname).offset, (cname, fname)
+
+
 def test_no_gpu_means_error_not_fallback():
     """Without a GPU the product path must raise; it never computes on the CPU."""
     from ancora_cutile_amd import _lib
