@@ -203,11 +203,15 @@ def test_fused_update_equals_separate_update_kernel(gpu, sr):
     W0 = [(0.02 * rng.standard_normal(s)).astype(np.float32) for s in shapes]
     G = [rng.standard_normal(s).astype(np.float32) for s in shapes]
 
-    def run(fused, skip_second=False):
+    def run(fused, skip_second=False, shared=False):
         ws = [dict(buf=DevBuf.zeros(s, np.float32), p32=DevBuf(w),
                    p16=None if i == 3 else DevBuf.zeros(s, np.uint16),
                    G=DevBuf(g), K=s[0], N=s[1], lid=i) for i, (s, w, g) in enumerate(zip(shapes, W0, G))]
         opt = BatchedProjMuon(ws, chunk=None, sr=sr, seed=5)
+        if shared:       # one packed buffer and workspace for all batches: one batch per call
+            from ancora_cutile_amd.muon import MuonEngine
+            opt.engine.free()
+            opt.engine = MuonEngine(ws, 0.95, 5, True, None, None, "bf16", sr, 5, concurrent=False)
         opt.engine.fused_update = fused
         guard = StepGuard(1e9)
         grads = [w["G"] for w in ws]
@@ -231,9 +235,12 @@ def test_fused_update_equals_separate_update_kernel(gpu, sr):
         for x, y in zip(a, b):
             for u, v in zip(x, y):
                 assert (u is None and v is None) or bits_equal(u, v)
+    a, b = run(True, shared=True), run(False)
+    for x, y in zip(a, b):
+        for u, v in zip(x, y):
+            assert (u is None and v is None) or bits_equal(u, v)
     one = run(True, True)
     # the skipped second step changed nothing: equal to a single step
-    ws1 = None
     from ancora_cutile_amd import BatchedProjMuon as BPM
     ws = [dict(buf=DevBuf.zeros(s, np.float32), p32=DevBuf(w), p16=None if i == 3 else DevBuf.zeros(s, np.uint16),
                G=DevBuf(g), K=s[0], N=s[1], lid=i) for i, (s, w, g) in enumerate(zip(shapes, W0, G))]
