@@ -15,3 +15,4 @@ from .muon import (Muon, DeviceMuon, MuonScratch, ResidentMuon, BatchedProjMuon,
 from .moe import ExpertMuonScratch, ExpertOptimizer                          # noqa: F401
 from .hybrid import HybridOptimizer, default_is_muon, resident_is_muon       # noqa: F401
 from .quant import Mxfp8WeightCache, quant_mxfp8_w                          # noqa: F401
+from .grads import gemm_dW, transpose_acts, DwWorkspace                       # noqa: F401

@@ -66,6 +66,13 @@ class NsProblem(C.Structure):
                 ("n_partials", i64), ("E", i64), ("M", i64), ("N", i64), ("workspace_bytes", i64)]
 
 
+class DwProblem(C.Structure):
+    """anc_dw_problem_t: one weight of the weight-gradient GEMM call."""
+    _fields_ = [("xT", u64), ("dy", u64), ("dW", u64), ("g16", u64), ("workspace", u64),
+                ("T", i64), ("K", i64), ("N", i64), ("workspace_bytes", i64),
+                ("accumulate", i32), ("reserved", i32)]
+
+
 # name -> (restype, argtypes); restype None means "int status, checked".
 _PROTOS = {
     "anc_last_error": (C.c_char_p, []),
@@ -113,6 +120,9 @@ _PROTOS = {
                                      u64]),
     "anc_transpose_bf16": (None, [u64, u64, i64, i64, i64, u64]),
     "anc_quant_mxfp8_w": (None, [u64, u64, u64, i64, i64, i64, C.c_int, u64]),
+    "anc_gemm_dw_workspace_bytes": (i64, [i64, i64, i64]),
+    "anc_gemm_dw_multi": (None, [C.POINTER(DwProblem), i32, u64]),
+    "anc_gemm_dw_info": (None, [i64, i64, i64, C.POINTER(C.c_double), C.POINTER(i32)]),
     "anc_ns_workspace_bytes": (i64, [i64, i64, i64, C.c_int]),
     "anc_ns_batched": (None, [u64, i64, i64, i64, C.c_int, C.POINTER(f32), f32, C.c_int, u64, i64,
                               u64]),
@@ -207,7 +217,7 @@ def stream_sync(stream=0):
 
 PROF_KINDS = ("adamw", "gradnorm_partials", "gradnorm_finalize", "muon_momentum", "muon_update",
               "ns_fro", "ns_prep", "ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx", "ns_gemm_f32",
-              "misc", "copy", "ns_gemm_bx_update")
+              "misc", "copy", "ns_gemm_bx_update", "dw_gemm", "dw_reduce")
 
 
 def profile_enable(on=True):

@@ -1,0 +1,144 @@
+// Weight-gradient GEMM dW (+)= x^T dy: the producer of the gradients the optimizer step reads.
+//
+// Replaces `_gemm_dW` / `_gemm_dW_acc` (ancora/kernels/fused.py:190-219, launched per weight at
+// ancora/model/resident_train.py:285-287): x (T, K) and dy (T, N) bf16, fp32 accumulation over the
+// T tokens, fp32 result, optionally added onto the existing dW (gradient accumulation in place).
+// Here the product runs on the Newton-Schulz chain's X = a X + B X K loop (128x256 tiles, bf16
+// MFMA, LDS-DMA stage ring): A = x^T (K, T) row-major -- the caller transposes the activations
+// once per group of weights that share them (anc_transpose_bf16) -- and B = dy as it lies.
+//
+// A single weight is 50-200 tiles, far fewer than the 512 a launch needs to fill 256 CUs, and the
+// backward pass produces one layer's gradients at a time. So the token axis is cut into S
+// segments: segment s of every tile is its own workgroup and leaves an fp32 partial tile in the
+// workspace; a second, HBM-bound kernel adds the S partials in ascending order (and the old dW
+// when accumulating) and can emit the bf16 copy the optimizer step reads. S depends on the
+// problem's shape alone, so the result's bits do not depend on what shares the launch: one
+// workgroup owns one (tile, segment) and its whole K loop, K tiles in ascending order, no atomics.
+#include "ns_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// Segments of the token axis: the smallest power of two that gives the problem at least 256
+// workgroups (one per CU), with at least 256 tokens per segment and segment length a multiple
+// of 32.
+int dw_segments(int64_t T, int64_t K, int64_t N) {
+  const int64_t tiles = (K / 128) * (N / 256);
+  int s = 1;
+  while (tiles * s < 256 && T % (2 * s * 32) == 0 && T / (2 * s) >= 256) s *= 2;
+  return s;
+}
+
+struct DwReduce {
+  const float *part;     // (S, n) partials
+  float *dW;             // (n)
+  uint16_t *g16;         // (n) or null
+  int64_t n;
+  int S;
+  int accumulate;
+};
+struct DwReduceMulti {
+  int count;
+  int64_t blk0[kMaxGroups + 1];
+  DwReduce r[kMaxGroups];
+};
+
+__global__ void __launch_bounds__(kThreads) k_dw_reduce(DwReduceMulti m) {
+  int q = 0;
+  while (q + 1 < m.count && (int64_t)blockIdx.x >= m.blk0[q + 1]) ++q;
+  const DwReduce &r = m.r[q];
+  const int64_t i = (((int64_t)blockIdx.x - m.blk0[q]) * kThreads + threadIdx.x) * 4;
+  if (i >= r.n) return;
+  anc_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (r.accumulate) acc = anc_ld_stream((const anc_f32x4 *)(r.dW + i));
+  for (int s = 0; s < r.S; ++s) {
+    const anc_f32x4 v = anc_ld_stream((const anc_f32x4 *)(r.part + (int64_t)s * r.n + i));
+    acc.x = acc.x + v.x; acc.y = acc.y + v.y; acc.z = acc.z + v.z; acc.w = acc.w + v.w;
+  }
+  anc_st_stream((anc_f32x4 *)(r.dW + i), acc);
+  if (r.g16 != nullptr) {
+    const anc_u32x2 h = {anc_bf16_rne_bits(acc.x) | (anc_bf16_rne_bits(acc.y) << 16),
+                         anc_bf16_rne_bits(acc.z) | (anc_bf16_rne_bits(acc.w) << 16)};
+    anc_st_stream((anc_u32x2 *)(r.g16 + i), h);
+  }
+}
+
+int check_dw(const anc_dw_problem_t &b, const char *who) {
+  ANC_REQUIRE(b.T > 0 && b.K > 0 && b.N > 0 && b.T % 32 == 0 && b.K % 128 == 0 && b.N % 256 == 0,
+              "%s: needs T %% 32 == 0, K %% 128 == 0, N %% 256 == 0 (T=%lld K=%lld N=%lld)", who,
+              (long long)b.T, (long long)b.K, (long long)b.N);
+  ANC_REQUIRE(b.T < (1ll << 31) && b.K < (1ll << 24) && b.N < (1ll << 24), "%s: dimension too large", who);
+  return ANC_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t anc_gemm_dw_workspace_bytes(int64_t T, int64_t K, int64_t N) {
+  anc_dw_problem_t b{};
+  b.T = T; b.K = K; b.N = N;
+  if (check_dw(b, "anc_gemm_dw_workspace_bytes")) return -1;
+  return (int64_t)dw_segments(T, K, N) * K * N * 4;
+}
+
+extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs, uint64_t stream) {
+  ANC_REQUIRE(probs != nullptr && n_probs >= 1 && n_probs <= kMaxGroups, "anc_gemm_dw_multi: 1..%d problems",
+              kMaxGroups);
+  hipStream_t s = anc_stream(stream);
+  NsGemm g[kMaxGroups];
+  int64_t Es[kMaxGroups];
+  DwReduceMulti rm{};
+  rm.count = n_probs;
+  int64_t blocks = 0;
+  for (int q = 0; q < n_probs; ++q) {
+    const anc_dw_problem_t &b = probs[q];
+    if (int rc = check_dw(b, "anc_gemm_dw_multi")) return rc;
+    ANC_REQUIRE(b.xT != 0 && b.dy != 0 && b.dW != 0 && b.workspace != 0 &&
+                ((b.xT | b.dy | b.dW | b.workspace) & 15) == 0 && (b.g16 & 7) == 0,
+                "anc_gemm_dw_multi: null or misaligned pointer");
+    const int S = dw_segments(b.T, b.K, b.N);
+    ANC_REQUIRE(b.workspace_bytes >= (int64_t)S * b.K * b.N * 4, "anc_gemm_dw_multi: workspace holds %lld bytes, %lld needed",
+                (long long)b.workspace_bytes, (long long)S * b.K * b.N * 4);
+    const int64_t seg = b.T / S;
+    NsGemm p{};
+    p.A[0] = (const uint16_t *)b.xT;
+    p.B[0] = (const uint16_t *)b.dy;
+    p.nterms = 1;
+    p.K = (int)seg;
+    p.ldA = (int)b.T;
+    p.strideA = seg;                 // segment e starts seg elements further along every row of x^T
+    p.strideB = seg * b.N;           // and seg rows further down dy
+    p.M = (int)b.K;
+    p.N = (int)b.N;
+    p.X32 = (float *)b.workspace;    // partial e at e * K * N
+    g[q] = p;
+    Es[q] = S;
+    rm.r[q] = DwReduce{(const float *)b.workspace, (float *)b.dW, (uint16_t *)b.g16, b.K * b.N, S, b.accumulate ? 1 : 0};
+    rm.blk0[q] = blocks;
+    blocks += (b.K * b.N / 4 + kThreads - 1) / kThreads;
+  }
+  rm.blk0[n_probs] = blocks;
+  ANC_REQUIRE(blocks < (1ll << 31), "anc_gemm_dw_multi: too large");
+  {
+    AncProfScope prof(ANC_PROF_DW_GEMM, s);
+    if (int rc = anc_ns_gemm_big_plain(g, Es, n_probs, s)) return rc;
+  }
+  {
+    AncProfScope prof(ANC_PROF_DW_REDUCE, s);
+    hipLaunchKernelGGL(k_dw_reduce, dim3((unsigned)blocks), dim3(kThreads), 0, s, rm);
+  }
+  ANC_LAUNCH_CHECK();
+  return ANC_OK;
+}
+
+// Executed = dense FLOPs of one problem (every tile is multiplied in full) and the number of
+// token segments it is cut into.
+extern "C" int anc_gemm_dw_info(int64_t T, int64_t K, int64_t N, double *flops, int32_t *segments) {
+  anc_dw_problem_t b{};
+  b.T = T; b.K = K; b.N = N;
+  if (int rc = check_dw(b, "anc_gemm_dw_info")) return rc;
+  ANC_REQUIRE(flops != nullptr && segments != nullptr, "anc_gemm_dw_info: null output");
+  *flops = 2.0 * (double)T * (double)K * (double)N;
+  *segments = dw_segments(T, K, N);
+  return ANC_OK;
+}

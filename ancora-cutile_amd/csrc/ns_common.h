@@ -55,6 +55,8 @@ struct NsGemm {
                              // ("NT" product); BX: the iterate itself, (K, N) row-major, ld = N
   int nterms;
   int K;
+  int ldA;                   // elements between consecutive rows of A; 0 means K (only the plain
+                             // product sets it: its A is a K-range of a longer row)
   int64_t strideA, strideB;  // elements between consecutive matrices
   int tiles_m, tiles_n;
   int lower;                 // symmetric output: tiles with tn <= tm only, mirrored
@@ -130,3 +132,5 @@ int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s);
 // `upd` (may be null) carries the scalars of the fused weight update for problems whose `upd` is set.
 int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s,
                           const NsUpdate *upd = nullptr);
+// Bare fp32 products C[e] = A[e] B[e] on the same K loop (ns_gemm_big.hip).
+int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s);

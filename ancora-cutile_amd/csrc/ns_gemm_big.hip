@@ -210,9 +210,12 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("" ::: "memory");
 }
 
-// FUSED (X = a X + B X only): the instantiation whose epilogue applies the weight update; kept
-// apart so that its extra registers do not weigh on the other launches.
-template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS, bool FUSED = false>
+// VAR (X = a X + B X only) selects a variant of the epilogue as its own instantiation, so that
+// the extra registers and branches do not weigh on the other launches: VAR_UPDATE applies the
+// weight update; VAR_PLAIN is the bare product C = A B written as fp32 (no iterate at the output
+// position, no row scaling), which the weight-gradient GEMM uses.
+enum { VAR_NONE = 0, VAR_UPDATE = 1, VAR_PLAIN = 2 };
+template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS, int VAR = VAR_NONE>
 __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemmMulti pm) {
   constexpr int NWN = TN / 64, NWAVES = (TM / 128) * NWN;
   constexpr int ROWB = TK * 2;                      // bytes per LDS row
@@ -278,11 +281,12 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   //      the swizzle: 128-byte rows use chunk ^ ((row>>1)&7), which alternates with the parity
   //      of the instruction index (RPI = 8); 64-byte rows use chunk ^ ((row>>2)&3), the same
   //      for every instruction (RPI = 16).
+  const int ldA = p.ldA > 0 ? p.ldA : K;
   const int lrow = lane / CPR, pchunk = lane % CPR;
   const int key0 = (TK == 64) ? (lrow >> 1) : ((lrow >> 2) & 3);
-  const uint32_t voff0 = (uint32_t)(lrow * K * 2 + ((pchunk ^ key0) * 16));
-  const uint32_t voff1 = (uint32_t)(lrow * K * 2 + ((pchunk ^ key0 ^ (TK == 64 ? 4 : 0)) * 16));
-  const int64_t ubaseA = ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * (IA * RPI)) * K) * 2;   // bytes
+  const uint32_t voff0 = (uint32_t)(lrow * ldA * 2 + ((pchunk ^ key0) * 16));
+  const uint32_t voff1 = (uint32_t)(lrow * ldA * 2 + ((pchunk ^ key0 ^ (TK == 64 ? 4 : 0)) * 16));
+  const int64_t ubaseA = ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * (IA * RPI)) * ldA) * 2;   // bytes
   const int64_t ubaseB = ((int64_t)e * p.strideB + (int64_t)(tn * TN + wave * (IB * RPI)) * K) * 2;
   // (k, n) B tile: TK rows of TN*2 = 512 bytes, two rows per DMA instruction; lane -> (row
   // lane/32, physical chunk lane%32); the chunk index is XORed with 4*(row&3), so that the 4
@@ -311,7 +315,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // DMA instruction i of a stage (0 .. IPS-1: the A tile's IA, then the B tile's IB)
   auto issue_piece = [&](int i, unsigned char *stage) {
     if (i < IA) {
-      const int64_t ro = (int64_t)(i * RPI) * K * 2;
+      const int64_t ro = (int64_t)(i * RPI) * ldA * 2;
       const uint32_t vo = (i & 1) ? voff1 : voff0;
       dma16(curA + ro + vo, lds_addr(stage + (wave * IA + i) * 1024));
     } else {
@@ -434,7 +438,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #ifdef ANC_DBG_NOEPI
   if (acc[0][0][0] + acc[3][1][7] != 12345.678f) return;
 #endif
-  if (FUSED && pm.ctl != nullptr && pm.ctl->skip != 0u) return;   // skipped step
+  if (VAR == VAR_UPDATE && pm.ctl != nullptr && pm.ctl->skip != 0u) return;   // skipped step
   const int M = p.M, N = p.N;
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
   unsigned char *region = st(wave / WPS) + (wave % WPS) * kStageRegion;
@@ -495,7 +499,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     fetch_a32(1);
   }
   unsigned char *dvec_lds = aux_w;
-  if (EPI == EPI_BX) {
+  if (EPI == EPI_BX && VAR != VAR_PLAIN) {
     asm volatile("" : "+v"(sc));      // the scale has arrived before the first DMA is issued
     // dB of the tile's 128 rows, one private copy per wavefront (lanes 32..63 repeat lanes 0..31),
     // fetched first: any ordinary load issued after the slab fetches would, completing in
@@ -519,7 +523,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     // epilogue reads that block of the fp32 master, subtracts lr*O, writes it back together with
     // its bf16 copy. The master block is requested (8 x 16 bytes per lane) before the wait for
     // the slab's DMA, so that its latency runs under the wait and the arithmetic.
-    constexpr bool fused = FUSED;
+    constexpr bool fused = (VAR == VAR_UPDATE);
+    constexpr bool plain = (VAR == VAR_PLAIN);
     float *W32 = nullptr;
     uint16_t *W16 = nullptr;
     float wlr = 0.0f;
@@ -553,7 +558,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       // the fetch of slab bi this wavefront issued the 8 row stores of slab bi-1 and the fetch
       // of slab bi+1 (8 DMA); in the fused update the stores of a slab are 8 (master) + 8 (bf16
       // copy, if there is one) and the 8 master loads of slab bi are younger too.
-      if (!fused) {
+      if (plain) {
+        // no inputs: nothing to wait for
+      } else if (!fused) {
         if (bi == 0 || bi == 3) wait_vm<8>(); else wait_vm<16>();
       } else if (W16 != nullptr) {
         if (bi == 0) wait_vm<16>(); else if (bi == 3) wait_vm<24>(); else wait_vm<32>();
@@ -561,29 +568,36 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         if (bi == 0) wait_vm<16>(); else if (bi == 3) wait_vm<16>(); else wait_vm<24>();
       }
       unsigned char *b = inbuf(bi);
-      const float dr = *(const float *)(dvec_lds + (bi * 32 + rr) * 4);
-      anc_u32x2 xh[2][4], xl[2][4];
-#pragma unroll
-      for (int bj = 0; bj < 2; ++bj)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int off = rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8;
-          xh[bj][q] = *(const anc_u32x2 *)(b + off);
-          xl[bj][q] = *(const anc_u32x2 *)(b + 4096 + off);
-        }
       float y[2][16];
-      const float cf = p.ca + dr;
+      if (plain) {
 #pragma unroll
-      for (int bj = 0; bj < 2; ++bj)
+        for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const uint32_t wh = (r & 2) ? xh[bj][r >> 2].y : xh[bj][r >> 2].x;
-          const uint32_t wl = (r & 2) ? xl[bj][r >> 2].y : xl[bj][r >> 2].x;
-          const float x = ((r & 1) ? __uint_as_float(wh & 0xFFFF0000u) : __uint_as_float(wh << 16)) +
-                          ((r & 1) ? __uint_as_float(wl & 0xFFFF0000u) : __uint_as_float(wl << 16));
-          y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
-        }
-      if (fp32_out || fused) {
+          for (int r = 0; r < 16; ++r) y[bj][r] = acc[bi][bj][r];
+      } else {
+        const float dr = *(const float *)(dvec_lds + (bi * 32 + rr) * 4);
+        anc_u32x2 xh[2][4], xl[2][4];
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int off = rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8;
+            xh[bj][q] = *(const anc_u32x2 *)(b + off);
+            xl[bj][q] = *(const anc_u32x2 *)(b + 4096 + off);
+          }
+        const float cf = p.ca + dr;
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const uint32_t wh = (r & 2) ? xh[bj][r >> 2].y : xh[bj][r >> 2].x;
+            const uint32_t wl = (r & 2) ? xl[bj][r >> 2].y : xl[bj][r >> 2].x;
+            const float x = ((r & 1) ? __uint_as_float(wh & 0xFFFF0000u) : __uint_as_float(wh << 16)) +
+                            ((r & 1) ? __uint_as_float(wl & 0xFFFF0000u) : __uint_as_float(wl << 16));
+            y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
+          }
+      }
+      if (fp32_out || fused || plain) {
         // fp32 result: [32 rows][16 chunks of 16 B], chunk XOR (row & 15)
 #pragma unroll
         for (int bj = 0; bj < 2; ++bj)
@@ -671,7 +685,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       __builtin_amdgcn_s_waitcnt(0xC07F);
       __builtin_amdgcn_wave_barrier();
       asm volatile("" ::: "memory");
-      if (bi + 2 < 4) fetch_in(bi + 2);
+      if (!plain && bi + 2 < 4) fetch_in(bi + 2);
     }
 #ifdef ANC_DBG_TRACE
     if (threadIdx.x == 0 && blockIdx.x < 16384) {
@@ -833,9 +847,37 @@ int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, h
   for (int k = 0; k < n; ++k) { any_upd = any_upd || ps[k].upd != nullptr; all_upd = all_upd && ps[k].upd != nullptr; }
   ANC_REQUIRE(any_upd == all_upd, "anc_ns_gemm_big: the fused update applies to every problem of a launch or to none");
   if (any_upd)
-    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, true>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_UPDATE>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   else
     hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+  ANC_LAUNCH_CHECK();
+  return ANC_OK;
+}
+
+// Bare products C[e] = A[e] B[e] (fp32 out, p.X32), A (M, K) with row pitch p.ldA, B (K, N)
+// row-major, on the X = a X + B X kernel's K loop: 128x256 tiles, M % 128 == 0, N % 256 == 0,
+// K % 32 == 0.
+int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
+  ANC_REQUIRE(n >= 1 && n <= kMaxGroups, "anc_ns_gemm_big_plain: 1..%d problems per launch", kMaxGroups);
+  NsGemmMulti pm{};
+  pm.n = n;
+  int64_t grid = 0;
+  for (int k = 0; k < n; ++k) {
+    ANC_REQUIRE(ps[k].M % 128 == 0 && ps[k].N % 256 == 0 && ps[k].K % 32 == 0 && ps[k].K >= 32,
+                "anc_ns_gemm_big_plain: needs M % 128 == 0, N % 256 == 0, K % 32 == 0");
+    ANC_REQUIRE(ps[k].X32 != nullptr && ps[k].nterms == 1 && ps[k].scale == nullptr && ps[k].upd == nullptr,
+                "anc_ns_gemm_big_plain: bad problem");
+    pm.g[k] = ps[k];
+    pm.g[k].tiles_m = ps[k].M / 128;
+    pm.g[k].tiles_n = ps[k].N / 256;
+    pm.g[k].lower = 0;
+    const int64_t t = Es[k] * (int64_t)pm.g[k].tiles_m * pm.g[k].tiles_n;
+    ANC_REQUIRE(t > 0 && t < (1ll << 30), "anc_ns_gemm_big_plain: grid out of range");
+    pm.tiles[k] = (int)t;
+    grid += t;
+  }
+  ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big_plain: grid out of range");
+  hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_PLAIN>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }

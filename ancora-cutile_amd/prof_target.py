@@ -8,6 +8,8 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
     python3 -m ancora_cutile_amd.prof_target gradnorm NUMEL [calls]      grad-norm partials + finalize
     python3 -m ancora_cutile_amd.prof_target quant K N E [cm] [calls]    MXFP8 weight re-quantisation
                                       (prints GB/s from HIP events around the calls)
+    python3 -m ancora_cutile_amd.prof_target dw T K N1[,N2,..] [calls]   weight-gradient GEMM of up to 4
+                                      weights (K, Ni) that share the activations, T tokens
     python3 -m ancora_cutile_amd.prof_target mfmamix                    matrix-instruction rate next to
                                       unrelated LDS / LDS-DMA traffic (anc_probe_mfma_mix), a table
 
@@ -82,6 +84,27 @@ def main(argv):
         nbytes = E * K * N * (2 + 1 + 1 / 32)
         print(f"quant_mxfp8_w {'column-major' if cm else 'row-major'} {E}x({K},{N}): {ms * 1e3:.1f} us per call, "
               f"{nbytes / ms / 1e9:.2f} TB/s of {nbytes / 1e9:.3f} GB algorithmic")
+    elif what == "dw":
+        from .grads import gemm_dW, DwWorkspace, dw_info
+        T, K = int(argv[1]), int(argv[2])
+        Ns = [int(v) for v in argv[3].split(",")]
+        calls = int(argv[4]) if len(argv) > 4 else 5
+        rng = np.random.default_rng(0)
+        bits = lambda a: (a.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        xT = DevBuf(bits(0.1 * rng.standard_normal((K, T))))
+        probs = [dict(xT=xT, dy=DevBuf(bits(0.1 * rng.standard_normal((T, N)))), dW=DevBuf.zeros((K, N), np.float32),
+                      g16=DevBuf.zeros((K, N), np.uint16), T=T, K=K, N=N, workspace=DwWorkspace()) for N in Ns]
+        gemm_dW(probs)
+        _lib.stream_sync(0)
+        _lib.profile_enable(True)
+        for _ in range(calls):
+            gemm_dW(probs)
+        pr = _lib.profile_read()
+        _lib.profile_enable(False)
+        fl = sum(dw_info(T, K, N)[0] for N in Ns)
+        gms, rms = pr["dw_gemm"][0] / calls, pr["dw_reduce"][0] / calls
+        print(f"dW T={T} K={K} N={Ns} segments={[dw_info(T, K, N)[1] for N in Ns]}: gemm {gms * 1e3:.1f} us "
+              f"({fl / gms / 1e9:.1f} TFLOP/s), reduce {rms * 1e3:.1f} us, together {fl / (gms + rms) / 1e9:.1f} TFLOP/s")
     elif what == "mfmamix":
         src = DevBuf.zeros((1 << 28,), np.float32)          # 1 GiB
         sink = DevBuf.zeros((512,), np.float32)

@@ -147,6 +147,60 @@ def side_workload(args):
                "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
                "data": "synthetic", "config": {"workload": "ns-196-matrices", "groups": [list(g) for g in groups]},
                "modes": res}
+    elif args.workload == "dw":
+        # the weight-gradient GEMMs of the 28 Qwen3-0.6B layers at `--tokens` tokens per micro-batch,
+        # launched as the backward pass would: per layer [q,k,v] (shared activations), [o],
+        # [gate,up] (shared), [down]; buffers of one layer reused for all layers
+        from ancora_cutile_amd.grads import gemm_dW, DwWorkspace, dw_info
+        from ancora_cutile_amd.bf16 import bf16_bits
+        T = args.tokens
+        rng = np.random.default_rng(0)
+        groups = ((1024, (2048, 1024, 1024)), (2048, (1024,)), (1024, (3072, 3072)), (3072, (1024,)))
+        calls, flops = [], 0.0
+        for K, Ns in groups:
+            xT = DevBuf(bf16_bits((0.1 * rng.standard_normal((K, T))).astype(np.float32)))
+            probs = []
+            for N in Ns:
+                probs.append(dict(xT=xT, dy=DevBuf(bf16_bits((0.1 * rng.standard_normal((T, N))).astype(np.float32))),
+                                  dW=DevBuf.zeros((K, N), np.float32), g16=DevBuf.zeros((K, N), np.uint16),
+                                  T=T, K=K, N=N, workspace=DwWorkspace(), accumulate=True))
+                flops += dw_info(T, K, N)[0]
+            calls.append(probs)
+        layers = 28
+
+        def step():
+            for _ in range(layers):
+                for probs in calls:
+                    gemm_dW(probs, 0)
+        for _ in range(max(1, args.warmup // 2)):
+            step()
+        e0.record(0)
+        for _ in range(args.steps):
+            step()
+        e1.record(0)
+        e1.sync()
+        ms = e0.elapsed_ms(e1) / args.steps
+        _lib.profile_enable(True)
+        step()
+        pr = _lib.profile_read()
+        _lib.profile_enable(False)
+        g_ms, r_ms = pr["dw_gemm"][0], pr["dw_reduce"][0]
+        tf = layers * flops / (ms * 1e-3) / 1e12
+        gtf = layers * flops / (g_ms * 1e-3) / 1e12
+        nparams = sum(K * N for K, Ns in groups for N in Ns) * layers
+        out = {"metric": "Qwen3-0.6B weight-gradient GEMMs (dW += x^T dy, 196 weights) ms per micro-batch",
+               "value": round(ms, 3), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+               "ms_per_step": round(ms, 3), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+               "dtype": "bf16", "data": "synthetic",
+               "config": {"workload": "qwen3-0.6b-weight-gradients", "tokens": T, "weights": 7 * layers,
+                          "params": nparams, "launch_groups_per_layer": 4, "accumulate": True, "bf16_copy": True},
+               "roofline": {"bound": "mfma", "achieved": round(gtf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                            "frac": round(gtf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                            "kernel": "k_ns_gemm_big<EPI_BX, ..., VAR_PLAIN> (partial tiles of x^T dy)",
+                            "launches_per_step": pr["dw_gemm"][1], "avg_launch_ms": round(g_ms / pr["dw_gemm"][1], 4),
+                            "tflop_per_step": round(layers * flops / 1e12, 3)},
+               "whole_tflops_per_s": round(tf, 1),
+               "reduce_kernel": {"ms": round(r_ms, 3), "launches": pr["dw_reduce"][1]}}
     else:
         n = 1_200_000_000
         rng = np.random.default_rng(0)
@@ -202,7 +256,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=28, help=argparse.SUPPRESS)   # smaller sets for debugging
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--workload", default="qwen3", choices=("qwen3", "moe", "ns", "adamw"),
+    ap.add_argument("--tokens", type=int, default=8192, help="tokens per micro-batch of --workload dw")
+    ap.add_argument("--workload", default="qwen3", choices=("qwen3", "moe", "ns", "adamw", "dw"),
                     help="qwen3: the headline hybrid step (default). moe: the 16-layer MoE family "
                          "(config 4). ns: the 196-matrix Newton-Schulz stress, bf16 and fp32 modes "
                          "(config 3). adamw: one flat 1.2e9-element buffer (config 5)")
@@ -214,7 +269,7 @@ def main():
         sys.exit("bench.py: this optimizer step runs on one GPU; --gpus must be 1 "
                  "(no multi-GPU path is built, see DESIGN.md)")
 
-    if args.workload in ("ns", "adamw"):
+    if args.workload in ("ns", "adamw", "dw"):
         return side_workload(args)
     from ancora_cutile_amd import HybridOptimizer, DevBuf, PE_SCHEDULE, _lib
     from ancora_cutile_amd.hybrid import resident_is_muon

@@ -110,7 +110,9 @@ int anc_copy_kernel(uint64_t dst, uint64_t src, int64_t n_bytes, uint64_t stream
 #define ANC_PROF_MISC        11   /* casts, conversions, transposes, fill         */
 #define ANC_PROF_COPY        12
 #define ANC_PROF_NS_BX_UPD   13   /* X = a X + B X whose epilogue applies the weight update */
-#define ANC_PROF_KINDS       14
+#define ANC_PROF_DW_GEMM     14   /* weight-gradient product, partial tiles (bf16 matrix-core GEMM) */
+#define ANC_PROF_DW_REDUCE   15   /* sum of the token segments, accumulation, bf16 emission */
+#define ANC_PROF_KINDS       16
 int anc_profile_enable(int on);
 int anc_profile_read(float *ms /* [ANC_PROF_KINDS] */, int64_t *launches /* [ANC_PROF_KINDS] */);
 
@@ -286,6 +288,29 @@ int anc_muon_update_multi(uint64_t desc_table, int32_t n_weights, int64_t total_
  * (ancora/kernels/moe.py:370-377). M, N multiples of 64. */
 int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
                        uint64_t stream);
+
+/* ------------------------------------------------------ weight gradients ----
+ * dW (+)= x^T dy for up to 4 weights per call: replaces `_gemm_dW` / `_gemm_dW_acc`
+ * (ancora/kernels/fused.py:190-219, launched per weight at ancora/model/resident_train.py:285-287),
+ * the producer of the fp32 gradients the optimizer step reads. xT is the activation matrix
+ * transposed, (K, T) bf16 row-major (anc_transpose_bf16 of the (T, K) activations, once per group
+ * of weights that share them); dy is (T, N) bf16; dW (K, N) fp32 is overwritten, or added onto when
+ * `accumulate` is set (micro-batch accumulation in place); g16, if not 0, receives the bf16 copy
+ * (RNE) of the final dW, the format the step reads. fp32 accumulation in a fixed order: the token
+ * axis is cut into anc_gemm_dw_info's `segments` pieces that depend on (T, K, N) only, each tile
+ * of each piece is one workgroup's whole K loop, and the pieces are added in ascending order, so
+ * the bits do not depend on what else is in the call. T % 32, K % 128, N % 256 == 0 (the reference:
+ * all % 64); pointers 16-byte aligned; workspace of anc_gemm_dw_workspace_bytes(T, K, N) bytes per
+ * problem (the partial tiles), not shared between the problems of a call. */
+typedef struct {
+  uint64_t xT, dy, dW, g16, workspace;
+  int64_t  T, K, N, workspace_bytes;
+  int32_t  accumulate, reserved;
+} anc_dw_problem_t;
+int64_t anc_gemm_dw_workspace_bytes(int64_t T, int64_t K, int64_t N);
+int anc_gemm_dw_multi(const anc_dw_problem_t *problems, int32_t n_problems, uint64_t stream);
+/* FLOPs of one problem (2 T K N, all executed) and its number of token segments. */
+int anc_gemm_dw_info(int64_t T, int64_t K, int64_t N, double *flops, int32_t *segments);
 
 /* MXFP8 re-quantisation of bf16 weights (E, K, N) after the step: per block of 32 consecutive K
  * and per column one E8M0 scale byte = (biased fp32 exponent of the block's amax) - 7 (0 below

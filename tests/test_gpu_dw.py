@@ -1,0 +1,112 @@
+"""GPU parity of the weight-gradient GEMM dW (+)= x^T dy against the fp64 product of the bf16
+inputs (the reference's own checker, tests/kernels/test_gemm_bwd.py), plus what the build adds:
+accumulation in place, the bf16 copy, independence of the result's bits from grouping."""
+import numpy as np
+import pytest
+
+from oracle.gemm_ref import gemm_dw
+from oracle.bf16_ref import bf16_rne_bits
+from util import rel_fro, bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(T, K, N, seed):
+    rng = np.random.default_rng(seed)
+    x = bf16_rne_bits((0.1 * rng.standard_normal((T, K))).astype(np.float32)).reshape(T, K)
+    dy = bf16_rne_bits((0.1 * rng.standard_normal((T, N))).astype(np.float32)).reshape(T, N)
+    return x, dy
+
+
+def _problem(x, dy, T, K, N, emit=False, dW0=None):
+    from ancora_cutile_amd import DevBuf
+    from ancora_cutile_amd.grads import transpose_acts, DwWorkspace
+    xd, xT = DevBuf(x), DevBuf.zeros((K, T), np.uint16)
+    transpose_acts(xd, xT, T, K)
+    p = dict(xT=xT, dy=DevBuf(dy), dW=DevBuf.zeros((K, N), np.float32) if dW0 is None else DevBuf(dW0),
+             T=T, K=K, N=N, workspace=DwWorkspace(), g16=DevBuf.zeros((K, N), np.uint16) if emit else None,
+             accumulate=dW0 is not None)
+    p["_x"] = xd
+    return p
+
+
+def _free(p):
+    for k in ("xT", "dy", "dW", "g16", "_x"):
+        if p.get(k) is not None:
+            p[k].free()
+    p["workspace"].free()
+
+
+@pytest.mark.parametrize("T,K,N", [(512, 1024, 1024), (256, 1024, 3072), (64, 128, 256), (2048, 128, 256),
+                                   (4096, 256, 512), (96, 384, 768)])
+def test_matches_fp64_product(gpu, T, K, N):
+    """The first two shapes are the reference's (test_gemm_bwd.py:49-50); the others reach one and
+    many token segments, a single tile, and a token count that is not a multiple of 64."""
+    from ancora_cutile_amd.grads import gemm_dW, dw_info
+    x, dy = _inputs(T, K, N, T + K + N)
+    p = _problem(x, dy, T, K, N, emit=True) if T % 64 == 0 else None
+    if p is None:                                  # the device transpose works on 64x64 tiles
+        from ancora_cutile_amd import DevBuf
+        from ancora_cutile_amd.grads import DwWorkspace
+        p = dict(xT=DevBuf(np.ascontiguousarray(x.T)), dy=DevBuf(dy), dW=DevBuf.zeros((K, N), np.float32),
+                 T=T, K=K, N=N, workspace=DwWorkspace(), g16=DevBuf.zeros((K, N), np.uint16), accumulate=False)
+    gemm_dW([p])
+    got = p["dW"].to_numpy()
+    want = gemm_dw(x, dy)
+    assert rel_fro(got, want) < 2e-5
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-4        # reference bar: 2e-2
+    assert bits_equal(p["g16"].to_numpy(), bf16_rne_bits(got).reshape(K, N))
+    fl, seg = dw_info(T, K, N)
+    assert fl == 2.0 * T * K * N and seg >= 1 and T % (32 * seg) == 0
+    _free(p)
+
+
+def test_accumulates_in_place_and_is_deterministic(gpu):
+    from ancora_cutile_amd.grads import gemm_dW
+    T, K, N = 1024, 256, 512
+    x1, dy1 = _inputs(T, K, N, 1)
+    x2, dy2 = _inputs(T, K, N, 2)
+    p1 = _problem(x1, dy1, T, K, N)
+    gemm_dW([p1])
+    first = p1["dW"].to_numpy()
+    p2 = _problem(x2, dy2, T, K, N, emit=True, dW0=first)
+    gemm_dW([p2])
+    total = p2["dW"].to_numpy()
+    assert rel_fro(total, gemm_dw(x2, dy2, gemm_dw(x1, dy1))) < 2e-5
+    assert bits_equal(p2["g16"].to_numpy(), bf16_rne_bits(total).reshape(K, N))
+    # the same call again on the same inputs gives the same bits
+    p3 = _problem(x2, dy2, T, K, N, dW0=first)
+    gemm_dW([p3])
+    assert bits_equal(p3["dW"].to_numpy(), total)
+    for p in (p1, p2, p3):
+        _free(p)
+
+
+def test_grouping_does_not_change_bits(gpu):
+    """q, k, v style: three weights that share the activations, alone and in one call."""
+    from ancora_cutile_amd.grads import gemm_dW
+    T, K = 1024, 256
+    Ns = (512, 256, 768)
+    x, _ = _inputs(T, K, 256, 5)
+    dys = [_inputs(T, K, N, 10 + i)[1] for i, N in enumerate(Ns)]
+    alone = []
+    for dy, N in zip(dys, Ns):
+        p = _problem(x, dy, T, K, N)
+        gemm_dW([p])
+        alone.append(p["dW"].to_numpy())
+        _free(p)
+    ps = [_problem(x, dy, T, K, N) for dy, N in zip(dys, Ns)]
+    gemm_dW(ps)
+    for p, a in zip(ps, alone):
+        assert bits_equal(p["dW"].to_numpy(), a)
+        _free(p)
+
+
+def test_shape_checks(gpu):
+    from ancora_cutile_amd import _lib
+    from ancora_cutile_amd.grads import dw_workspace_bytes
+    with pytest.raises(_lib.AncoraError):
+        dw_workspace_bytes(100, 128, 256)
+    with pytest.raises(_lib.AncoraError):
+        dw_workspace_bytes(128, 64, 256)
+    assert dw_workspace_bytes(64, 128, 256) == 128 * 256 * 4

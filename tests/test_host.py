@@ -51,6 +51,7 @@ def test_header_is_plain_c_and_layouts_match_ctypes(tmp_path):
     pairs = [("anc_step_ctl_t", _lib.StepCtl), ("anc_adamw_hyper_t", _lib.AdamWHyper),
              ("anc_adamw_desc_t", _lib.AdamWDesc), ("anc_gn_desc_t", _lib.GnDesc),
              ("anc_muon_desc_t", _lib.MuonDesc), ("anc_ns_problem_t", _lib.NsProblem),
+             ("anc_dw_problem_t", _lib.DwProblem),
              ("anc_device_info_t", _lib.DeviceInfo)]
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "anc_optim.h"', 'int main(void) {']
     for cname, ct in pairs:
