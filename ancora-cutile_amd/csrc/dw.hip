@@ -14,11 +14,12 @@
 // when accumulating) and can emit the bf16 copy the optimizer step reads. S depends on the
 // problem's shape alone, so the result's bits do not depend on what shares the launch: one
 // workgroup owns one (tile, segment) and its whole K loop, K tiles in ascending order, no atomics.
+#include "reduce.h"
 #include "ns_common.h"
 
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = anc_reduce::kThreads;
 
 // Segments of the token axis: the smallest power of two that gives the problem at least 256
 // workgroups (one per CU), with at least 256 tokens per segment and segment length a multiple
@@ -34,6 +35,7 @@ struct DwReduce {
   const float *part;     // (S, n) partials
   float *dW;             // (n)
   uint16_t *g16;         // (n) or null
+  double *gn;            // (n / ANC_GN_CHUNK) grad-norm partials or null
   int64_t n;
   int S;
   int accumulate;
@@ -44,24 +46,51 @@ struct DwReduceMulti {
   DwReduce r[kMaxGroups];
 };
 
+// One block per 8192-element chunk of the flat gradient, elements dealt to the lanes exactly as
+// the grad-norm kernel deals them (anc_reduce: run j*256 + lane = 8 consecutive elements), so that
+// the chunk's sum of squares -- of the bf16 copy if one is emitted, else of the fp32 gradient --
+// comes out with the bits the grad-norm kernel would produce from the stored gradient.
 __global__ void __launch_bounds__(kThreads) k_dw_reduce(DwReduceMulti m) {
+  using namespace anc_reduce;
   int q = 0;
   while (q + 1 < m.count && (int64_t)blockIdx.x >= m.blk0[q + 1]) ++q;
   const DwReduce &r = m.r[q];
-  const int64_t i = (((int64_t)blockIdx.x - m.blk0[q]) * kThreads + threadIdx.x) * 4;
-  if (i >= r.n) return;
-  anc_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (r.accumulate) acc = anc_ld_stream((const anc_f32x4 *)(r.dW + i));
-  for (int s = 0; s < r.S; ++s) {
-    const anc_f32x4 v = anc_ld_stream((const anc_f32x4 *)(r.part + (int64_t)s * r.n + i));
-    acc.x = acc.x + v.x; acc.y = acc.y + v.y; acc.z = acc.z + v.z; acc.w = acc.w + v.w;
+  const int64_t chunk = (int64_t)blockIdx.x - m.blk0[q];
+  float ss[kIters];
+#pragma unroll
+  for (int j = 0; j < kIters; ++j) {
+    const int64_t i = chunk * (int64_t)ANC_GN_CHUNK + ((int64_t)j * kThreads + threadIdx.x) * kRun;
+    anc_f32x4 a0 = {0.0f, 0.0f, 0.0f, 0.0f}, a1 = a0;
+    if (r.accumulate) {
+      a0 = anc_ld_stream((const anc_f32x4 *)(r.dW + i));
+      a1 = anc_ld_stream((const anc_f32x4 *)(r.dW + i + 4));
+    }
+    for (int s = 0; s < r.S; ++s) {
+      const float *pp = r.part + (int64_t)s * r.n + i;
+      const anc_f32x4 v0 = anc_ld_stream((const anc_f32x4 *)pp);
+      const anc_f32x4 v1 = anc_ld_stream((const anc_f32x4 *)(pp + 4));
+      a0.x = a0.x + v0.x; a0.y = a0.y + v0.y; a0.z = a0.z + v0.z; a0.w = a0.w + v0.w;
+      a1.x = a1.x + v1.x; a1.y = a1.y + v1.y; a1.z = a1.z + v1.z; a1.w = a1.w + v1.w;
+    }
+    anc_st_stream((anc_f32x4 *)(r.dW + i), a0);
+    anc_st_stream((anc_f32x4 *)(r.dW + i + 4), a1);
+    float x[kRun] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    if (r.g16 != nullptr) {
+      uint32_t hb[kRun];
+#pragma unroll
+      for (int k = 0; k < kRun; ++k) {
+        hb[k] = anc_bf16_rne_bits(x[k]);
+        x[k] = anc_bf16_bits_to_f32(hb[k]);
+      }
+      const anc_u32x4 h = {hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16), hb[4] | (hb[5] << 16), hb[6] | (hb[7] << 16)};
+      anc_st_stream((anc_u32x4 *)(r.g16 + i), h);
+    }
+    float sq = x[0] * x[0];
+#pragma unroll
+    for (int k = 1; k < kRun; ++k) sq = sq + x[k] * x[k];
+    ss[j] = sq;
   }
-  anc_st_stream((anc_f32x4 *)(r.dW + i), acc);
-  if (r.g16 != nullptr) {
-    const anc_u32x2 h = {anc_bf16_rne_bits(acc.x) | (anc_bf16_rne_bits(acc.y) << 16),
-                         anc_bf16_rne_bits(acc.z) | (anc_bf16_rne_bits(acc.w) << 16)};
-    anc_st_stream((anc_u32x2 *)(r.g16 + i), h);
-  }
+  if (r.gn != nullptr) chunk_finish(ss, r.gn + chunk);      // uniform over the block
 }
 
 int check_dw(const anc_dw_problem_t &b, const char *who) {
@@ -94,7 +123,7 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
     const anc_dw_problem_t &b = probs[q];
     if (int rc = check_dw(b, "anc_gemm_dw_multi")) return rc;
     ANC_REQUIRE(b.xT != 0 && b.dy != 0 && b.dW != 0 && b.workspace != 0 &&
-                ((b.xT | b.dy | b.dW | b.workspace) & 15) == 0 && (b.g16 & 7) == 0,
+                ((b.xT | b.dy | b.dW | b.workspace | b.g16) & 15) == 0 && (b.gn_partials & 7) == 0,
                 "anc_gemm_dw_multi: null or misaligned pointer");
     const int S = dw_segments(b.T, b.K, b.N);
     ANC_REQUIRE(b.workspace_bytes >= (int64_t)S * b.K * b.N * 4, "anc_gemm_dw_multi: workspace holds %lld bytes, %lld needed",
@@ -113,9 +142,10 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
     p.X32 = (float *)b.workspace;    // partial e at e * K * N
     g[q] = p;
     Es[q] = S;
-    rm.r[q] = DwReduce{(const float *)b.workspace, (float *)b.dW, (uint16_t *)b.g16, b.K * b.N, S, b.accumulate ? 1 : 0};
+    rm.r[q] = DwReduce{(const float *)b.workspace, (float *)b.dW, (uint16_t *)b.g16, (double *)b.gn_partials,
+                       b.K * b.N, S, b.accumulate ? 1 : 0};
     rm.blk0[q] = blocks;
-    blocks += (b.K * b.N / 4 + kThreads - 1) / kThreads;
+    blocks += b.K * b.N / ANC_GN_CHUNK;            // K % 128 and N % 256: whole chunks only
   }
   rm.blk0[n_probs] = blocks;
   ANC_REQUIRE(blocks < (1ll << 31), "anc_gemm_dw_multi: too large");

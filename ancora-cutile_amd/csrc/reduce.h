@@ -51,17 +51,9 @@ __device__ __forceinline__ float run_sumsq(const void *g, int64_t e, int64_t n) 
   return s;
 }
 
-template <int GD>
-__device__ __forceinline__ void chunk_partial(const void *g, int64_t n, int64_t chunk,
-                                              double *__restrict__ out) {
+// The chunk's partial from the kIters run sums of every lane (s[j]: run j*kThreads + lane).
+__device__ __forceinline__ void chunk_finish(const float (&s)[kIters], double *__restrict__ out) {
   __shared__ double wave_sum[kThreads / 64];
-  const int64_t base = chunk * (int64_t)ANC_GN_CHUNK;
-  float s[kIters];
-#pragma unroll
-  for (int j = 0; j < kIters; ++j) {
-    const int64_t e = base + ((int64_t)j * kThreads + threadIdx.x) * kRun;
-    s[j] = (e < n) ? run_sumsq<GD>(g, e, n) : 0.0f;
-  }
   double acc = 0.0;
 #pragma unroll
   for (int j = 0; j < kIters; ++j) acc = acc + (double)s[j];
@@ -74,6 +66,19 @@ __device__ __forceinline__ void chunk_partial(const void *g, int64_t n, int64_t 
     for (int w = 1; w < kThreads / 64; ++w) t = t + wave_sum[w];
     *out = t;
   }
+}
+
+template <int GD>
+__device__ __forceinline__ void chunk_partial(const void *g, int64_t n, int64_t chunk,
+                                              double *__restrict__ out) {
+  const int64_t base = chunk * (int64_t)ANC_GN_CHUNK;
+  float s[kIters];
+#pragma unroll
+  for (int j = 0; j < kIters; ++j) {
+    const int64_t e = base + ((int64_t)j * kThreads + threadIdx.x) * kRun;
+    s[j] = (e < n) ? run_sumsq<GD>(g, e, n) : 0.0f;
+  }
+  chunk_finish(s, out);
 }
 
 }  // namespace anc_reduce

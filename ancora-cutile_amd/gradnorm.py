@@ -34,30 +34,50 @@ class StepGuard:
         self.eps = float(eps)
         self.ctl = DevBuf.zeros((8,), np.uint32)
         self._partials = None
-        self._table = None
+        self._tables = {}
+        self._part0 = []
         self._key = None
 
     @property
     def ptr(self):
         return self.ctl.ptr
 
-    def compute(self, grads, stream=0):
-        """grads: list of DevBuf (float32 or uint16/bf16), in a fixed order. Asynchronous."""
+    def plan(self, grads):
+        """Lay out the partial sums for this list of gradients (fixed order) without computing
+        anything: afterwards `partials_ptr(i)` is where tensor i's partials live, so that a
+        producer of the gradients can write them itself (`gemm_dW(..., gn_partials=...)`)."""
         key = tuple((g.ptr, g.size, g.dtype.str) for g in grads)
         if key != self._key:
             self._free_tables()
-            descs, chunk0 = [], 0
+            self._part0, chunk0 = [], 0
             for g in grads:
-                nch = api.anc_gradnorm_num_partials(g.size)
-                descs.append(GnDesc(g.ptr, g.size, chunk0, chunk0, _dtype_code(g.dtype), 0))
-                chunk0 += nch
+                self._part0.append(chunk0)
+                chunk0 += api.anc_gradnorm_num_partials(g.size)
             self._n_partials = chunk0
-            self._n_tensors = len(descs)
-            self._table = upload_table(descs)
             self._partials = DevBuf.empty((chunk0,), np.float64)
+            self._tables = {}
             self._key = key
-        api.anc_gradnorm_partials_multi(self._table.ptr, self._n_tensors, self._n_partials,
-                                        self._partials.ptr, int(stream))
+
+    def partials_ptr(self, i):
+        return self._partials.ptr + 8 * self._part0[i]
+
+    def compute(self, grads, stream=0, produced=()):
+        """grads: list of DevBuf (float32 or uint16/bf16), in a fixed order. `produced`: indices
+        of gradients whose partial sums are already in place (written by their producer since the
+        last call). The result is the same bits either way. Asynchronous."""
+        self.plan(grads)
+        produced = tuple(sorted(set(int(i) for i in produced)))
+        if produced not in self._tables:
+            descs, chunk0 = [], 0
+            for i, g in enumerate(grads):
+                if i in produced:
+                    continue
+                descs.append(GnDesc(g.ptr, g.size, chunk0, self._part0[i], _dtype_code(g.dtype), 0))
+                chunk0 += api.anc_gradnorm_num_partials(g.size)
+            self._tables[produced] = (upload_table(descs) if descs else None, len(descs), chunk0)
+        table, n_tensors, n_chunks = self._tables[produced]
+        if table is not None:
+            api.anc_gradnorm_partials_multi(table.ptr, n_tensors, n_chunks, self._partials.ptr, int(stream))
         api.anc_gradnorm_finalize(self._partials.ptr, self._n_partials, self.max_norm, self.eps,
                                   self.ctl.ptr, int(stream))
 
@@ -68,10 +88,11 @@ class StepGuard:
         return {"sumsq": c.sumsq, "norm": c.norm, "clip_scale": c.clip_scale, "skip": bool(c.skip)}
 
     def _free_tables(self):
-        for b in (self._partials, self._table):
+        for b in [self._partials] + [t[0] for t in self._tables.values()]:
             if b is not None:
                 b.free()
-        self._partials = self._table = None
+        self._partials = None
+        self._tables = {}
 
     def free(self):
         self._free_tables()

@@ -59,8 +59,9 @@ class DwWorkspace:
 
 def gemm_dW(problems, si=0):
     """problems: list of dicts {xT, dy, dW: DevBuf; T, K, N: int; workspace: DwWorkspace;
-    g16: DevBuf or None; accumulate: bool}. dW (+)= x^T dy for each, 4 per launch. Asynchronous
-    on stream `si`."""
+    g16: DevBuf or None; accumulate: bool; gn_partials: int device address or None (where the
+    grad-norm partial sums of this gradient go, `StepGuard.partials_ptr`)}. dW (+)= x^T dy for
+    each, 4 per launch. Asynchronous on stream `si`."""
     _lib.init()
     for i0 in range(0, len(problems), MAX_PER_CALL):
         group = problems[i0:i0 + MAX_PER_CALL]
@@ -71,5 +72,6 @@ def gemm_dW(problems, si=0):
             ws = p["workspace"].ensure(nb)
             g16 = p.get("g16")
             arr[k] = DwProblem(p["xT"].ptr, p["dy"].ptr, p["dW"].ptr, 0 if g16 is None else g16.ptr, ws.ptr,
-                               T, K, N, ws.nbytes, int(bool(p.get("accumulate", False))), 0)
+                               T, K, N, ws.nbytes, int(bool(p.get("accumulate", False))), 0,
+                               int(p.get("gn_partials") or 0))
         api.anc_gemm_dw_multi(arr, len(group), int(si))

@@ -77,7 +77,17 @@ class HybridOptimizer:
             out.append(g if isinstance(g, DevBuf) else self.adamw.st[n]["g"])
         return out
 
-    def step(self, grads, stream_int):
+    def gn_partials_ptr(self, grads, name):
+        """Device address where the grad-norm partial sums of gradient `name` live for this set of
+        gradient buffers: a producer (`gemm_dW(..., gn_partials=...)`) that writes them there can be
+        named in `step(..., produced=[...])`, and the norm then skips its pass over that tensor."""
+        bufs = self._grad_bufs(grads)
+        self.guard.plan(bufs)
+        return self.guard.partials_ptr((self.muon_names + self.adamw_names).index(name))
+
+    def step(self, grads, stream_int, produced=()):
+        """`produced`: names of resident gradients whose grad-norm partial sums their producer has
+        already written (see `gn_partials_ptr`); same result bits with or without."""
         if self.guard is None:
             self.muon.step({n: grads[n] for n in self.muon_names}, stream_int)
             self.adamw.step({n: grads[n] for n in self.adamw_names}, stream_int)
@@ -97,7 +107,8 @@ class HybridOptimizer:
             for n in names:
                 g = grads[n]
                 resident[n] = g if isinstance(g, DevBuf) else opt.st[n]["g"]
-        self.guard.compute(self._grad_bufs(grads), stream_int)
+        order = self.muon_names + self.adamw_names
+        self.guard.compute(self._grad_bufs(grads), stream_int, produced=[order.index(n) for n in produced])
         # Muon's per-shape chains fork onto their own streams; AdamW runs beside them
         self.muon.launch({n: resident[n] for n in self.muon_names}, stream_int, self.guard,
                          defer_join=True)

@@ -301,11 +301,15 @@ int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
  * of each piece is one workgroup's whole K loop, and the pieces are added in ascending order, so
  * the bits do not depend on what else is in the call. T % 32, K % 128, N % 256 == 0 (the reference:
  * all % 64); pointers 16-byte aligned; workspace of anc_gemm_dw_workspace_bytes(T, K, N) bytes per
- * problem (the partial tiles), not shared between the problems of a call. */
+ * problem (the partial tiles), not shared between the problems of a call. g16 16-byte aligned. */
 typedef struct {
   uint64_t xT, dy, dW, g16, workspace;
   int64_t  T, K, N, workspace_bytes;
   int32_t  accumulate, reserved;
+  uint64_t gn_partials;        /* 0, or double[K*N / ANC_GN_CHUNK]: the grad-norm partial sums of this
+                                  gradient (of its bf16 copy if g16 is set), bit-identical to what
+                                  anc_gradnorm_partials would compute from the stored gradient, so
+                                  that the step's norm needs no pass of its own over it */
 } anc_dw_problem_t;
 int64_t anc_gemm_dw_workspace_bytes(int64_t T, int64_t K, int64_t N);
 int anc_gemm_dw_multi(const anc_dw_problem_t *problems, int32_t n_problems, uint64_t stream);

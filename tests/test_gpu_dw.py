@@ -110,3 +110,71 @@ def test_shape_checks(gpu):
     with pytest.raises(_lib.AncoraError):
         dw_workspace_bytes(128, 64, 256)
     assert dw_workspace_bytes(64, 128, 256) == 128 * 256 * 4
+
+
+def test_producer_writes_the_grad_norm_partials(gpu):
+    """With `gn_partials` the reduce kernel leaves the chunk sums of squares of the gradient it
+    emits (bf16 copy, or the fp32 gradient when there is none) where StepGuard keeps them; the
+    control block then has the bits of a norm pass over the stored gradients."""
+    from ancora_cutile_amd import DevBuf, StepGuard
+    from ancora_cutile_amd.grads import gemm_dW
+    T, K = 512, 256
+    Ns = (512, 256)
+    x, _ = _inputs(T, K, 256, 3)
+    ps = [_problem(x, _inputs(T, K, N, 20 + i)[1], T, K, N, emit=(i == 0)) for i, N in enumerate(Ns)]
+    other = DevBuf(bf16_rne_bits((1e-2 * np.random.default_rng(4).standard_normal(50000)).astype(np.float32)))
+    grads = [ps[0]["g16"], other, ps[1]["dW"]]          # bf16 copy, an unrelated tensor, an fp32 gradient
+    guard = StepGuard(1.0)
+    guard.plan(grads)
+    ps[0]["gn_partials"], ps[1]["gn_partials"] = guard.partials_ptr(0), guard.partials_ptr(2)
+    gemm_dW(ps)
+    guard.compute(grads, 0, produced=(0, 2))
+    got = guard.ctl.to_numpy()
+    guard2 = StepGuard(1.0)
+    guard2.compute(grads, 0)
+    want = guard2.ctl.to_numpy()
+    assert np.array_equal(got, want)
+    c = guard.read()
+    assert c["norm"] > 0 and not c["skip"]
+    guard.free(); guard2.free(); other.free()
+    for p in ps:
+        _free(p)
+
+
+def test_backward_to_step_hand_off(gpu):
+    """The weight-gradient GEMM feeds the optimizer step directly: bf16 gradients and grad-norm
+    partial sums from the producer, `step(..., produced=...)`; same weights, bit for bit, as the
+    step computing the norm itself from the same gradients."""
+    from ancora_cutile_amd import HybridOptimizer, DevBuf, PE_SCHEDULE as PE
+    from ancora_cutile_amd.grads import gemm_dW
+    rng = np.random.default_rng(12)
+    T, K = 512, 256
+    shapes = {"layer0.q_proj": (K, 512), "layer0.k_proj": (K, 256)}
+    params = {n: (0.02 * rng.standard_normal(s)).astype(np.float32) for n, s in shapes.items()}
+    params["layer0.input_ln"] = (1.0 + 0.05 * rng.standard_normal(256)).astype(np.float32)
+    x, _ = _inputs(T, K, 256, 30)
+    dys = {n: _inputs(T, K, s[1], 31 + i)[1] for i, (n, s) in enumerate(shapes.items())}
+    g_ln = DevBuf(bf16_rne_bits((1e-2 * rng.standard_normal(256)).astype(np.float32)))
+
+    def run(use_produced):
+        opt = HybridOptimizer(params, max_grad_norm=1.0, grad_dtype=np.uint16,
+                              muon_kw=dict(lr=0.02, momentum=0.95, ns_steps=5, schedule=PE))
+        ps = {n: _problem(x, dys[n], T, K, s[1], emit=True) for n, s in shapes.items()}
+        grads = {n: ps[n]["g16"] for n in shapes}
+        grads["layer0.input_ln"] = g_ln
+        if use_produced:
+            for n in shapes:
+                ps[n]["gn_partials"] = opt.gn_partials_ptr(grads, n)
+        gemm_dW(list(ps.values()))
+        opt.step(grads, 0, produced=list(shapes) if use_produced else ())
+        out = {**opt.muon.master(), **opt.adamw.master()}, opt.last_ctl
+        opt.free()
+        for p in ps.values():
+            _free(p)
+        return out
+
+    (ma, ca), (mb, cb) = run(True), run(False)
+    assert ca == cb and ca["clip_scale"] < 1.0
+    for n in params:
+        assert bits_equal(ma[n], mb[n])
+    g_ln.free()
