@@ -428,6 +428,14 @@ int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, int mode, i
 int anc_probe_mfma_mix(int nread, int ndma, int hbm, int iters, uint64_t src,
                        int64_t span_bytes, uint64_t sink, double *tflops,
                        double *cycles_per_iter);
+/* Diagnostics, no reference counterpart: the GEMM's K loop alone (256x256x32 tiles, 8 wavefronts
+ * of 128x64 or 4 of 128x128 per workgroup, 4-stage LDS-DMA ring, real fragment reads, one barrier
+ * per K tile, no epilogue) on 256 workgroups. Groups of `share` (1..32, power of two) workgroups
+ * of one XCD multiply the same two 256-row operands (2 x 256 x 32*k_tiles bf16 per group at
+ * `src`): share = 32 means nearly every operand load is served from L2 (what the loop structure
+ * reaches when memory is out of the way), share = 4 about three in four. */
+int anc_probe_kloop(int waves, int share, int k_tiles, int reps, uint64_t src, int64_t span_bytes,
+                    uint64_t sink, double *tflops);
 
 /* fp32 <-> bf16 conversion of packed batches (entry/exit of the bf16-typed
  * reference drivers): dst_f32 = float(src_bf16); dst_bf16 = RNE(src_f32). */

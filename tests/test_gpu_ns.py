@@ -231,3 +231,18 @@ def test_mfma_mix_probe_runs(gpu):
     with pytest.raises(_lib.AncoraError):
         _lib.api.anc_probe_mfma_mix(5, 5, 0, 10, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf), ctypes.byref(cyc))
     src.free(); sink.free()
+
+
+def test_kloop_probe_runs(gpu):
+    """The K-loop diagnostics entry returns a plausible rate and rejects a bad configuration."""
+    import ctypes
+    from ancora_cutile_amd import DevBuf, _lib
+    src = DevBuf.zeros((1 << 22,), np.float32)        # 16 MiB: 8 groups of 2 x 256 x 2048 bf16
+    sink = DevBuf.zeros((512,), np.float32)
+    tf = ctypes.c_double(0)
+    for waves in (8, 4):
+        _lib.api.anc_probe_kloop(waves, 32, 64, 4, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf))
+        assert 300.0 < tf.value < 2500.0
+    with pytest.raises(_lib.AncoraError):
+        _lib.api.anc_probe_kloop(6, 32, 64, 4, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf))
+    src.free(); sink.free()
