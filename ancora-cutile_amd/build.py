@@ -9,7 +9,9 @@ Ablation switches of csrc/ns_gemm_big.hip: ANC_DBG_NOEPI (no epilogue), ANC_DBG_
 tiles fetched for the first K tiles only), ANC_DBG_NOMFMA (matrix instructions replaced by an add),
 ANC_DBG_TRACE (per-workgroup timestamps of K loop and epilogue, read with anc_dbg_trace_read),
 ANC_DBG_KNOWAIT (K loop does not wait for its DMA), ANC_DBG_EPI_NOST / ANC_DBG_EPI_NOLD (epilogue
-without its global stores / without its input DMA). All but TRACE give wrong results: timing only.
+without its global stores / without its input DMA); of csrc/ns.hip: ANC_DBG_SAMEOPS (every matrix of
+a batch multiplies the first matrix's operands, i.e. cache-resident operands). All but TRACE give
+wrong results: timing only.
 
 hipcc cross-compiles without a GPU. Flags: no FMA contraction (the AdamW kernel must
 reproduce a numpy fp32 evaluation operation by operation), correctly rounded fp32
