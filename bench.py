@@ -267,7 +267,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this optimizer step runs on one GPU; --gpus must be 1 "
-                 "(no multi-GPU path is built, see DESIGN.md)")
+                 "(no multi-GPU path is built: every box has one GPU and the step needs no collective)")
 
     if args.workload in ("ns", "adamw", "dw"):
         return side_workload(args)
