@@ -373,7 +373,8 @@ def main():
     # no update kernel exists and its traffic (10 B per parameter) is inside that GEMM launch.
     upd_fused = "muon_update" not in kind_ms
     elem_ms = kind_ms["muon_momentum"] + kind_ms.get("muon_update", 0.0)
-    elem_bytes = 12.0 if upd_fused else 24.0
+    # momentum: bf16 g read, fp32 momentum read and written, bf16 pair written = 14 B; update: 10 B
+    elem_bytes = 14.0 if upd_fused else 24.0
     elem_gbps = elem_bytes * n_muon / (elem_ms * 1e-3) / 1e9
 
     # HBM bytes per k_ns_gemm_big launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE on this
