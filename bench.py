@@ -373,8 +373,10 @@ def main():
     # no update kernel exists and its traffic (10 B per parameter) is inside that GEMM launch.
     upd_fused = "muon_update" not in kind_ms
     elem_ms = kind_ms["muon_momentum"] + kind_ms.get("muon_update", 0.0)
-    # momentum: bf16 g read, fp32 momentum read and written, bf16 pair written = 14 B; update: 10 B
-    elem_bytes = 14.0 if upd_fused else 24.0
+    # algorithmic bytes of the momentum stage: bf16 g + fp32 momentum read, fp32 momentum + bf16 u
+    # written = 12 B; this kernel writes u as a bf16 pair, so it moves 14 B
+    elem_bytes = 12.0 if upd_fused else 24.0
+    elem_moved = 14.0 if upd_fused else 26.0
     elem_gbps = elem_bytes * n_muon / (elem_ms * 1e-3) / 1e9
 
     # HBM bytes per k_ns_gemm_big launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE on this
@@ -417,6 +419,8 @@ def main():
                          "ms": round(kind_ms["gradnorm_partials"], 4)},
         "muon_elementwise_hbm": {"achieved": round(elem_gbps, 1), "unit": "GB/s",
                                  "frac": round(elem_gbps / PEAK_HBM_GBPS, 4), "bytes_per_param": int(elem_bytes),
+                                 "moved_bytes_per_param": int(elem_moved),
+                                 "moved_gbps": round(elem_gbps * elem_moved / elem_bytes, 1),
                                  "ms": round(elem_ms, 4),
                                  "kernels": "momentum; the update runs in the epilogue of the chain's last GEMM"
                                  if upd_fused else "momentum + update"},
