@@ -11,9 +11,11 @@
 // backward pass produces one layer's gradients at a time. So the token axis is cut into S
 // segments: segment s of every tile is its own workgroup and leaves an fp32 partial tile in the
 // workspace; a second, HBM-bound kernel adds the S partials in ascending order (and the old dW
-// when accumulating) and can emit the bf16 copy the optimizer step reads. S depends on the
-// problem's shape alone, so the result's bits do not depend on what shares the launch: one
-// workgroup owns one (tile, segment) and its whole K loop, K tiles in ascending order, no atomics.
+// when accumulating) and can emit the bf16 copy the optimizer step reads. S is the caller's
+// (`segments`: a caller that collects a whole layer's 7 weights into one call fills the CUs with
+// S = 1 and saves the partials' traffic) or, by default, a function of the problem's shape alone;
+// either way the result's bits do not depend on what shares the launch: one workgroup owns one
+// (tile, segment) and its whole K loop, K tiles in ascending order, no atomics.
 #include "reduce.h"
 #include "ns_common.h"
 
@@ -125,7 +127,10 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
     ANC_REQUIRE(b.xT != 0 && b.dy != 0 && b.dW != 0 && b.workspace != 0 &&
                 ((b.xT | b.dy | b.dW | b.workspace | b.g16) & 15) == 0 && (b.gn_partials & 7) == 0,
                 "anc_gemm_dw_multi: null or misaligned pointer");
-    const int S = dw_segments(b.T, b.K, b.N);
+    const int S = b.segments > 0 ? b.segments : dw_segments(b.T, b.K, b.N);
+    ANC_REQUIRE(b.segments >= 0 && S <= 256 && b.T % ((int64_t)S * 32) == 0,
+                "anc_gemm_dw_multi: segments=%d must be 0 (shape rule) or divide T=%lld into multiples of 32 tokens",
+                (int)b.segments, (long long)b.T);
     ANC_REQUIRE(b.workspace_bytes >= (int64_t)S * b.K * b.N * 4, "anc_gemm_dw_multi: workspace holds %lld bytes, %lld needed",
                 (long long)b.workspace_bytes, (long long)S * b.K * b.N * 4);
     const int64_t seg = b.T / S;

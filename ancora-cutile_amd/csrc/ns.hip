@@ -721,7 +721,7 @@ extern "C" int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partia
   return run_bf16_chain(&cp, 1, steps, coef, force_small, s);
 }
 
-// n_probs <= 4 independent batches (the shape groups of one optimizer step) through the chain
+// n_probs <= 8 independent batches (the shape groups of one optimizer step) through the chain
 // side by side: each product of each step is one launch over all of them, which keeps the
 // CUs busy where per-batch launches would each end in a partly filled last wave. Same
 // results, bit for bit, as anc_ns_batched_pair on each batch. All dims multiples of 256.

@@ -60,6 +60,9 @@ struct NsGemm {
   int64_t strideA, strideB;  // elements between consecutive matrices
   int tiles_m, tiles_n;
   int lower;                 // symmetric output: tiles with tn <= tm only, mirrored
+  int blk_r, blk_c;          // plain product: the tile sequence of a matrix runs block by block, blocks of
+                             // blk_r x blk_c tiles (rows x columns), so that the contiguous eighth of it that
+                             // lands on one XCD is a compact patch of the output; 0 = row by row
   int M, N;                  // matrix dims of the chain (A, B are MxM; X is MxN)
   float ca, cb, cc;
   float *A32;                // (E,M,M) fp32 A            GRAM out, BMAT in
@@ -80,10 +83,13 @@ struct NsGemm {
 };
 
 
-// Up to 4 independent problems of the same kind (the same product of different shape groups)
+// Up to 8 independent problems of the same kind (the same product of different shape groups)
 // in one launch: tiles[k] workgroups belong to problem k. One launch over all groups keeps the
 // CUs busy where separate launches would each end in a partly filled last wave.
-constexpr int kMaxGroups = 4;
+#ifndef ANC_MAX_GROUPS
+#define ANC_MAX_GROUPS 8
+#endif
+constexpr int kMaxGroups = ANC_MAX_GROUPS;
 struct NsGemmMulti {
   int n;
   int tiles[kMaxGroups];

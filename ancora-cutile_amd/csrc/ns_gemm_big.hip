@@ -36,7 +36,7 @@
 // operands exchanged (transposed accumulator layout: a lane holds runs of 4 consecutive columns
 // of one output row) and reads and writes LDS 8 or 16 bytes at a time.
 //
-// One launch covers up to 4 problems (the shape groups of an optimizer step), see NsGemmMulti.
+// One launch covers up to 8 problems (the shape groups of an optimizer step), see NsGemmMulti.
 //
 // Accumulation order per output element is the same in every tile configuration and in the
 // 128x128 kernel of ns.hip (terms in order, k ascending, one accumulator).
@@ -266,6 +266,10 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     int left = t;
     while (left >= tm / R + 1) { left -= tm / R + 1; ++tm; }
     tn = left;
+  } else if (VAR == VAR_PLAIN && p.blk_r > 0) {
+    const int per = p.blk_r * p.blk_c, b = t / per, i = t % per, across = p.tiles_n / p.blk_c;
+    tm = (b / across) * p.blk_r + i / p.blk_c;
+    tn = (b % across) * p.blk_c + i % p.blk_c;
   } else {
     tm = t / p.tiles_n;
     tn = t % p.tiles_n;
@@ -871,6 +875,21 @@ int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_
     pm.g[k].tiles_m = ps[k].M / 128;
     pm.g[k].tiles_n = ps[k].N / 256;
     pm.g[k].lower = 0;
+    // Every XCD runs a contiguous eighth of the problem's tile sequence and has an L2 of its
+    // own: cut the tile grid into gx x gy = 8 blocks and walk it block by block, choosing the
+    // cut whose blocks need the fewest operand bytes (128 rows of A per tile row, 256 columns
+    // of B per tile column); then every operand byte is fetched by 8/gx or 8/gy XCDs, not 8.
+    {
+      const int tmk = pm.g[k].tiles_m, tnk = pm.g[k].tiles_n;
+      int best = 0;
+      pm.g[k].blk_r = pm.g[k].blk_c = 0;
+      for (int gx = 1; gx <= 8; gx *= 2) {
+        const int gy = 8 / gx;
+        if (tmk % gx != 0 || tnk % gy != 0) continue;
+        const int cost = 128 * (tmk / gx) + 256 * (tnk / gy);
+        if (best == 0 || cost < best) { best = cost; pm.g[k].blk_r = tmk / gx; pm.g[k].blk_c = tnk / gy; }
+      }
+    }
     const int64_t t = Es[k] * (int64_t)pm.g[k].tiles_m * pm.g[k].tiles_n;
     ANC_REQUIRE(t > 0 && t < (1ll << 30), "anc_ns_gemm_big_plain: grid out of range");
     pm.tiles[k] = (int)t;

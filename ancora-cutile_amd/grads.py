@@ -3,10 +3,15 @@ step reads.
 
 Mirror of `ResidentLayerTrain._dW` (ancora/model/resident_train.py:285-287), which launches
 `_gemm_dW` or, with gradient accumulation, `_gemm_dW_acc` (ancora/kernels/fused.py:190-219) once
-per weight: x (T, K) and dy (T, N) bf16 bits, dW (K, N) fp32. Here up to 4 weights go into one
+per weight: x (T, K) and dy (T, N) bf16 bits, dW (K, N) fp32. Here up to 8 weights go into one
 call (`gemm_dW`), the activations are passed transposed (`transpose_acts`, once per group of
 weights that share them), and the call can also leave the bf16 copy of the finished gradient,
 which is what `HybridOptimizer(grad_dtype=np.uint16)` reads.
+
+The token axis is cut into `segments` pieces so that a call fills the GPU (512 workgroups of
+128x256 outputs). By default every problem gets the number of pieces its shape needs to do that
+alone; a caller that hands over the 7 weights of a whole layer in one call passes `segments=1`
+(480 workgroups at Qwen3-0.6B shapes) and saves the partial tiles' traffic.
 """
 import ctypes
 
@@ -16,7 +21,7 @@ from . import _lib
 from ._lib import api, DwProblem
 from .devbuf import DevBuf
 
-MAX_PER_CALL = 4
+MAX_PER_CALL = 8
 
 
 def dw_workspace_bytes(T, K, N):
@@ -57,21 +62,34 @@ class DwWorkspace:
             self.buf = None
 
 
-def gemm_dW(problems, si=0):
+def gemm_dW(problems, si=0, segments=None):
     """problems: list of dicts {xT, dy, dW: DevBuf; T, K, N: int; workspace: DwWorkspace;
     g16: DevBuf or None; accumulate: bool; gn_partials: int device address or None (where the
-    grad-norm partial sums of this gradient go, `StepGuard.partials_ptr`)}. dW (+)= x^T dy for
-    each, 4 per launch. Asynchronous on stream `si`."""
+    grad-norm partial sums of this gradient go, `StepGuard.partials_ptr`); segments: int, optional}.
+    dW (+)= x^T dy for each, 8 per launch. `segments` (argument, or per problem) fixes the number
+    of token segments; None / 0 = the shape rule (a function of T, K, N alone); "fill" = per
+    launch, the largest power of two that keeps the launch within the 512 workgroups the GPU runs
+    at once (so it depends on what shares the call). The result's bits depend on the number of
+    segments and on nothing else. Asynchronous on stream `si`."""
     _lib.init()
     for i0 in range(0, len(problems), MAX_PER_CALL):
         group = problems[i0:i0 + MAX_PER_CALL]
+        fill = 0
+        if segments == "fill":
+            tiles = sum((int(p["K"]) // 128) * (int(p["N"]) // 256) for p in group)
+            tmin = min(int(p["T"]) for p in group)
+            fill = 1
+            while tiles * fill * 2 <= 512 and all(int(p["T"]) % (fill * 2 * 32) == 0 for p in group) \
+                    and tmin // (fill * 2) >= 256:
+                fill *= 2
         arr = (DwProblem * len(group))()
         for k, p in enumerate(group):
             T, K, N = int(p["T"]), int(p["K"]), int(p["N"])
-            nb = dw_workspace_bytes(T, K, N)
+            S = int(p.get("segments") or fill or (0 if segments == "fill" else segments) or 0)
+            nb = S * K * N * 4 if S > 0 else dw_workspace_bytes(T, K, N)
             ws = p["workspace"].ensure(nb)
             g16 = p.get("g16")
             arr[k] = DwProblem(p["xT"].ptr, p["dy"].ptr, p["dW"].ptr, 0 if g16 is None else g16.ptr, ws.ptr,
-                               T, K, N, ws.nbytes, int(bool(p.get("accumulate", False))), 0,
+                               T, K, N, ws.nbytes, int(bool(p.get("accumulate", False))), S,
                                int(p.get("gn_partials") or 0))
         api.anc_gemm_dw_multi(arr, len(group), int(si))

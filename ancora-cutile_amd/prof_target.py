@@ -8,7 +8,8 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
     python3 -m ancora_cutile_amd.prof_target gradnorm NUMEL [calls]      grad-norm partials + finalize
     python3 -m ancora_cutile_amd.prof_target quant K N E [cm] [calls]    MXFP8 weight re-quantisation
                                       (prints GB/s from HIP events around the calls)
-    python3 -m ancora_cutile_amd.prof_target dw T K N1[,N2,..] [calls]   weight-gradient GEMM of up to 4
+    python3 -m ancora_cutile_amd.prof_target dwlayer [T] [calls]         weight-gradient GEMMs of one layer in one call
+    python3 -m ancora_cutile_amd.prof_target dw T K N1[,N2,..] [calls]   weight-gradient GEMM of up to 8
                                       weights (K, Ni) that share the activations, T tokens
     python3 -m ancora_cutile_amd.prof_target kloop                       the GEMM K loop alone on cache-resident
                                       operands (anc_probe_kloop), 8 and 4 wavefronts per workgroup
@@ -107,6 +108,31 @@ def main(argv):
         gms, rms = pr["dw_gemm"][0] / calls, pr["dw_reduce"][0] / calls
         print(f"dW T={T} K={K} N={Ns} segments={[dw_info(T, K, N)[1] for N in Ns]}: gemm {gms * 1e3:.1f} us "
               f"({fl / gms / 1e9:.1f} TFLOP/s), reduce {rms * 1e3:.1f} us, together {fl / (gms + rms) / 1e9:.1f} TFLOP/s")
+    elif what == "dwlayer":
+        # the 7 weights of one Qwen3-0.6B layer in one call, one token segment each
+        from .grads import gemm_dW, DwWorkspace, dw_info
+        T = int(argv[1]) if len(argv) > 1 else 8192
+        calls = int(argv[2]) if len(argv) > 2 else 5
+        rng = np.random.default_rng(0)
+        bits = lambda a: (a.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        probs, fl = [], 0.0
+        for K, Ns in ((1024, (2048, 1024, 1024)), (2048, (1024,)), (1024, (3072, 3072)), (3072, (1024,))):
+            xT = DevBuf(bits(0.1 * rng.standard_normal((K, T))))
+            for N in Ns:
+                probs.append(dict(xT=xT, dy=DevBuf(bits(0.1 * rng.standard_normal((T, N)))),
+                                  dW=DevBuf.zeros((K, N), np.float32), g16=DevBuf.zeros((K, N), np.uint16),
+                                  T=T, K=K, N=N, workspace=DwWorkspace(), accumulate=True))
+                fl += dw_info(T, K, N)[0]
+        gemm_dW(probs, 0, segments=1)
+        _lib.stream_sync(0)
+        _lib.profile_enable(True)
+        for _ in range(calls):
+            gemm_dW(probs, 0, segments=1)
+        pr = _lib.profile_read()
+        _lib.profile_enable(False)
+        gms, rms = pr["dw_gemm"][0] / calls, pr["dw_reduce"][0] / calls
+        print(f"dW of one layer (7 weights, T={T}, 1 segment, 480 workgroups): gemm {gms * 1e3:.1f} us "
+              f"({fl / gms / 1e9:.1f} TFLOP/s), finish {rms * 1e3:.1f} us, together {fl / (gms + rms) / 1e9:.1f} TFLOP/s")
     elif what == "kloop":
         src = DevBuf.zeros((1 << 29,), np.float32)          # 2 GiB
         sink = DevBuf.zeros((512,), np.float32)

@@ -148,9 +148,11 @@ def side_workload(args):
                "data": "synthetic", "config": {"workload": "ns-196-matrices", "groups": [list(g) for g in groups]},
                "modes": res}
     elif args.workload == "dw":
-        # the weight-gradient GEMMs of the 28 Qwen3-0.6B layers at `--tokens` tokens per micro-batch,
-        # launched as the backward pass would: per layer [q,k,v] (shared activations), [o],
-        # [gate,up] (shared), [down]; buffers of one layer reused for all layers
+        # the weight-gradient GEMMs of the 28 Qwen3-0.6B layers at `--tokens` tokens per micro-batch;
+        # buffers of one layer reused for all layers. --dw-launch layer: one call per layer with
+        # its 7 weights, one token segment each (480 workgroups); group: as the backward pass
+        # reaches them, per layer [q,k,v] (shared activations), [o], [gate,up] (shared), [down],
+        # every weight cut into the token segments that let it fill the GPU alone
         from ancora_cutile_amd.grads import gemm_dW, DwWorkspace, dw_info
         from ancora_cutile_amd.bf16 import bf16_bits
         T = args.tokens
@@ -167,11 +169,15 @@ def side_workload(args):
                 flops += dw_info(T, K, N)[0]
             calls.append(probs)
         layers = 28
+        per_layer = [p for probs in calls for p in probs]
 
         def step():
             for _ in range(layers):
-                for probs in calls:
-                    gemm_dW(probs, 0)
+                if args.dw_launch == "layer":
+                    gemm_dW(per_layer, 0, segments=1)
+                else:
+                    for probs in calls:
+                        gemm_dW(probs, 0, segments="fill" if args.dw_launch == "group-fill" else None)
         for _ in range(max(1, args.warmup // 2)):
             step()
         e0.record(0)
@@ -193,7 +199,10 @@ def side_workload(args):
                "ms_per_step": round(ms, 3), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
                "dtype": "bf16", "data": "synthetic",
                "config": {"workload": "qwen3-0.6b-weight-gradients", "tokens": T, "weights": 7 * layers,
-                          "params": nparams, "launch_groups_per_layer": 4, "accumulate": True, "bf16_copy": True},
+                          "params": nparams, "launch": args.dw_launch,
+                          "launches_per_layer": 1 if args.dw_launch == "layer" else 4,
+                          "token_segments": {"layer": 1, "group": "shape rule", "group-fill": "per launch, <= 512 workgroups"}[args.dw_launch],
+                          "accumulate": True, "bf16_copy": True},
                "roofline": {"bound": "mfma", "achieved": round(gtf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                             "frac": round(gtf / PEAK_BF16_TFLOPS, 4), "traffic": None,
                             "kernel": "k_ns_gemm_big<EPI_BX, ..., VAR_PLAIN> (partial tiles of x^T dy)",
@@ -257,6 +266,8 @@ def main():
     ap.add_argument("--layers", type=int, default=28, help=argparse.SUPPRESS)   # smaller sets for debugging
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens per micro-batch of --workload dw")
+    ap.add_argument("--dw-launch", default="layer", choices=("layer", "group", "group-fill"),
+                    help="--workload dw: one call per layer (7 weights, 1 token segment) or 4 calls per layer")
     ap.add_argument("--workload", default="qwen3", choices=("qwen3", "moe", "ns", "adamw", "dw"),
                     help="qwen3: the headline hybrid step (default). moe: the 16-layer MoE family "
                          "(config 4). ns: the 196-matrix Newton-Schulz stress, bf16 and fp32 modes "

@@ -290,22 +290,25 @@ int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
                        uint64_t stream);
 
 /* ------------------------------------------------------ weight gradients ----
- * dW (+)= x^T dy for up to 4 weights per call: replaces `_gemm_dW` / `_gemm_dW_acc`
+ * dW (+)= x^T dy for up to 8 weights per call: replaces `_gemm_dW` / `_gemm_dW_acc`
  * (ancora/kernels/fused.py:190-219, launched per weight at ancora/model/resident_train.py:285-287),
  * the producer of the fp32 gradients the optimizer step reads. xT is the activation matrix
  * transposed, (K, T) bf16 row-major (anc_transpose_bf16 of the (T, K) activations, once per group
  * of weights that share them); dy is (T, N) bf16; dW (K, N) fp32 is overwritten, or added onto when
  * `accumulate` is set (micro-batch accumulation in place); g16, if not 0, receives the bf16 copy
  * (RNE) of the final dW, the format the step reads. fp32 accumulation in a fixed order: the token
- * axis is cut into anc_gemm_dw_info's `segments` pieces that depend on (T, K, N) only, each tile
- * of each piece is one workgroup's whole K loop, and the pieces are added in ascending order, so
- * the bits do not depend on what else is in the call. T % 32, K % 128, N % 256 == 0 (the reference:
- * all % 64); pointers 16-byte aligned; workspace of anc_gemm_dw_workspace_bytes(T, K, N) bytes per
- * problem (the partial tiles), not shared between the problems of a call. g16 16-byte aligned. */
+ * axis is cut into S equal pieces, each tile of each piece is one workgroup's whole K loop, and
+ * the pieces are added in ascending order, so the bits depend on S but not on what else is in the
+ * call. S = `segments` if > 0 (T must be a multiple of 32 S; a call that carries a whole layer's
+ * weights fills the GPU with S = 1), else anc_gemm_dw_info's shape rule, which makes a problem
+ * fill the GPU by itself. T % 32, K % 128, N % 256 == 0 (the reference: all % 64); pointers
+ * 16-byte aligned; workspace of S * K * N * 4 bytes per problem (the partial tiles;
+ * anc_gemm_dw_workspace_bytes(T, K, N) for the shape rule), not shared between the problems of a
+ * call. g16 16-byte aligned. */
 typedef struct {
   uint64_t xT, dy, dW, g16, workspace;
   int64_t  T, K, N, workspace_bytes;
-  int32_t  accumulate, reserved;
+  int32_t  accumulate, segments;
   uint64_t gn_partials;        /* 0, or double[K*N / ANC_GN_CHUNK]: the grad-norm partial sums of this
                                   gradient (of its bf16 copy if g16 is set), bit-identical to what
                                   anc_gradnorm_partials would compute from the stored gradient, so
@@ -384,7 +387,7 @@ int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partials, int64_t
  * CUs stay busy where per-batch launches would each end in a partly filled last wave of
  * workgroups. No reference counterpart (the reference runs its shape groups one after the
  * other, ancora/optim/muon.py:257-277). Results equal anc_ns_batched_pair on each batch bit
- * for bit. n_probs <= 4; every M and N a multiple of 256; steps >= 2; bf16 modes. */
+ * for bit. n_probs <= 8; every M and N a multiple of 256; steps >= 2; bf16 modes. */
 typedef struct {
   uint64_t Uh, Ul;            /* input bf16 pair, (E,M,N) each                        */
   uint64_t fro_partials;      /* n_partials sums of u*u per matrix                     */

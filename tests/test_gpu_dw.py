@@ -102,6 +102,52 @@ def test_grouping_does_not_change_bits(gpu):
         _free(p)
 
 
+def test_whole_layer_in_one_call_with_explicit_segments(gpu):
+    """Seven weights of four shapes in one call, one token segment each (the launch a caller makes
+    who collects a layer's gradient GEMMs), against the fp64 product; a weight's bits are the
+    same alone and in the group, equal to the shape rule's when that also gives one segment, and
+    2 and 4 segments stay within the same error."""
+    from ancora_cutile_amd.grads import gemm_dW, dw_info
+    T = 512
+    shapes = [(256, 512), (256, 256), (256, 256), (512, 256), (256, 768), (256, 768), (768, 256)]
+    xs, ps = {}, []
+    for i, (K, N) in enumerate(shapes):
+        x, dy = _inputs(T, K, N, 40 + i)
+        ps.append(_problem(x, dy, T, K, N, emit=True))
+        xs[i] = (x, dy)
+    gemm_dW(ps, segments=1)
+    outs = [p["dW"].to_numpy() for p in ps]
+    for i, (K, N) in enumerate(shapes):
+        assert rel_fro(outs[i], gemm_dw(*xs[i])) < 2e-5
+        assert bits_equal(ps[i]["g16"].to_numpy(), bf16_rne_bits(outs[i]).reshape(K, N))
+    for i in (0, 6):
+        K, N = shapes[i]
+        q = _problem(xs[i][0], xs[i][1], T, K, N)
+        gemm_dW([q], segments=1)
+        assert bits_equal(q["dW"].to_numpy(), outs[i])
+        for S in (2, 4):
+            gemm_dW([q], segments=S)
+            assert rel_fro(q["dW"].to_numpy(), gemm_dw(*xs[i])) < 2e-5
+        q["segments"] = 2                       # per problem, and again: same bits
+        gemm_dW([q])
+        a = q["dW"].to_numpy()
+        gemm_dW([q], segments=2)
+        assert bits_equal(q["dW"].to_numpy(), a)
+        _free(q)
+    # shape rule with one segment == explicit one segment
+    K, N = 2048, 4096
+    assert dw_info(64, K, N)[1] == 1
+    x, dy = _inputs(64, K, N, 50)
+    q = _problem(x, dy, 64, K, N)
+    gemm_dW([q])
+    a = q["dW"].to_numpy()
+    gemm_dW([q], segments=1)
+    assert bits_equal(q["dW"].to_numpy(), a)
+    _free(q)
+    for p in ps:
+        _free(p)
+
+
 def test_shape_checks(gpu):
     from ancora_cutile_amd import _lib
     from ancora_cutile_amd.grads import dw_workspace_bytes
@@ -110,6 +156,12 @@ def test_shape_checks(gpu):
     with pytest.raises(_lib.AncoraError):
         dw_workspace_bytes(128, 64, 256)
     assert dw_workspace_bytes(64, 128, 256) == 128 * 256 * 4
+    from ancora_cutile_amd.grads import gemm_dW
+    x, dy = _inputs(64, 128, 256, 1)
+    q = _problem(x, dy, 64, 128, 256)
+    with pytest.raises(_lib.AncoraError):
+        gemm_dW([q], segments=4)                # 64 tokens do not split into 4 x 32k
+    _free(q)
 
 
 def test_producer_writes_the_grad_norm_partials(gpu):
