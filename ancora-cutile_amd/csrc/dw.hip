@@ -124,14 +124,19 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
   for (int q = 0; q < n_probs; ++q) {
     const anc_dw_problem_t &b = probs[q];
     if (int rc = check_dw(b, "anc_gemm_dw_multi")) return rc;
-    ANC_REQUIRE(b.xT != 0 && b.dy != 0 && b.dW != 0 && b.workspace != 0 &&
-                ((b.xT | b.dy | b.dW | b.workspace | b.g16) & 15) == 0 && (b.gn_partials & 7) == 0,
-                "anc_gemm_dw_multi: null or misaligned pointer");
     const int S = b.segments > 0 ? b.segments : dw_segments(b.T, b.K, b.N);
     ANC_REQUIRE(b.segments >= 0 && S <= 256 && b.T % ((int64_t)S * 32) == 0,
                 "anc_gemm_dw_multi: segments=%d must be 0 (shape rule) or divide T=%lld into multiples of 32 tokens",
                 (int)b.segments, (long long)b.T);
-    ANC_REQUIRE(b.workspace_bytes >= (int64_t)S * b.K * b.N * 4, "anc_gemm_dw_multi: workspace holds %lld bytes, %lld needed",
+    // One segment and no grad-norm sums wanted: the GEMM's epilogue finishes the gradient itself
+    // (old dW or 0 + product, bf16 copy), no partial tile and no second kernel. Same bits as
+    // the two-kernel route: one fp32 addition per element onto the same accumulator value.
+    const bool direct = S == 1 && b.gn_partials == 0;
+    ANC_REQUIRE(b.xT != 0 && b.dy != 0 && b.dW != 0 && (direct || b.workspace != 0) &&
+                ((b.xT | b.dy | b.dW | b.workspace | b.g16) & 15) == 0 && (b.gn_partials & 7) == 0,
+                "anc_gemm_dw_multi: null or misaligned pointer");
+    ANC_REQUIRE(direct || b.workspace_bytes >= (int64_t)S * b.K * b.N * 4,
+                "anc_gemm_dw_multi: workspace holds %lld bytes, %lld needed",
                 (long long)b.workspace_bytes, (long long)S * b.K * b.N * 4);
     const int64_t seg = b.T / S;
     NsGemm p{};
@@ -145,12 +150,18 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
     p.M = (int)b.K;
     p.N = (int)b.N;
     p.X32 = (float *)b.workspace;    // partial e at e * K * N
+    if (direct) {
+      p.plain_sum = 1;
+      p.X32 = (float *)b.dW;
+      p.A32 = b.accumulate ? (float *)b.dW : nullptr;
+      p.Yh = (uint16_t *)b.g16;
+    }
     g[q] = p;
     Es[q] = S;
     rm.r[q] = DwReduce{(const float *)b.workspace, (float *)b.dW, (uint16_t *)b.g16, (double *)b.gn_partials,
                        b.K * b.N, S, b.accumulate ? 1 : 0};
     rm.blk0[q] = blocks;
-    blocks += b.K * b.N / ANC_GN_CHUNK;            // K % 128 and N % 256: whole chunks only
+    if (!direct) blocks += b.K * b.N / ANC_GN_CHUNK;     // K % 128 and N % 256: whole chunks only
   }
   rm.blk0[n_probs] = blocks;
   ANC_REQUIRE(blocks < (1ll << 31), "anc_gemm_dw_multi: too large");
@@ -158,7 +169,7 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
     AncProfScope prof(ANC_PROF_DW_GEMM, s);
     if (int rc = anc_ns_gemm_big_plain(g, Es, n_probs, s)) return rc;
   }
-  {
+  if (blocks > 0) {
     AncProfScope prof(ANC_PROF_DW_REDUCE, s);
     hipLaunchKernelGGL(k_dw_reduce, dim3((unsigned)blocks), dim3(kThreads), 0, s, rm);
   }

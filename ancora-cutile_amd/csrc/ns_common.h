@@ -60,6 +60,8 @@ struct NsGemm {
   int64_t strideA, strideB;  // elements between consecutive matrices
   int tiles_m, tiles_n;
   int lower;                 // symmetric output: tiles with tn <= tm only, mirrored
+  int plain_sum;             // plain product: 1 = write X32 = (A32, if not null, else 0) + A B and, if Yh is
+                             // not null, its bf16 copy (RNE) to Yh; 0 = write X32 = A B
   int blk_r, blk_c;          // plain product: the tile sequence of a matrix runs block by block, blocks of
                              // blk_r x blk_c tiles (rows x columns), so that the contiguous eighth of it that
                              // lands on one XCD is a compact patch of the output; 0 = row by row

@@ -213,7 +213,8 @@ __device__ __forceinline__ void lds_barrier() {
 // VAR (X = a X + B X only) selects a variant of the epilogue as its own instantiation, so that
 // the extra registers and branches do not weigh on the other launches: VAR_UPDATE applies the
 // weight update; VAR_PLAIN is the bare product C = A B written as fp32 (no iterate at the output
-// position, no row scaling), which the weight-gradient GEMM uses.
+// position, no row scaling), which the weight-gradient GEMM uses; with `plain_sum` set it writes
+// C = (A32 or 0) + A B and, if Yh is set, the bf16 copy of C.
 enum { VAR_NONE = 0, VAR_UPDATE = 1, VAR_PLAIN = 2 };
 template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS, int VAR = VAR_NONE>
 __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemmMulti pm) {
@@ -558,6 +559,15 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #pragma unroll
         for (int pz = 0; pz < 8; ++pz) pv[pz] = anc_ld_stream((const anc_f32x4 *)(W32 + w_off(gi0, pz)));
       }
+      // Plain product with an addend (C = A32 + A B, in place when A32 == X32): same early request
+      const bool plain_add = plain && p.plain_sum && p.A32 != nullptr;
+      if (plain_add) {
+#pragma unroll
+        for (int pz = 0; pz < 8; ++pz) {
+          const int idx = pz * 64 + lane;
+          pv[pz] = anc_ld_stream((const anc_f32x4 *)(p.A32 + mn + (int64_t)(gi0 + (idx >> 4)) * N + gj0w + (idx & 15) * 4));
+        }
+      }
       // Wait for this slab's DMA only. Vector memory operations complete in issue order; after
       // the fetch of slab bi this wavefront issued the 8 row stores of slab bi-1 and the fetch
       // of slab bi+1 (8 DMA); in the fused update the stores of a slab are 8 (master) + 8 (bf16
@@ -612,7 +622,23 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           }
         __builtin_amdgcn_s_waitcnt(0xC07F);
         __builtin_amdgcn_wave_barrier();
-        if (!fused) {
+        if (plain && p.plain_sum) {
+          // C = (A32 or 0) + A B, and its bf16 copy (round to nearest even) if Yh is set
+#pragma unroll
+          for (int pz = 0; pz < 8; ++pz) {
+            const int idx = pz * 64 + lane, row = idx >> 4, c = idx & 15;
+            const anc_f32x4 v4 = *(const anc_f32x4 *)(b + row * 256 + ((c ^ (row & 15)) * 16));
+            const anc_f32x4 a4 = plain_add ? pv[pz] : anc_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            const anc_f32x4 o4 = {a4.x + v4.x, a4.y + v4.y, a4.z + v4.z, a4.w + v4.w};
+            const int64_t off = mn + (int64_t)(gi0 + row) * N + gj0w + c * 4;
+            epi_st((anc_f32x4 *)(p.X32 + off), o4);
+            if (p.Yh != nullptr) {
+              const anc_u32x2 ho = {(anc_bf16_rne_bits(o4.x) & 0xFFFFu) | (anc_bf16_rne_bits(o4.y) << 16),
+                                    (anc_bf16_rne_bits(o4.z) & 0xFFFFu) | (anc_bf16_rne_bits(o4.w) << 16)};
+              epi_st((anc_u32x2 *)(p.Yh + off), ho);
+            }
+          }
+        } else if (!fused) {
 #pragma unroll
           for (int pz = 0; pz < 8; ++pz) {
             const int idx = pz * 64 + lane, row = idx >> 4, c = idx & 15;
@@ -869,7 +895,8 @@ int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_
   for (int k = 0; k < n; ++k) {
     ANC_REQUIRE(ps[k].M % 128 == 0 && ps[k].N % 256 == 0 && ps[k].K % 32 == 0 && ps[k].K >= 32,
                 "anc_ns_gemm_big_plain: needs M % 128 == 0, N % 256 == 0, K % 32 == 0");
-    ANC_REQUIRE(ps[k].X32 != nullptr && ps[k].nterms == 1 && ps[k].scale == nullptr && ps[k].upd == nullptr,
+    ANC_REQUIRE(ps[k].X32 != nullptr && ps[k].nterms == 1 && ps[k].scale == nullptr && ps[k].upd == nullptr &&
+                (ps[k].plain_sum || (ps[k].A32 == nullptr && ps[k].Yh == nullptr)),
                 "anc_ns_gemm_big_plain: bad problem");
     pm.g[k] = ps[k];
     pm.g[k].tiles_m = ps[k].M / 128;

@@ -86,10 +86,13 @@ def gemm_dW(problems, si=0, segments=None):
         for k, p in enumerate(group):
             T, K, N = int(p["T"]), int(p["K"]), int(p["N"])
             S = int(p.get("segments") or fill or (0 if segments == "fill" else segments) or 0)
-            nb = S * K * N * 4 if S > 0 else dw_workspace_bytes(T, K, N)
-            ws = p["workspace"].ensure(nb)
+            gn = int(p.get("gn_partials") or 0)
+            if S == 1 and gn == 0:                 # finished by the GEMM's epilogue: no partial tiles
+                ws_ptr = ws_bytes = 0
+            else:
+                ws = p["workspace"].ensure(S * K * N * 4 if S > 0 else dw_workspace_bytes(T, K, N))
+                ws_ptr, ws_bytes = ws.ptr, ws.nbytes
             g16 = p.get("g16")
-            arr[k] = DwProblem(p["xT"].ptr, p["dy"].ptr, p["dW"].ptr, 0 if g16 is None else g16.ptr, ws.ptr,
-                               T, K, N, ws.nbytes, int(bool(p.get("accumulate", False))), S,
-                               int(p.get("gn_partials") or 0))
+            arr[k] = DwProblem(p["xT"].ptr, p["dy"].ptr, p["dW"].ptr, 0 if g16 is None else g16.ptr, ws_ptr,
+                               T, K, N, ws_bytes, int(bool(p.get("accumulate", False))), S, gn)
         api.anc_gemm_dw_multi(arr, len(group), int(si))

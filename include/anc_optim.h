@@ -304,7 +304,9 @@ int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
  * fill the GPU by itself. T % 32, K % 128, N % 256 == 0 (the reference: all % 64); pointers
  * 16-byte aligned; workspace of S * K * N * 4 bytes per problem (the partial tiles;
  * anc_gemm_dw_workspace_bytes(T, K, N) for the shape rule), not shared between the problems of a
- * call. g16 16-byte aligned. */
+ * call. g16 16-byte aligned. With S = 1 and gn_partials = 0 the GEMM's epilogue adds onto dW and
+ * writes g16 itself: no second kernel runs and no workspace is needed (workspace may be 0); the
+ * bits are those of the two-kernel route. */
 typedef struct {
   uint64_t xT, dy, dW, g16, workspace;
   int64_t  T, K, N, workspace_bytes;

@@ -148,6 +148,38 @@ def test_whole_layer_in_one_call_with_explicit_segments(gpu):
         _free(p)
 
 
+def test_one_segment_route_through_the_epilogue_has_the_two_kernel_bits(gpu):
+    """With one token segment and no grad-norm sums asked for, the GEMM's epilogue adds onto dW and
+    writes the bf16 copy itself; asking for the sums sends the same problem through the partial
+    tile and the finishing kernel. Same bits either way, with and without accumulation."""
+    from ancora_cutile_amd import DevBuf
+    from ancora_cutile_amd.grads import gemm_dW
+    T, K, N = 512, 256, 768
+    x, dy = _inputs(T, K, N, 60)
+    dW0 = (0.5 * np.random.default_rng(61).standard_normal((K, N))).astype(np.float32)
+    sums = DevBuf.zeros((K * N // 8192,), np.float64)
+    for prev in (None, dW0):
+        a = _problem(x, dy, T, K, N, emit=True, dW0=prev)
+        b = _problem(x, dy, T, K, N, emit=True, dW0=prev)
+        b["gn_partials"] = sums.ptr
+        gemm_dW([a], segments=1)
+        gemm_dW([b], segments=1)
+        assert a["workspace"].buf is None and b["workspace"].buf is not None
+        assert bits_equal(a["dW"].to_numpy(), b["dW"].to_numpy())
+        assert bits_equal(a["g16"].to_numpy(), b["g16"].to_numpy())
+        assert rel_fro(a["dW"].to_numpy(), gemm_dw(x, dy, prev)) < 2e-5
+        _free(a); _free(b)
+    # all-zero activations: the product is +0 on both routes
+    z = np.zeros_like(x)
+    a, b = _problem(z, dy, T, K, N), _problem(z, dy, T, K, N)
+    b["gn_partials"] = sums.ptr
+    gemm_dW([a], segments=1)
+    gemm_dW([b], segments=1)
+    assert bits_equal(a["dW"].to_numpy(), b["dW"].to_numpy()) and not a["dW"].to_numpy().any()
+    _free(a); _free(b)
+    sums.free()
+
+
 def test_shape_checks(gpu):
     from ancora_cutile_amd import _lib
     from ancora_cutile_amd.grads import dw_workspace_bytes
