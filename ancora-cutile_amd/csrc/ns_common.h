@@ -63,8 +63,8 @@ struct NsGemm {
   int plain_sum;             // plain product: 1 = write X32 = (A32, if not null, else 0) + A B and, if Yh is
                              // not null, its bf16 copy (RNE) to Yh; 0 = write X32 = A B
   int blk_r, blk_c;          // plain product: the tile sequence of a matrix runs block by block, blocks of
-                             // blk_r x blk_c tiles (rows x columns), so that the contiguous eighth of it that
-                             // lands on one XCD is a compact patch of the output; 0 = row by row
+                             // blk_r x blk_c tiles (rows x columns): (tiles_m, 1) = column panel by column
+                             // panel, (1, tiles_n) or 0 = row by row
   int M, N;                  // matrix dims of the chain (A, B are MxM; X is MxN)
   float ca, cb, cc;
   float *A32;                // (E,M,M) fp32 A            GRAM out, BMAT in
@@ -94,6 +94,7 @@ struct NsGemm {
 constexpr int kMaxGroups = ANC_MAX_GROUPS;
 struct NsGemmMulti {
   int n;
+  int seq;                   // plain product: 1 = anc_seq_tile dealing, 0 = anc_group_tile
   int tiles[kMaxGroups];
   NsGemm g[kMaxGroups];
   // fused weight update (problems with `upd` set): lr*shape_scale by descriptor scale index,
@@ -131,6 +132,17 @@ __device__ __forceinline__ void anc_group_tile(const NsGemmMulti &pm, int bid, i
       }
       pos -= c;
     }
+}
+
+// The other dealing: the problems' tile sequences one after the other, cut into 8 contiguous runs,
+// one per XCD. An XCD then works on one or two problems only and fetches their operands into its
+// L2 once, where the dealing above makes every XCD fetch a part of every problem's operands. For
+// launches whose tiles all cost the same (the plain product: one K length).
+__device__ __forceinline__ void anc_seq_tile(const NsGemmMulti &pm, int bid, int grid, int &g, int &L) {
+  int pos = xcd_remap(bid, grid);
+  g = 0;
+  while (g + 1 < pm.n && pos >= pm.tiles[g]) { pos -= pm.tiles[g]; ++g; }
+  L = pos;
 }
 
 // 256x256-tile kernel (ns_gemm_big.hip): same products, same accumulation order and

@@ -246,7 +246,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const unsigned long long dbg_t0 = wall_clock64();
 #endif
   int gsel, L;
-  anc_group_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
+  if (VAR == VAR_PLAIN && pm.seq) anc_seq_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
+  else anc_group_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
   const NsGemm &p = pm.g[gsel];
   // Symmetric outputs: only tiles that reach the diagonal or lie below it. Row tm of TM-row
   // tiles has tm/R + 1 of them (R = TN/TM); a tile entirely below the diagonal is mirrored.
@@ -902,27 +903,39 @@ int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_
     pm.g[k].tiles_m = ps[k].M / 128;
     pm.g[k].tiles_n = ps[k].N / 256;
     pm.g[k].lower = 0;
-    // Every XCD runs a contiguous eighth of the problem's tile sequence and has an L2 of its
-    // own: cut the tile grid into gx x gy = 8 blocks and walk it block by block, choosing the
-    // cut whose blocks need the fewest operand bytes (128 rows of A per tile row, 256 columns
-    // of B per tile column); then every operand byte is fetched by 8/gx or 8/gy XCDs, not 8.
-    {
-      const int tmk = pm.g[k].tiles_m, tnk = pm.g[k].tiles_n;
-      int best = 0;
-      pm.g[k].blk_r = pm.g[k].blk_c = 0;
-      for (int gx = 1; gx <= 8; gx *= 2) {
-        const int gy = 8 / gx;
-        if (tmk % gx != 0 || tnk % gy != 0) continue;
-        const int cost = 128 * (tmk / gx) + 256 * (tnk / gy);
-        if (best == 0 || cost < best) { best = cost; pm.g[k].blk_r = tmk / gx; pm.g[k].blk_c = tnk / gy; }
-      }
-    }
     const int64_t t = Es[k] * (int64_t)pm.g[k].tiles_m * pm.g[k].tiles_n;
     ANC_REQUIRE(t > 0 && t < (1ll << 30), "anc_ns_gemm_big_plain: grid out of range");
     pm.tiles[k] = (int)t;
     grid += t;
   }
   ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big_plain: grid out of range");
+  // Every XCD has an L2 of its own, so which tiles it runs decides how often an operand byte is
+  // fetched from HBM. A launch that fits the GPU's 512 workgroup slots runs in one round: its
+  // problems' tile sequences are dealt one after the other (anc_seq_tile), an XCD works on one or
+  // two problems, and a problem's tile grid is walked along its smaller operand -- column panel by
+  // column panel when A = (M, K) is the smaller one, so that a run of tiles reads all of A once
+  // and only its own panels of B; row by row when B is. (One layer of Qwen3-0.6B weight
+  // gradients, 480 tiles: 744 MiB of HBM reads per launch; with an eighth of every problem on
+  // every XCD in row order 1800 MiB.) Larger launches measured better with an eighth of every
+  // problem on every XCD (anc_group_tile), each eighth a compact block of the tile grid: the grid
+  // cut 1x8, 2x4, 4x2 or 8x1, whichever needs the fewest operand bytes per block.
+  pm.seq = grid <= 512 ? 1 : 0;
+  for (int k = 0; k < n; ++k) {
+    NsGemm &g = pm.g[k];
+    if (pm.seq) {
+      if (g.M <= g.N) { g.blk_r = g.tiles_m; g.blk_c = 1; }
+      else { g.blk_r = 1; g.blk_c = g.tiles_n; }
+      continue;
+    }
+    int best = 0;
+    g.blk_r = g.blk_c = 0;
+    for (int gx = 1; gx <= 8; gx *= 2) {
+      const int gy = 8 / gx;
+      if (g.tiles_m % gx != 0 || g.tiles_n % gy != 0) continue;
+      const int cost = 128 * (g.tiles_m / gx) + 256 * (g.tiles_n / gy);
+      if (best == 0 || cost < best) { best = cost; g.blk_r = g.tiles_m / gx; g.blk_c = g.tiles_n / gy; }
+    }
+  }
   hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_PLAIN>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
