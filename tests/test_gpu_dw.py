@@ -134,6 +134,18 @@ def test_whole_layer_in_one_call_with_explicit_segments(gpu):
         gemm_dW([q], segments=2)
         assert bits_equal(q["dW"].to_numpy(), a)
         _free(q)
+    # the per-launch rule: 3 weights of 4 + 2 + 2 tiles at 512 tokens -> 2 segments of 256 tokens
+    for p3 in ps[:3]:
+        p3["dW"].upload(np.zeros(p3["dW"].shape, np.float32))
+    gemm_dW(ps[:3], segments="fill")
+    for i in range(3):
+        got = ps[i]["dW"].to_numpy()
+        assert rel_fro(got, gemm_dw(*xs[i])) < 2e-5
+        K, N = shapes[i]
+        q = _problem(xs[i][0], xs[i][1], T, K, N)
+        gemm_dW([q], segments=2)
+        assert bits_equal(q["dW"].to_numpy(), got)
+        _free(q)
     # shape rule with one segment == explicit one segment
     K, N = 2048, 4096
     assert dw_info(64, K, N)[1] == 1
