@@ -70,7 +70,8 @@ class DwProblem(C.Structure):
     """anc_dw_problem_t: one weight of the weight-gradient GEMM call."""
     _fields_ = [("xT", u64), ("dy", u64), ("dW", u64), ("g16", u64), ("workspace", u64),
                 ("T", i64), ("K", i64), ("N", i64), ("workspace_bytes", i64),
-                ("accumulate", i32), ("segments", i32), ("gn_partials", u64)]
+                ("accumulate", i32), ("segments", i32), ("gn_partials", u64),
+                ("x_row_major", i32), ("reserved", i32)]
 
 
 # name -> (restype, argtypes); restype None means "int status, checked".

@@ -4,8 +4,9 @@
 // ancora/model/resident_train.py:285-287): x (T, K) and dy (T, N) bf16, fp32 accumulation over the
 // T tokens, fp32 result, optionally added onto the existing dW (gradient accumulation in place).
 // Here the product runs on the Newton-Schulz chain's X = a X + B X K loop (128x256 tiles, bf16
-// MFMA, LDS-DMA stage ring): A = x^T (K, T) row-major -- the caller transposes the activations
-// once per group of weights that share them (anc_transpose_bf16) -- and B = dy as it lies.
+// MFMA, LDS-DMA stage ring): B = dy as it lies, and A either the activations as they lie, x (T, K)
+// (`x_row_major`: the A tile is then [tokens][128 columns] and its fragments come from transposing
+// LDS reads, like B's), or x^T (K, T) for a caller that keeps the activations transposed.
 //
 // A single weight is 50-200 tiles, far fewer than the 512 a launch needs to fill 256 CUs, and the
 // backward pass produces one layer's gradients at a time. So the token axis is cut into S
@@ -121,6 +122,7 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
   DwReduceMulti rm{};
   rm.count = n_probs;
   int64_t blocks = 0;
+  const bool tn = probs[0].x_row_major != 0;
   for (int q = 0; q < n_probs; ++q) {
     const anc_dw_problem_t &b = probs[q];
     if (int rc = check_dw(b, "anc_gemm_dw_multi")) return rc;
@@ -138,14 +140,15 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
     ANC_REQUIRE(direct || b.workspace_bytes >= (int64_t)S * b.K * b.N * 4,
                 "anc_gemm_dw_multi: workspace holds %lld bytes, %lld needed",
                 (long long)b.workspace_bytes, (long long)S * b.K * b.N * 4);
+    ANC_REQUIRE((b.x_row_major != 0) == tn, "anc_gemm_dw_multi: the problems of a call must agree on x_row_major");
     const int64_t seg = b.T / S;
     NsGemm p{};
     p.A[0] = (const uint16_t *)b.xT;
     p.B[0] = (const uint16_t *)b.dy;
     p.nterms = 1;
     p.K = (int)seg;
-    p.ldA = (int)b.T;
-    p.strideA = seg;                 // segment e starts seg elements further along every row of x^T
+    p.ldA = tn ? (int)b.K : (int)b.T;
+    p.strideA = tn ? seg * b.K : seg;  // segment e starts seg rows further down x / seg elements further along every row of x^T
     p.strideB = seg * b.N;           // and seg rows further down dy
     p.M = (int)b.K;
     p.N = (int)b.N;
@@ -167,7 +170,7 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
   ANC_REQUIRE(blocks < (1ll << 31), "anc_gemm_dw_multi: too large");
   {
     AncProfScope prof(ANC_PROF_DW_GEMM, s);
-    if (int rc = anc_ns_gemm_big_plain(g, Es, n_probs, s)) return rc;
+    if (int rc = anc_ns_gemm_big_plain(g, Es, n_probs, s, tn)) return rc;
   }
   if (blocks > 0) {
     AncProfScope prof(ANC_PROF_DW_REDUCE, s);

@@ -152,5 +152,6 @@ int anc_ns_gemm_big(int epi, const NsGemm &p, int64_t E, hipStream_t s);
 // `upd` (may be null) carries the scalars of the fused weight update for problems whose `upd` is set.
 int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s,
                           const NsUpdate *upd = nullptr);
-// Bare fp32 products C[e] = A[e] B[e] on the same K loop (ns_gemm_big.hip).
-int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s);
+// Bare fp32 products C[e] = A[e] B[e] on the same K loop (ns_gemm_big.hip); a_transposed: A is
+// given as (K, M) row-major with row pitch ldA (and strideA between matrices), C = A^T B.
+int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s, bool a_transposed = false);

@@ -214,8 +214,11 @@ __device__ __forceinline__ void lds_barrier() {
 // the extra registers and branches do not weigh on the other launches: VAR_UPDATE applies the
 // weight update; VAR_PLAIN is the bare product C = A B written as fp32 (no iterate at the output
 // position, no row scaling), which the weight-gradient GEMM uses; with `plain_sum` set it writes
-// C = (A32 or 0) + A B and, if Yh is set, the bf16 copy of C.
-enum { VAR_NONE = 0, VAR_UPDATE = 1, VAR_PLAIN = 2 };
+// C = (A32 or 0) + A B and, if Yh is set, the bf16 copy of C. VAR_PLAIN_TN is the same product
+// with A given transposed, (K, M) row-major with row pitch ldA (C = A^T B: the activations of a
+// weight-gradient GEMM as they lie): its A tile is [k][128 columns] like the B tile and its
+// fragments come from transposing LDS reads too.
+enum { VAR_NONE = 0, VAR_UPDATE = 1, VAR_PLAIN = 2, VAR_PLAIN_TN = 3 };
 template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS, int VAR = VAR_NONE>
 __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemmMulti pm) {
   constexpr int NWN = TN / 64, NWAVES = (TM / 128) * NWN;
@@ -246,7 +249,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const unsigned long long dbg_t0 = wall_clock64();
 #endif
   int gsel, L;
-  if (VAR == VAR_PLAIN && pm.seq) anc_seq_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
+  constexpr bool PLAINV = (VAR == VAR_PLAIN || VAR == VAR_PLAIN_TN);
+  constexpr bool AT = (VAR == VAR_PLAIN_TN);
+  if (PLAINV && pm.seq) anc_seq_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
   else anc_group_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
   const NsGemm &p = pm.g[gsel];
   // Symmetric outputs: only tiles that reach the diagonal or lie below it. Row tm of TM-row
@@ -268,7 +273,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     int left = t;
     while (left >= tm / R + 1) { left -= tm / R + 1; ++tm; }
     tn = left;
-  } else if (VAR == VAR_PLAIN && p.blk_r > 0) {
+  } else if (PLAINV && p.blk_r > 0) {
     const int per = p.blk_r * p.blk_c, b = t / per, i = t % per, across = p.tiles_n / p.blk_c;
     tm = (b / across) * p.blk_r + i / p.blk_c;
     tn = (b % across) * p.blk_c + i % p.blk_c;
@@ -292,7 +297,12 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const int key0 = (TK == 64) ? (lrow >> 1) : ((lrow >> 2) & 3);
   const uint32_t voff0 = (uint32_t)(lrow * ldA * 2 + ((pchunk ^ key0) * 16));
   const uint32_t voff1 = (uint32_t)(lrow * ldA * 2 + ((pchunk ^ key0 ^ (TK == 64 ? 4 : 0)) * 16));
-  const int64_t ubaseA = ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * (IA * RPI)) * ldA) * 2;   // bytes
+  // (k, m) A tile (AT): TK rows of TM*2 = 256 bytes, four rows per DMA instruction; lane -> (row
+  // lane/16, physical chunk lane%16), chunk index XORed with 4*(row&3) as for the B tile.
+  static_assert(!AT || (TM == 128 && IA * NWAVES * 4 == TK), "(k,m) tile layout");
+  const uint32_t voffAT = (uint32_t)((lane >> 4) * ldA * 2 + (((lane & 15) ^ ((lane >> 4) << 2)) * 16));
+  const int64_t ubaseA = AT ? ((int64_t)e * p.strideA + (int64_t)tm * TM + (int64_t)(wave * IA * 4) * ldA) * 2
+                            : ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * (IA * RPI)) * ldA) * 2;   // bytes
   const int64_t ubaseB = ((int64_t)e * p.strideB + (int64_t)(tn * TN + wave * (IB * RPI)) * K) * 2;
   // (k, n) B tile: TK rows of TN*2 = 512 bytes, two rows per DMA instruction; lane -> (row
   // lane/32, physical chunk lane%32); the chunk index is XORed with 4*(row&3), so that the 4
@@ -316,13 +326,14 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     Bbase[t3] = (const char *)p.B[t3] + (BT ? ubaseBT : ubaseB);
   }
   const int64_t advB = BT ? (int64_t)TK * ldn * 2 : (int64_t)ROWB;
+  const int64_t advA = AT ? (int64_t)TK * ldA * 2 : (int64_t)ROWB;
   const char *curA = Abase[0], *curB = Bbase[0];
   int is_kt = 0, is_term = 0;
   // DMA instruction i of a stage (0 .. IPS-1: the A tile's IA, then the B tile's IB)
   auto issue_piece = [&](int i, unsigned char *stage) {
     if (i < IA) {
-      const int64_t ro = (int64_t)(i * RPI) * ldA * 2;
-      const uint32_t vo = (i & 1) ? voff1 : voff0;
+      const int64_t ro = AT ? (int64_t)(i * 4) * ldA * 2 : (int64_t)(i * RPI) * ldA * 2;
+      const uint32_t vo = AT ? voffAT : ((i & 1) ? voff1 : voff0);
       dma16(curA + ro + vo, lds_addr(stage + (wave * IA + i) * 1024));
     } else {
       const int j = i - IA;
@@ -332,7 +343,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     }
   };
   auto issue_advance = [&]() {
-    curA += ROWB;
+    curA += advA;
     curB += advB;
     if (++is_kt == nk) {
       is_kt = 0;
@@ -364,8 +375,24 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       tb[bj] = TM * ROWB + (8 * (g16 >> 1) + (s16 >> 2)) * 512 + ((chunk ^ ((s16 >> 2) << 2)) * 16) + (s16 & 1) * 8;
     }
   }
+  int ta[4] = {0, 0, 0, 0};
+  if (AT) {
+    const int s16 = lane & 15, g16 = lane >> 4;
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi) {
+      const int chunk = bi * 4 + 2 * (g16 & 1) + ((s16 & 3) >> 1);
+      ta[bi] = (8 * (g16 >> 1) + (s16 >> 2)) * 256 + ((chunk ^ ((s16 >> 2) << 2)) * 16) + (s16 & 1) * 8;
+    }
+  }
   auto frags = [&](const unsigned char *stg, int kk, Frags &f) {
-    if (BT) load_frags_bt<TK>(stg, a_base, swz[kk], tb, kk, f);
+    if (AT) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        f.a[i] = anc_lds_tr_frag(stg + ta[i] + kk * (16 * 256), stg + ta[i] + kk * (16 * 256) + 4 * 256);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        f.b[i] = anc_lds_tr_frag(stg + tb[i] + kk * (16 * 512), stg + tb[i] + kk * (16 * 512) + 4 * 512);
+    } else if (BT) load_frags_bt<TK>(stg, a_base, swz[kk], tb, kk, f);
     else load_frags<TK>(stg, stg, a_base, b_base, swz[kk], f);
   };
 
@@ -505,7 +532,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     fetch_a32(1);
   }
   unsigned char *dvec_lds = aux_w;
-  if (EPI == EPI_BX && VAR != VAR_PLAIN) {
+  if (EPI == EPI_BX && !PLAINV) {
     asm volatile("" : "+v"(sc));      // the scale has arrived before the first DMA is issued
     // dB of the tile's 128 rows, one private copy per wavefront (lanes 32..63 repeat lanes 0..31),
     // fetched first: any ordinary load issued after the slab fetches would, completing in
@@ -530,7 +557,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     // its bf16 copy. The master block is requested (8 x 16 bytes per lane) before the wait for
     // the slab's DMA, so that its latency runs under the wait and the arithmetic.
     constexpr bool fused = (VAR == VAR_UPDATE);
-    constexpr bool plain = (VAR == VAR_PLAIN);
+    constexpr bool plain = PLAINV;
     float *W32 = nullptr;
     uint16_t *W16 = nullptr;
     float wlr = 0.0f;
@@ -885,10 +912,10 @@ int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, h
   return ANC_OK;
 }
 
-// Bare products C[e] = A[e] B[e] (fp32 out, p.X32), A (M, K) with row pitch p.ldA, B (K, N)
-// row-major, on the X = a X + B X kernel's K loop: 128x256 tiles, M % 128 == 0, N % 256 == 0,
+// Bare products C[e] = A[e] B[e] (fp32 out, p.X32), A (M, K) with row pitch p.ldA -- or, with
+// a_transposed, (K, M) with row pitch p.ldA >= M (a multiple of 8) --, B (K, N) row-major, on the X = a X + B X kernel's K loop: 128x256 tiles, M % 128 == 0, N % 256 == 0,
 // K % 32 == 0.
-int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
+int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s, bool a_transposed) {
   ANC_REQUIRE(n >= 1 && n <= kMaxGroups, "anc_ns_gemm_big_plain: 1..%d problems per launch", kMaxGroups);
   NsGemmMulti pm{};
   pm.n = n;
@@ -936,7 +963,10 @@ int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_
       if (best == 0 || cost < best) { best = cost; g.blk_r = g.tiles_m / gx; g.blk_c = g.tiles_n / gy; }
     }
   }
-  hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_PLAIN>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+  if (a_transposed)
+    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_PLAIN_TN>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+  else
+    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_PLAIN>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }

@@ -4,9 +4,9 @@ step reads.
 Mirror of `ResidentLayerTrain._dW` (ancora/model/resident_train.py:285-287), which launches
 `_gemm_dW` or, with gradient accumulation, `_gemm_dW_acc` (ancora/kernels/fused.py:190-219) once
 per weight: x (T, K) and dy (T, N) bf16 bits, dW (K, N) fp32. Here up to 8 weights go into one
-call (`gemm_dW`), the activations are passed transposed (`transpose_acts`, once per group of
-weights that share them), and the call can also leave the bf16 copy of the finished gradient,
-which is what `HybridOptimizer(grad_dtype=np.uint16)` reads.
+call (`gemm_dW`), the activations are passed as they lie (`x`) or transposed (`xT`, for a caller
+that keeps them so), and the call can also leave the bf16 copy of the finished gradient, which is
+what `HybridOptimizer(grad_dtype=np.uint16)` reads.
 
 The token axis is cut into `segments` pieces so that a call fills the GPU (512 workgroups of
 128x256 outputs). By default every problem gets the number of pieces its shape needs to do that
@@ -63,7 +63,7 @@ class DwWorkspace:
 
 
 def gemm_dW(problems, si=0, segments=None):
-    """problems: list of dicts {xT, dy, dW: DevBuf; T, K, N: int; workspace: DwWorkspace;
+    """problems: list of dicts {x (T, K) or xT (K, T), dy, dW: DevBuf; T, K, N: int; workspace: DwWorkspace;
     g16: DevBuf or None; accumulate: bool; gn_partials: int device address or None (where the
     grad-norm partial sums of this gradient go, `StepGuard.partials_ptr`); segments: int, optional}.
     dW (+)= x^T dy for each, 8 per launch. `segments` (argument, or per problem) fixes the number
@@ -72,8 +72,15 @@ def gemm_dW(problems, si=0, segments=None):
     at once (so it depends on what shares the call). The result's bits depend on the number of
     segments and on nothing else. Asynchronous on stream `si`."""
     _lib.init()
-    for i0 in range(0, len(problems), MAX_PER_CALL):
-        group = problems[i0:i0 + MAX_PER_CALL]
+    runs, cur = [], []
+    for p in problems:                       # a native call takes one activation layout
+        if cur and ((p.get("x") is None) != (cur[0].get("x") is None) or len(cur) == MAX_PER_CALL):
+            runs.append(cur)
+            cur = []
+        cur.append(p)
+    if cur:
+        runs.append(cur)
+    for group in runs:
         fill = 0
         if segments == "fill":
             tiles = sum((int(p["K"]) // 128) * (int(p["N"]) // 256) for p in group)
@@ -93,6 +100,8 @@ def gemm_dW(problems, si=0, segments=None):
                 ws = p["workspace"].ensure(S * K * N * 4 if S > 0 else dw_workspace_bytes(T, K, N))
                 ws_ptr, ws_bytes = ws.ptr, ws.nbytes
             g16 = p.get("g16")
-            arr[k] = DwProblem(p["xT"].ptr, p["dy"].ptr, p["dW"].ptr, 0 if g16 is None else g16.ptr, ws_ptr,
-                               T, K, N, ws_bytes, int(bool(p.get("accumulate", False))), S, gn)
+            x = p.get("x")
+            arr[k] = DwProblem((p["xT"] if x is None else x).ptr, p["dy"].ptr, p["dW"].ptr,
+                               0 if g16 is None else g16.ptr, ws_ptr, T, K, N, ws_bytes,
+                               int(bool(p.get("accumulate", False))), S, gn, 0 if x is None else 1, 0)
         api.anc_gemm_dw_multi(arr, len(group), int(si))

@@ -8,7 +8,7 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
     python3 -m ancora_cutile_amd.prof_target gradnorm NUMEL [calls]      grad-norm partials + finalize
     python3 -m ancora_cutile_amd.prof_target quant K N E [cm] [calls]    MXFP8 weight re-quantisation
                                       (prints GB/s from HIP events around the calls)
-    python3 -m ancora_cutile_amd.prof_target dwlayer [T] [calls]         weight-gradient GEMMs of one layer in one call
+    python3 -m ancora_cutile_amd.prof_target dwlayer [T] [calls] [x|xT]  weight-gradient GEMMs of one layer in one call
     python3 -m ancora_cutile_amd.prof_target dw T K N1[,N2,..] [calls]   weight-gradient GEMM of up to 8
                                       weights (K, Ni) that share the activations, T tokens
     python3 -m ancora_cutile_amd.prof_target kloop                       the GEMM K loop alone on cache-resident
@@ -113,13 +113,14 @@ def main(argv):
         from .grads import gemm_dW, DwWorkspace, dw_info
         T = int(argv[1]) if len(argv) > 1 else 8192
         calls = int(argv[2]) if len(argv) > 2 else 5
+        xkey = argv[3] if len(argv) > 3 else "x"          # x: activations (T, K) as they lie; xT: (K, T)
         rng = np.random.default_rng(0)
         bits = lambda a: (a.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
         probs, fl = [], 0.0
         for K, Ns in ((1024, (2048, 1024, 1024)), (2048, (1024,)), (1024, (3072, 3072)), (3072, (1024,))):
-            xT = DevBuf(bits(0.1 * rng.standard_normal((K, T))))
+            xT = DevBuf(bits(0.1 * rng.standard_normal((T, K) if xkey == "x" else (K, T))))
             for N in Ns:
-                probs.append(dict(xT=xT, dy=DevBuf(bits(0.1 * rng.standard_normal((T, N)))),
+                probs.append(dict(**{xkey: xT}, dy=DevBuf(bits(0.1 * rng.standard_normal((T, N)))),
                                   dW=DevBuf.zeros((K, N), np.float32), g16=DevBuf.zeros((K, N), np.uint16),
                                   T=T, K=K, N=N, workspace=DwWorkspace(), accumulate=True))
                 fl += dw_info(T, K, N)[0]

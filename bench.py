@@ -161,9 +161,14 @@ def side_workload(args):
         calls, flops = [], 0.0
         for K, Ns in groups:
             xT = DevBuf(bf16_bits((0.1 * rng.standard_normal((K, T))).astype(np.float32)))
+            xkey = "xT"
+            if args.dw_acts == "x":                # the activations as they lie, (T, K)
+                xkey, old = "x", xT
+                xT = DevBuf(np.ascontiguousarray(old.to_numpy().T))
+                old.free()
             probs = []
             for N in Ns:
-                probs.append(dict(xT=xT, dy=DevBuf(bf16_bits((0.1 * rng.standard_normal((T, N))).astype(np.float32))),
+                probs.append(dict(**{xkey: xT}, dy=DevBuf(bf16_bits((0.1 * rng.standard_normal((T, N))).astype(np.float32))),
                                   dW=DevBuf.zeros((K, N), np.float32), g16=DevBuf.zeros((K, N), np.uint16),
                                   T=T, K=K, N=N, workspace=DwWorkspace(), accumulate=True))
                 flops += dw_info(T, K, N)[0]
@@ -191,6 +196,20 @@ def side_workload(args):
         pr = _lib.profile_read()
         _lib.profile_enable(False)
         g_ms, r_ms = pr["dw_gemm"][0], pr["dw_reduce"][0]
+        # the (T, K) -> (K, T) transposes of the activations that the GEMM's A operand layout asks
+        # for (once per group of weights that share them), timed apart: not in `value`
+        from ancora_cutile_amd.grads import transpose_acts
+        xs = [(DevBuf.zeros((T, K), np.uint16), DevBuf.zeros((K, T), np.uint16), K) for (K, _), probs in zip(groups, calls)]
+        for x, xT, K in xs:
+            transpose_acts(x, xT, T, K, 0)
+        e0.record(0)
+        for _ in range(layers):
+            for x, xT, K in xs:
+                transpose_acts(x, xT, T, K, 0)
+        e1.record(0)
+        e1.sync()
+        tr_ms = e0.elapsed_ms(e1)
+        tr_bytes = layers * sum(4 * T * K for _, _, K in xs)
         tf = layers * flops / (ms * 1e-3) / 1e12
         gtf = layers * flops / (g_ms * 1e-3) / 1e12
         nparams = sum(K * N for K, Ns in groups for N in Ns) * layers
@@ -202,14 +221,18 @@ def side_workload(args):
                           "params": nparams, "launch": args.dw_launch,
                           "launches_per_layer": 1 if args.dw_launch == "layer" else 4,
                           "token_segments": {"layer": 1, "group": "shape rule", "group-fill": "per launch, <= 512 workgroups"}[args.dw_launch],
-                          "accumulate": True, "bf16_copy": True},
+                          "accumulate": True, "bf16_copy": True,
+                          "activations": "x (T,K) as they lie" if args.dw_acts == "x" else "x^T (K,T), transposed by the caller"},
                "roofline": {"bound": "mfma", "achieved": round(gtf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                             "frac": round(gtf / PEAK_BF16_TFLOPS, 4), "traffic": None,
                             "kernel": "k_ns_gemm_big<EPI_BX, ..., VAR_PLAIN> (partial tiles of x^T dy)",
                             "launches_per_step": pr["dw_gemm"][1], "avg_launch_ms": round(g_ms / pr["dw_gemm"][1], 4),
                             "tflop_per_step": round(layers * flops / 1e12, 3)},
                "whole_tflops_per_s": round(tf, 1),
-               "reduce_kernel": {"ms": round(r_ms, 3), "launches": pr["dw_reduce"][1]}}
+               "reduce_kernel": {"ms": round(r_ms, 3), "launches": pr["dw_reduce"][1]},
+               "activation_transposes": {"ms": round(tr_ms, 3), "launches": layers * len(xs),
+                                         "gbps": round(tr_bytes / (tr_ms * 1e-3) / 1e9, 1),
+                                         "note": "what a caller of the x^T form pays on top: x (T,K) -> x^T (K,T) once per group of weights sharing x; never in value"}}
     else:
         n = 1_200_000_000
         rng = np.random.default_rng(0)
@@ -266,6 +289,8 @@ def main():
     ap.add_argument("--layers", type=int, default=28, help=argparse.SUPPRESS)   # smaller sets for debugging
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens per micro-batch of --workload dw")
+    ap.add_argument("--dw-acts", default="x", choices=("x", "xT"),
+                    help="--workload dw: activations as they lie (T,K), or transposed by the caller")
     ap.add_argument("--dw-launch", default="layer", choices=("layer", "group", "group-fill"),
                     help="--workload dw: one call per layer (7 weights, 1 token segment) or 4 calls per layer")
     ap.add_argument("--workload", default="qwen3", choices=("qwen3", "moe", "ns", "adamw", "dw"),

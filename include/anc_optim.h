@@ -292,9 +292,8 @@ int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
 /* ------------------------------------------------------ weight gradients ----
  * dW (+)= x^T dy for up to 8 weights per call: replaces `_gemm_dW` / `_gemm_dW_acc`
  * (ancora/kernels/fused.py:190-219, launched per weight at ancora/model/resident_train.py:285-287),
- * the producer of the fp32 gradients the optimizer step reads. xT is the activation matrix
- * transposed, (K, T) bf16 row-major (anc_transpose_bf16 of the (T, K) activations, once per group
- * of weights that share them); dy is (T, N) bf16; dW (K, N) fp32 is overwritten, or added onto when
+ * the producer of the fp32 gradients the optimizer step reads. xT is the activation matrix, either
+ * transposed, (K, T) bf16 row-major, or as it lies, x (T, K), with x_row_major = 1; dy is (T, N) bf16; dW (K, N) fp32 is overwritten, or added onto when
  * `accumulate` is set (micro-batch accumulation in place); g16, if not 0, receives the bf16 copy
  * (RNE) of the final dW, the format the step reads. fp32 accumulation in a fixed order: the token
  * axis is cut into S equal pieces, each tile of each piece is one workgroup's whole K loop, and
@@ -315,6 +314,10 @@ typedef struct {
                                   gradient (of its bf16 copy if g16 is set), bit-identical to what
                                   anc_gradnorm_partials would compute from the stored gradient, so
                                   that the step's norm needs no pass of its own over it */
+  int32_t  x_row_major;        /* 1: `xT` points at the activations as they lie, x (T, K) row-major (the
+                                  reference's argument); 0: at x^T (K, T). Same bits either way; all
+                                  problems of a call must agree */
+  int32_t  reserved;
 } anc_dw_problem_t;
 int64_t anc_gemm_dw_workspace_bytes(int64_t T, int64_t K, int64_t N);
 int anc_gemm_dw_multi(const anc_dw_problem_t *problems, int32_t n_problems, uint64_t stream);

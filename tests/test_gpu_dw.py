@@ -192,6 +192,28 @@ def test_one_segment_route_through_the_epilogue_has_the_two_kernel_bits(gpu):
     sums.free()
 
 
+@pytest.mark.parametrize("T,K,N,S", [(512, 1024, 1024, None), (256, 1024, 3072, 1), (2048, 128, 256, None),
+                                     (96, 384, 768, 1), (1024, 256, 512, 4)])
+def test_activations_as_they_lie_give_the_bits_of_the_transposed_route(gpu, T, K, N, S):
+    """`x` (T, K), the reference's argument, against `xT` (K, T): the same products summed in the
+    same order, so the same bits; and within the bar of the fp64 product."""
+    from ancora_cutile_amd import DevBuf
+    from ancora_cutile_amd.grads import gemm_dW, DwWorkspace
+    x, dy = _inputs(T, K, N, 70 + T)
+    dW0 = (0.5 * np.random.default_rng(71).standard_normal((K, N))).astype(np.float32)
+    outs = []
+    for lay in ("x", "xT"):
+        p = dict(dy=DevBuf(dy), dW=DevBuf(dW0), T=T, K=K, N=N, workspace=DwWorkspace(),
+                 g16=DevBuf.zeros((K, N), np.uint16), accumulate=True)
+        p[lay] = DevBuf(x if lay == "x" else np.ascontiguousarray(x.T))
+        gemm_dW([p], segments=S)
+        outs.append((p["dW"].to_numpy(), p["g16"].to_numpy()))
+        p.pop(lay).free()
+        _free(p)
+    assert rel_fro(outs[0][0], gemm_dw(x, dy, dW0)) < 2e-5
+    assert bits_equal(outs[0][0], outs[1][0]) and bits_equal(outs[0][1], outs[1][1])
+
+
 def test_shape_checks(gpu):
     from ancora_cutile_amd import _lib
     from ancora_cutile_amd.grads import dw_workspace_bytes
