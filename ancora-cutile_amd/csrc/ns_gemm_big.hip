@@ -67,6 +67,13 @@ namespace {
 // vmcnt(0), leave lgkmcnt/expcnt alone (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// X = a X + B X reads its symmetric B operand by rows k (see AT below) unless switched off.
+#ifdef ANC_DBG_BX_NT
+constexpr bool kBxReadsBByRows = false;
+#else
+constexpr bool kBxReadsBByRows = true;
+#endif
+
 struct Frags {
   bf16x8 a[4], b[2];
 };
@@ -214,12 +221,15 @@ __device__ __forceinline__ void lds_barrier() {
 // the extra registers and branches do not weigh on the other launches: VAR_UPDATE applies the
 // weight update; VAR_PLAIN is the bare product C = A B written as fp32 (no iterate at the output
 // position, no row scaling), which the weight-gradient GEMM uses; with `plain_sum` set it writes
-// C = (A32 or 0) + A B and, if Yh is set, the bf16 copy of C. VAR_PLAIN_TN is the same product
-// with A given transposed, (K, M) row-major with row pitch ldA (C = A^T B: the activations of a
-// weight-gradient GEMM as they lie): its A tile is [k][128 columns] like the B tile and its
-// fragments come from transposing LDS reads too.
-enum { VAR_NONE = 0, VAR_UPDATE = 1, VAR_PLAIN = 2, VAR_PLAIN_TN = 3 };
-template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS, int VAR = VAR_NONE>
+// C = (A32 or 0) + A B and, if Yh is set, the bf16 copy of C.
+// AT (X = a X + B X kernel only): the A operand is read transposed, from a (K, M) row-major matrix
+// with row pitch ldA: its tile is [k][128 columns] like the B tile, fetched in 256-byte rows
+// instead of 64-byte row pieces, and its fragments come from transposing LDS reads too. Used
+// for the activations of a weight-gradient GEMM as they lie (C = x^T dy) and for the chain's
+// own B X, whose B is symmetric (stored in full): B read by rows k is B^T read by rows m, the
+// same values in the same order of summation.
+enum { VAR_NONE = 0, VAR_UPDATE = 1, VAR_PLAIN = 2 };
+template <int EPI, int TM, int TN, int TK, int NS, int MINBLOCKS, int VAR = VAR_NONE, bool AT = false>
 __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_gemm_big(NsGemmMulti pm) {
   constexpr int NWN = TN / 64, NWAVES = (TM / 128) * NWN;
   constexpr int ROWB = TK * 2;                      // bytes per LDS row
@@ -249,8 +259,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const unsigned long long dbg_t0 = wall_clock64();
 #endif
   int gsel, L;
-  constexpr bool PLAINV = (VAR == VAR_PLAIN || VAR == VAR_PLAIN_TN);
-  constexpr bool AT = (VAR == VAR_PLAIN_TN);
+  constexpr bool PLAINV = (VAR == VAR_PLAIN);
   if (PLAINV && pm.seq) anc_seq_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
   else anc_group_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
   const NsGemm &p = pm.g[gsel];
@@ -904,10 +913,23 @@ int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, h
   bool any_upd = false, all_upd = true;
   for (int k = 0; k < n; ++k) { any_upd = any_upd || ps[k].upd != nullptr; all_upd = all_upd && ps[k].upd != nullptr; }
   ANC_REQUIRE(any_upd == all_upd, "anc_ns_gemm_big: the fused update applies to every problem of a launch or to none");
-  if (any_upd)
-    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_UPDATE>), dim3((unsigned)grid), dim3(256), 0, s, pm);
-  else
-    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+  // B is symmetric and stored in full, so its tile can be fetched by rows k (256-byte rows) as
+  // well as by rows m (64-byte row pieces): same values, same order of summation. Measured per 5
+  // launches: 84 x (1024, 3072) 4.12 against 4.27 ms, 208 x (1024, 1024) 3.37 against 3.56 ms,
+  // but 64 x (512, 512) 0.238 against 0.212 ms: by rows k from M = 1024 on.
+  bool by_rows = kBxReadsBByRows;
+  for (int k = 0; k < n; ++k) by_rows = by_rows && ps[k].M >= 1024;
+  if (any_upd) {
+    if (by_rows)
+      hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_UPDATE, true>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+    else
+      hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_UPDATE, false>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+  } else {
+    if (by_rows)
+      hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_NONE, true>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+    else
+      hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_NONE, false>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+  }
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
@@ -964,7 +986,7 @@ int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_
     }
   }
   if (a_transposed)
-    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_PLAIN_TN>), dim3((unsigned)grid), dim3(256), 0, s, pm);
+    hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_PLAIN, true>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   else
     hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_PLAIN>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   ANC_LAUNCH_CHECK();
