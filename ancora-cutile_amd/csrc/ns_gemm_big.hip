@@ -40,6 +40,8 @@
 //
 // Accumulation order per output element is the same in every tile configuration and in the
 // 128x128 kernel of ns.hip (terms in order, k ascending, one accumulator).
+#include <type_traits>
+
 #include "ns_common.h"
 
 // Epilogue store; the timing-only ablation ANC_DBG_EPI_NOST never executes it.
@@ -427,9 +429,12 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   frags(stage0, 0, f[0]);
 
   // f[kk&1] holds k-step kk (KSTEPS is even, so every tile starts on f[0] and ends on f[1]).
-  auto body = [&](int step, unsigned char *cur, unsigned char *nxt, unsigned char *fill) {
-    const bool more = step + 1 < total;
-    const bool refill = step + NS - 1 < total;
+  // `steady` (a std::true_type): the caller knows that this tile refills the ring and has a
+  // successor, so the body carries no branch.
+  auto body = [&](auto steady, int step, unsigned char *cur, unsigned char *nxt, unsigned char *fill) {
+    constexpr bool kSteady = decltype(steady)::value;
+    const bool more = kSteady || step + 1 < total;
+    const bool refill = kSteady || step + NS - 1 < total;
 #ifndef ANC_DBG_NODMA
     if (KSTEPS == 2) {
       // The stage's DMA instructions go out between the MFMAs of the first k-step, one every
@@ -466,10 +471,19 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     if (more) frags(nxt, 0, f[0]);
     mfma8<BT>(f[(KSTEPS - 1) & 1], acc);
   };
-  for (int step = 0; step < total; step += NS) {
+  int step = 0;
+#ifndef ANC_DBG_NOSTEADY
+  // rounds of NS tiles in which even the last tile (step + NS - 1) still refills the ring
+  for (; step + 2 * NS - 2 < total; step += NS) {
 #pragma unroll
     for (int s0 = 0; s0 < NS; ++s0)
-      if (step + s0 < total) body(step + s0, st(s0), st((s0 + 1) % NS), st((s0 + NS - 1) % NS));
+      body(std::true_type{}, step + s0, st(s0), st((s0 + 1) % NS), st((s0 + NS - 1) % NS));
+  }
+#endif
+  for (; step < total; step += NS) {
+#pragma unroll
+    for (int s0 = 0; s0 < NS; ++s0)
+      if (step + s0 < total) body(std::false_type{}, step + s0, st(s0), st((s0 + 1) % NS), st((s0 + NS - 1) % NS));
   }
   __syncthreads();
 
