@@ -892,16 +892,10 @@ int launch_sym(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
 
 }  // namespace
 
-// Symmetric products run on 256x256 tiles (lower triangle); X = a X + B X runs on 128x256 tiles
-// (the tile counts of the problems are recomputed here).
-int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s,
-                          const NsUpdate *upd) {
-  ANC_REQUIRE(n >= 1 && n <= kMaxGroups, "anc_ns_gemm_big: 1..%d problems per launch", kMaxGroups);
-  for (int k = 0; k < n; ++k)
-    ANC_REQUIRE(ps[k].M % 256 == 0 && ps[k].N % 256 == 0 && ps[k].K % 32 == 0,
-                "anc_ns_gemm_big: dims must be multiples of 256");
-  if (epi == EPI_GRAM) return launch_sym<EPI_GRAM>(ps, Es, n, s);
-  if (epi == EPI_BMAT) return launch_sym<EPI_BMAT>(ps, Es, n, s);
+namespace {
+
+// One X = a X + B X launch over the given problems, B fetched by rows k or by rows m.
+int launch_bx(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s, const NsUpdate *upd, bool by_rows) {
   NsGemmMulti pm{};
   pm.n = n;
   int64_t grid = 0;
@@ -916,24 +910,14 @@ int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, h
     grid += t;
   }
   ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
-  if (upd != nullptr) {
+  const bool fused = ps[0].upd != nullptr;
+  if (fused) {
     for (int k = 0; k < ANC_MUON_MAX_SCALES; ++k) pm.lr[k] = upd->lr[k];
     pm.sr = upd->sr;
     pm.seed_base = upd->seed_base;
     pm.ctl = upd->ctl;
-  } else {
-    for (int k = 0; k < n; ++k) ANC_REQUIRE(ps[k].upd == nullptr, "anc_ns_gemm_big: fused update without its scalars");
   }
-  bool any_upd = false, all_upd = true;
-  for (int k = 0; k < n; ++k) { any_upd = any_upd || ps[k].upd != nullptr; all_upd = all_upd && ps[k].upd != nullptr; }
-  ANC_REQUIRE(any_upd == all_upd, "anc_ns_gemm_big: the fused update applies to every problem of a launch or to none");
-  // B is symmetric and stored in full, so its tile can be fetched by rows k (256-byte rows) as
-  // well as by rows m (64-byte row pieces): same values, same order of summation. Measured per 5
-  // launches: 84 x (1024, 3072) 4.12 against 4.27 ms, 208 x (1024, 1024) 3.37 against 3.56 ms,
-  // but 64 x (512, 512) 0.238 against 0.212 ms: by rows k from M = 1024 on.
-  bool by_rows = kBxReadsBByRows;
-  for (int k = 0; k < n; ++k) by_rows = by_rows && ps[k].M >= 1024;
-  if (any_upd) {
+  if (fused) {
     if (by_rows)
       hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_UPDATE, true>), dim3((unsigned)grid), dim3(256), 0, s, pm);
     else
@@ -945,6 +929,43 @@ int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, h
       hipLaunchKernelGGL((k_ns_gemm_big<EPI_BX, 128, 256, 32, 3, 2, VAR_NONE, false>), dim3((unsigned)grid), dim3(256), 0, s, pm);
   }
   ANC_LAUNCH_CHECK();
+  return ANC_OK;
+}
+
+}  // namespace
+
+// Symmetric products run on 256x256 tiles (lower triangle); X = a X + B X runs on 128x256 tiles
+// (the tile counts of the problems are recomputed here).
+int anc_ns_gemm_big_multi(int epi, const NsGemm *ps, const int64_t *Es, int n, hipStream_t s,
+                          const NsUpdate *upd) {
+  ANC_REQUIRE(n >= 1 && n <= kMaxGroups, "anc_ns_gemm_big: 1..%d problems per launch", kMaxGroups);
+  for (int k = 0; k < n; ++k)
+    ANC_REQUIRE(ps[k].M % 256 == 0 && ps[k].N % 256 == 0 && ps[k].K % 32 == 0,
+                "anc_ns_gemm_big: dims must be multiples of 256");
+  if (epi == EPI_GRAM) return launch_sym<EPI_GRAM>(ps, Es, n, s);
+  if (epi == EPI_BMAT) return launch_sym<EPI_BMAT>(ps, Es, n, s);
+  bool any_upd = false, all_upd = true;
+  for (int k = 0; k < n; ++k) { any_upd = any_upd || ps[k].upd != nullptr; all_upd = all_upd && ps[k].upd != nullptr; }
+  ANC_REQUIRE(any_upd == all_upd, "anc_ns_gemm_big: the fused update applies to every problem of a launch or to none");
+  ANC_REQUIRE(!any_upd || upd != nullptr, "anc_ns_gemm_big: fused update without its scalars");
+  // B is symmetric and stored in full, so its tile can be fetched by rows k (256-byte rows) as
+  // well as by rows m (64-byte row pieces). Measured per 5 launches: 84 x (1024, 3072) 4.12
+  // against 4.27 ms, 208 x (1024, 1024) 3.37 against 3.56 ms, but 64 x (512, 512) 0.238 against
+  // 0.212 ms: by rows k from M = 1024 on. The two ways read the same values except inside the
+  // diagonal 256x256 tiles of a B that descends from an A = X X^T with residual terms: there
+  // element (i, j) and element (j, i) add the same products in a different order and may differ
+  // in the last bit. So the way of reading is a property of the problem's shape, never of what
+  // it shares a call with: a call with problems of both kinds becomes two launches.
+  NsGemm part[kMaxGroups];
+  int64_t pe[kMaxGroups];
+  for (int pass = 0; pass < 2; ++pass) {
+    const bool by_rows = pass == 0;
+    int m = 0;
+    for (int k = 0; k < n; ++k)
+      if ((kBxReadsBByRows && ps[k].M >= 1024) == by_rows) { part[m] = ps[k]; pe[m] = Es[k]; ++m; }
+    if (m > 0)
+      if (int rc = launch_bx(part, pe, m, s, upd, by_rows)) return rc;
+  }
   return ANC_OK;
 }
 

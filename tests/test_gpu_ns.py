@@ -187,7 +187,7 @@ def test_grouped_launch_equals_per_batch_bits(gpu):
     from ancora_cutile_amd._lib import api
     from ancora_cutile_amd.muon_ns import ns_batched_pair, ns_workspace_bytes, coef_array, MODES
     rng = np.random.default_rng(11)
-    shapes = [(3, 256, 256), (2, 256, 768), (5, 512, 512)]
+    shapes = [(3, 256, 256), (2, 256, 768), (5, 512, 512), (1, 1024, 1024), (2, 512, 1024), (1, 256, 512)]
     host, alone = [], []
     for (E, M, N) in shapes:
         X = (0.01 * rng.standard_normal((E, M, N))).astype(np.float32)
@@ -200,8 +200,8 @@ def test_grouped_launch_equals_per_batch_bits(gpu):
         ns_batched_pair(U, fro, 2, E, M, N, 0, steps=5, schedule=PE_SCHEDULE, mode="bf16")
         alone.append(U.to_numpy())
         U.free(); fro.free()
-    for order in ([0, 1, 2], [2, 0, 1]):
-        bufs, probs = [], (_lib.NsProblem * 3)()
+    for order in ([0, 1, 2], [2, 0, 1], [3, 4, 5, 0, 1, 2], [3]):
+        bufs, probs = [], (_lib.NsProblem * len(order))()
         for k, q in enumerate(order):
             E, M, N = shapes[q]
             U, fro = DevBuf(host[q][0]), DevBuf(host[q][1])
@@ -210,7 +210,7 @@ def test_grouped_launch_equals_per_batch_bits(gpu):
             wptr = (ws.ptr + 255) // 256 * 256
             probs[k] = _lib.NsProblem(U.ptr, U.ptr + E * M * N * 2, fro.ptr, U.ptr, wptr, 2, E, M, N, nb)
             bufs.append((U, fro, ws))
-        api.anc_ns_batched_pair_multi(probs, 3, 5, coef_array(PE_SCHEDULE, 5), 1e-7, MODES["bf16"], 0)
+        api.anc_ns_batched_pair_multi(probs, len(order), 5, coef_array(PE_SCHEDULE, 5), 1e-7, MODES["bf16"], 0)
         for k, q in enumerate(order):
             assert bits_equal(bufs[k][0].to_numpy(), alone[q])
         for t in bufs:
