@@ -122,6 +122,29 @@ def test_chunk_and_scope_are_bitwise_neutral(gpu):
                 assert bits_equal(x, y)
 
 
+def test_weights_do_not_depend_on_what_shares_the_grouped_step(gpu):
+    """A 1024x1024 weight (residual terms in its chain; its B operand is fetched by rows) stepped
+    together with smaller shapes in one grouped, fused-update Muon step gets the bits it gets
+    when stepped alone, and so do the others."""
+    from ancora_cutile_amd import Muon, PE_SCHEDULE as PE
+    rng = np.random.default_rng(8)
+    shapes = {"a": (1024, 1024), "b": (512, 768), "c": (256, 256), "d": (768, 512)}
+    W = {n: (0.02 * rng.standard_normal(s)).astype(np.float32) for n, s in shapes.items()}
+    G = [{n: rng.standard_normal(s).astype(np.float32) for n, s in shapes.items()} for _ in range(2)]
+
+    def run(names):
+        opt = Muon({n: W[n] for n in names}, lr=0.02, momentum=0.95, ns_steps=5, schedule=PE)
+        for g in G:
+            opt.step({n: g[n] for n in names}, 0)
+        out = opt.master()
+        opt.free()
+        return out
+
+    together = run(list(shapes))
+    for n in shapes:
+        assert bits_equal(run([n])[n], together[n]), n
+
+
 @pytest.mark.parametrize("Ie", [128, 256])
 def test_expert_optimizer(gpu, Ie):
     """Stacked [E,K,N] experts: Muon per slice, idle experts (zero grad) leave their weights
