@@ -214,6 +214,37 @@ def test_activations_as_they_lie_give_the_bits_of_the_transposed_route(gpu, T, K
     assert bits_equal(outs[0][0], outs[1][0]) and bits_equal(outs[0][1], outs[1][1])
 
 
+def test_qwen3_layer_at_full_shape(gpu):
+    """The launch the benchmark times: the 7 weight gradients of one Qwen3-0.6B layer in one call
+    (activations as they lie, one token segment, accumulation, bf16 copy), 4096 tokens, against the
+    fp64 product."""
+    from ancora_cutile_amd import DevBuf
+    from ancora_cutile_amd.grads import gemm_dW, DwWorkspace
+    rng = np.random.default_rng(5)
+    T = 4096
+    layer = [(1024, 2048), (1024, 1024), (1024, 1024), (2048, 1024), (1024, 3072), (1024, 3072), (3072, 1024)]
+    xs, probs, refs = {}, [], []
+    for (K, N) in layer:
+        if K not in xs:
+            x = bf16_rne_bits((0.1 * rng.standard_normal((T, K))).astype(np.float32)).reshape(T, K)
+            xs[K] = (x, DevBuf(x))
+        x, xd = xs[K]
+        dy = bf16_rne_bits((0.1 * rng.standard_normal((T, N))).astype(np.float32)).reshape(T, N)
+        dW0 = (0.3 * rng.standard_normal((K, N))).astype(np.float32)
+        probs.append(dict(x=xd, dy=DevBuf(dy), dW=DevBuf(dW0), g16=DevBuf.zeros((K, N), np.uint16), T=T, K=K,
+                          N=N, workspace=DwWorkspace(), accumulate=True))
+        refs.append((x, dy, dW0))
+    gemm_dW(probs, 0, segments=1)
+    for p, (x, dy, dW0) in zip(probs, refs):
+        got = p["dW"].to_numpy()
+        assert rel_fro(got, gemm_dw(x, dy, dW0)) < 2e-5
+        assert bits_equal(p["g16"].to_numpy(), bf16_rne_bits(got).reshape(p["K"], p["N"]))
+        for k in ("dy", "dW", "g16"):
+            p[k].free()
+    for _, xd in xs.values():
+        xd.free()
+
+
 def test_shape_checks(gpu):
     from ancora_cutile_amd import _lib
     from ancora_cutile_amd.grads import dw_workspace_bytes
