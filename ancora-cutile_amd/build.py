@@ -10,8 +10,11 @@ tiles fetched for the first K tiles only), ANC_DBG_NOMFMA (matrix instructions r
 ANC_DBG_TRACE (per-workgroup timestamps of K loop and epilogue, read with anc_dbg_trace_read),
 ANC_DBG_KNOWAIT (K loop does not wait for its DMA), ANC_DBG_EPI_NOST / ANC_DBG_EPI_NOLD (epilogue
 without its global stores / without its input DMA); of csrc/ns.hip: ANC_DBG_SAMEOPS (every matrix of
-a batch multiplies the first matrix's operands, i.e. cache-resident operands). All but TRACE give
-wrong results: timing only.
+a batch multiplies the first matrix's operands, i.e. cache-resident operands). All of these but
+TRACE give wrong results: timing only. Two more switch an optimisation off and leave the results'
+bits alone: ANC_DBG_NOSTEADY (the K loop always runs its branching body), ANC_DBG_BX_NT
+(X = a X + B X fetches B by rows m in 64-byte pieces at every size; identical bits except for
+chains with residual terms at M >= 1024).
 
 hipcc cross-compiles without a GPU. Flags: no FMA contraction (the AdamW kernel must
 reproduce a numpy fp32 evaluation operation by operation), correctly rounded fp32
