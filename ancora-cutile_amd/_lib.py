@@ -136,9 +136,6 @@ _PROTOS = {
     "anc_ns_flops": (None, [i64, i64, i64, C.c_int, C.c_int, C.POINTER(C.c_double),
                             C.POINTER(C.c_double)]),
     "anc_ns_product_flops": (None, [i64, i64, i64, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]),
-    "anc_probe_mfma_mix": (None, [C.c_int, C.c_int, C.c_int, C.c_int, u64, i64, u64,
-                                  C.POINTER(C.c_double), C.POINTER(C.c_double)]),
-    "anc_probe_kloop": (None, [C.c_int, C.c_int, C.c_int, C.c_int, u64, i64, u64, C.POINTER(C.c_double)]),
     "anc_bf16_to_f32": (None, [u64, u64, i64, u64]),
     "anc_f32_to_bf16": (None, [u64, u64, i64, u64]),
 }

@@ -511,9 +511,6 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
         ga[q].nterms = 3;
       }
       ga[q].K = (int)N; ga[q].strideA = mn; ga[q].strideB = mn; ga[q].tiles_m = tM; ga[q].tiles_n = tM; ga[q].lower = 1;
-#ifdef ANC_DBG_SAMEOPS
-      ga[q].strideA = ga[q].strideB = 0;      // timing only: every matrix multiplies the first one's operands
-#endif
       // B = b A + c A A
       gb[q] = g;
       gb[q].A[0] = pl.Fh; gb[q].B[0] = pl.Fh; gb[q].nterms = 1;
@@ -529,9 +526,6 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       if (split) { gx[q].A[gx[q].nterms] = pl.Bh; gx[q].B[gx[q].nterms] = curL[q]; ++gx[q].nterms; }
       if (split_fb) { gx[q].A[gx[q].nterms] = pl.Bl; gx[q].B[gx[q].nterms] = curH[q]; ++gx[q].nterms; }
       gx[q].K = (int)M; gx[q].strideA = M * M; gx[q].strideB = mn; gx[q].tiles_m = tM; gx[q].tiles_n = tN; gx[q].lower = 0;
-#ifdef ANC_DBG_SAMEOPS
-      gx[q].strideA = gx[q].strideB = 0;
-#endif
       gx[q].Xh = curH[q]; gx[q].Xl = curL[q];
       gx[q].Yh = last ? nullptr : pl.Xh[nxt[q]];
       gx[q].Yl = last ? nullptr : pl.Xl[nxt[q]];

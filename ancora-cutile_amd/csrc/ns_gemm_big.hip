@@ -44,22 +44,8 @@
 
 #include "ns_common.h"
 
-// Epilogue store; the timing-only ablation ANC_DBG_EPI_NOST never executes it.
-template <typename T> __device__ __forceinline__ void epi_st(T *p, T v) {
-#if defined(ANC_DBG_EPI_NOST)
-  if (((uintptr_t)p & 1) != 0) *p = v;
-#else
-  anc_st_stream(p, v);
-#endif
-}
-
-#ifdef ANC_DBG_TRACE
-// Debug build only: per-workgroup timestamps (100 MHz wall clock) of the last launch of each kind.
-__device__ unsigned long long anc_dbg_ts[3][16384][4];
-extern "C" int anc_dbg_trace_read(void *host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(anc_dbg_ts), sizeof(unsigned long long) * 3 * 16384 * 4);
-}
-#endif
+// Epilogue store: streaming, the written tile is not read again by this launch.
+template <typename T> __device__ __forceinline__ void epi_st(T *p, T v) { anc_st_stream(p, v); }
 
 namespace {
 
@@ -69,12 +55,8 @@ namespace {
 // vmcnt(0), leave lgkmcnt/expcnt alone (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
-// X = a X + B X reads its symmetric B operand by rows k (see AT below) unless switched off.
-#ifdef ANC_DBG_BX_NT
-constexpr bool kBxReadsBByRows = false;
-#else
+// X = a X + B X reads its symmetric B operand by rows k (see AT below).
 constexpr bool kBxReadsBByRows = true;
-#endif
 
 struct Frags {
   bf16x8 a[4], b[2];
@@ -111,12 +93,8 @@ __device__ __forceinline__ void load_frags_bt(const unsigned char *st, int a_bas
 template <bool SWAP>
 __device__ __forceinline__ void mfma1(const Frags &f, f32x16 (&acc)[4][2], int idx) {
   const int bi = idx >> 1, bj = idx & 1;
-#ifndef ANC_DBG_NOMFMA
   acc[bi][bj] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[bj], f.a[bi], acc[bi][bj], 0, 0, 0)
                      : __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[bi], f.b[bj], acc[bi][bj], 0, 0, 0);
-#else
-  acc[bi][bj][0] += (float)f.a[bi][0] + (float)f.b[bj][0];
-#endif
 }
 template <bool SWAP>
 __device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
@@ -124,12 +102,8 @@ __device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
   for (int bi = 0; bi < 4; ++bi)
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj)
-#ifndef ANC_DBG_NOMFMA
       acc[bi][bj] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[bj], f.a[bi], acc[bi][bj], 0, 0, 0)
                          : __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[bi], f.b[bj], acc[bi][bj], 0, 0, 0);
-#else
-      acc[bi][bj][0] += (float)f.a[bi][0] + (float)f.b[bj][0];
-#endif
 }
 
 // bf16 tile staging through LDS. `v` holds, for the wavefront's 32-row slab, the bf16 values of
@@ -197,13 +171,7 @@ __device__ __forceinline__ void dma16(const void *g, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(g)
                : "memory", "m0");
 }
-__device__ __forceinline__ void dma16_epi(const void *g, uint32_t lds_base) {
-#if defined(ANC_DBG_EPI_NOLD)
-  (void)g; (void)lds_base;
-#else
-  dma16(g, lds_base);
-#endif
-}
+__device__ __forceinline__ void dma16_epi(const void *g, uint32_t lds_base) { dma16(g, lds_base); }
 __device__ __forceinline__ uint32_t lds_addr(const void *p) {
   return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const void *)p);
 }
@@ -257,9 +225,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // X = a X + B X: of the dB entries of its 128 rows
   __shared__ __attribute__((aligned(1024))) unsigned char aux[EPI != EPI_GRAM ? NWAVES * 1024 : 16];
 
-#ifdef ANC_DBG_TRACE
-  const unsigned long long dbg_t0 = wall_clock64();
-#endif
   int gsel, L;
   constexpr bool PLAINV = (VAR == VAR_PLAIN);
   if (PLAINV && pm.seq) anc_seq_tile(pm, (int)blockIdx.x, (int)gridDim.x, gsel, L);
@@ -435,7 +400,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     constexpr bool kSteady = decltype(steady)::value;
     const bool more = kSteady || step + 1 < total;
     const bool refill = kSteady || step + NS - 1 < total;
-#ifndef ANC_DBG_NODMA
     if (KSTEPS == 2) {
       // The stage's DMA instructions go out between the MFMAs of the first k-step, one every
       // 8/IPS matrix instructions, instead of as a burst during which the matrix pipe idles.
@@ -452,34 +416,26 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           }
       }
       if (refill) issue_advance();
-    } else
-#endif
-    {
-#ifndef ANC_DBG_NODMA
+    } else {
       if (refill) issue(fill);
-#endif
 #pragma unroll
       for (int kk = 0; kk < KSTEPS - 1; ++kk) {
         frags(cur, kk + 1, f[(kk + 1) & 1]);
         mfma8<BT>(f[kk & 1], acc);
       }
     }
-#ifndef ANC_DBG_KNOWAIT
     if (refill) wait_vm<(NS - 2) * IPS>(); else wait_vm<0>();
-#endif
     lds_barrier();
     if (more) frags(nxt, 0, f[0]);
     mfma8<BT>(f[(KSTEPS - 1) & 1], acc);
   };
   int step = 0;
-#ifndef ANC_DBG_NOSTEADY
   // rounds of NS tiles in which even the last tile (step + NS - 1) still refills the ring
   for (; step + 2 * NS - 2 < total; step += NS) {
 #pragma unroll
     for (int s0 = 0; s0 < NS; ++s0)
       body(std::true_type{}, step + s0, st(s0), st((s0 + 1) % NS), st((s0 + NS - 1) % NS));
   }
-#endif
   for (; step < total; step += NS) {
 #pragma unroll
     for (int s0 = 0; s0 < NS; ++s0)
@@ -488,12 +444,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   __syncthreads();
 
   // ---- epilogue
-#ifdef ANC_DBG_TRACE
-  const unsigned long long dbg_t1 = wall_clock64();
-#endif
-#ifdef ANC_DBG_NOEPI
-  if (acc[0][0][0] + acc[3][1][7] != 12345.678f) return;
-#endif
   if (VAR == VAR_UPDATE && pm.ctl != nullptr && pm.ctl->skip != 0u) return;   // skipped step
   const int M = p.M, N = p.N;
   const int64_t mm = (int64_t)e * M * M, mn = (int64_t)e * M * N, mv = (int64_t)e * M;
@@ -768,14 +718,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       asm volatile("" ::: "memory");
       if (!plain && bi + 2 < 4) fetch_in(bi + 2);
     }
-#ifdef ANC_DBG_TRACE
-    if (threadIdx.x == 0 && blockIdx.x < 16384) {
-      anc_dbg_ts[EPI][blockIdx.x][0] = dbg_t0;
-      anc_dbg_ts[EPI][blockIdx.x][1] = dbg_t1;
-      anc_dbg_ts[EPI][blockIdx.x][2] = wall_clock64();
-      anc_dbg_ts[EPI][blockIdx.x][3] = 0;
-    }
-#endif
     return;
   }
 #pragma unroll
@@ -857,18 +799,6 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       if (bi + 2 < 4) fetch_a32(bi + 2);
     }
   }
-#ifdef ANC_DBG_TRACE
-  if (threadIdx.x == 0 && blockIdx.x < 16384) {
-    unsigned int hwid;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-    unsigned int xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-    anc_dbg_ts[EPI][blockIdx.x][0] = dbg_t0;
-    anc_dbg_ts[EPI][blockIdx.x][1] = dbg_t1;
-    anc_dbg_ts[EPI][blockIdx.x][2] = wall_clock64();
-    anc_dbg_ts[EPI][blockIdx.x][3] = ((unsigned long long)xcc << 32) | hwid;
-  }
-#endif
 }
 
 template <int EPI>

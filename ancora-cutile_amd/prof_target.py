@@ -11,10 +11,6 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
     python3 -m ancora_cutile_amd.prof_target dwlayer [T] [calls] [x|xT]  weight-gradient GEMMs of one layer in one call
     python3 -m ancora_cutile_amd.prof_target dw T K N1[,N2,..] [calls]   weight-gradient GEMM of up to 8
                                       weights (K, Ni) that share the activations, T tokens
-    python3 -m ancora_cutile_amd.prof_target kloop                       the GEMM K loop alone on cache-resident
-                                      operands (anc_probe_kloop), 8 and 4 wavefronts per workgroup
-    python3 -m ancora_cutile_amd.prof_target mfmamix                    matrix-instruction rate next to
-                                      unrelated LDS / LDS-DMA traffic (anc_probe_mfma_mix), a table
 
 Each target allocates its operands, runs the kernel(s) `calls` times on the null stream and
 synchronises; nothing is checked here (parity lives in tests/).
@@ -134,33 +130,6 @@ def main(argv):
         gms, rms = pr["dw_gemm"][0] / calls, pr["dw_reduce"][0] / calls
         print(f"dW of one layer (7 weights, T={T}, 1 segment, 480 workgroups): gemm {gms * 1e3:.1f} us "
               f"({fl / gms / 1e9:.1f} TFLOP/s), finish {rms * 1e3:.1f} us, together {fl / (gms + rms) / 1e9:.1f} TFLOP/s")
-    elif what == "kloop":
-        src = DevBuf.zeros((1 << 29,), np.float32)          # 2 GiB
-        sink = DevBuf.zeros((512,), np.float32)
-        tf = ctypes.c_double(0)
-        _lib.api.anc_probe_kloop(8, 32, 128, 16, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf))     # clocks settle
-        print("K loop alone (256x256x32 tiles, 4-stage LDS-DMA ring, no epilogue), 256 workgroups")
-        for waves, share, kt, reps in ((8, 32, 128, 16), (4, 32, 128, 16), (8, 4, 128, 16), (8, 2, 128, 16), (8, 1, 128, 16),
-                                       (8, 32, 4096, 1), (8, 4, 1024, 1), (8, 32, 128, 16)):
-            _lib.api.anc_probe_kloop(waves, share, kt, reps, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf))
-            mib = 256 * kt * 32 * 2 / 2 ** 20
-            how = f"read {reps} times" if reps > 1 else "read once (first touch)"
-            print(f"  {waves} wavefronts x {'128x64' if waves == 8 else '128x128'}, {share:2d} workgroups per operand pair of "
-                  f"2 x {mib:.0f} MiB, {how}: {tf.value:7.1f} TFLOP/s = {tf.value / 25:.1f} % of 2.5 PFLOP/s, "
-                  f"{256 * 256 * 32 * 2 * 256 / (tf.value * 1e6):.2f} us per K tile")
-    elif what == "mfmamix":
-        src = DevBuf.zeros((1 << 28,), np.float32)          # 1 GiB
-        sink = DevBuf.zeros((512,), np.float32)
-        print("16 MFMA per wavefront-iteration, 8 wavefronts per CU, 256 CUs")
-        tf, cyc = ctypes.c_double(0), ctypes.c_double(0)
-        _lib.api.anc_probe_mfma_mix(0, 0, 0, 100000, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf),
-                                    ctypes.byref(cyc))                     # clocks settle; discarded
-        for nread, ndma, hbm in ((0, 0, 0), (12, 0, 0), (0, 4, 0), (12, 4, 0), (24, 8, 0), (12, 4, 1),
-                                 (0, 0, 0)):
-            _lib.api.anc_probe_mfma_mix(nread, ndma, hbm, 50000, src.ptr, src.nbytes, sink.ptr,
-                                        ctypes.byref(tf), ctypes.byref(cyc))
-            print(f"  + {nread:2d} ds_read_b128 + {ndma} LDS-DMA KiB ({'HBM stream' if hbm else 'L2 resident'}): "
-                  f"{tf.value:7.1f} TFLOP/s = {tf.value / 25:.1f} % of 2.5 PFLOP/s")
     else:
         raise SystemExit(__doc__)
     _lib.api.anc_device_sync()

@@ -427,24 +427,6 @@ int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
 int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, int mode, int k, int product,
                          double *executed);
 
-/* Diagnostics, no reference counterpart: rate of the bf16 matrix instruction on register
- * operands while the same wavefronts issue `nread` LDS fragment reads and `ndma` LDS-DMA loads
- * of 1 KiB per 16 matrix instructions that nothing depends on (the proportions of the
- * Newton-Schulz GEMM's K loop are 12 and 4), from an L2-resident source or, with hbm != 0,
- * streaming through `span_bytes` of HBM. (nread, ndma) one of (0,0) (12,0) (0,4) (12,4)
- * (24,8). `cycles_per_iter` is scaled so that the matrix instructions alone take 1024. */
-int anc_probe_mfma_mix(int nread, int ndma, int hbm, int iters, uint64_t src,
-                       int64_t span_bytes, uint64_t sink, double *tflops,
-                       double *cycles_per_iter);
-/* Diagnostics, no reference counterpart: the GEMM's K loop alone (256x256x32 tiles, 8 wavefronts
- * of 128x64 or 4 of 128x128 per workgroup, 4-stage LDS-DMA ring, real fragment reads, one barrier
- * per K tile, no epilogue) on 256 workgroups. Groups of `share` (1..32, power of two) workgroups
- * of one XCD multiply the same two 256-row operands (2 x 256 x 32*k_tiles bf16 per group at
- * `src`): share = 32 means nearly every operand load is served from L2 (what the loop structure
- * reaches when memory is out of the way), share = 4 about three in four. */
-int anc_probe_kloop(int waves, int share, int k_tiles, int reps, uint64_t src, int64_t span_bytes,
-                    uint64_t sink, double *tflops);
-
 /* fp32 <-> bf16 conversion of packed batches (entry/exit of the bf16-typed
  * reference drivers): dst_f32 = float(src_bf16); dst_bf16 = RNE(src_f32). */
 int anc_bf16_to_f32(uint64_t src, uint64_t dst, int64_t n, uint64_t stream);

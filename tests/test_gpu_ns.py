@@ -216,33 +216,3 @@ def test_grouped_launch_equals_per_batch_bits(gpu):
         for t in bufs:
             for b in t:
                 b.free()
-
-
-def test_mfma_mix_probe_runs(gpu):
-    """The diagnostics entry returns a plausible matrix-instruction rate (below the 2.5 PFLOP/s
-    peak, above a tenth of it) and rejects a mix it has no kernel for."""
-    import ctypes
-    from ancora_cutile_amd import DevBuf, _lib
-    src = DevBuf.zeros((1 << 24,), np.float32)        # 64 MiB
-    sink = DevBuf.zeros((512,), np.float32)
-    tf, cyc = ctypes.c_double(0), ctypes.c_double(0)
-    _lib.api.anc_probe_mfma_mix(12, 4, 0, 2000, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf), ctypes.byref(cyc))
-    assert 250.0 < tf.value < 2500.0 and cyc.value > 1024.0
-    with pytest.raises(_lib.AncoraError):
-        _lib.api.anc_probe_mfma_mix(5, 5, 0, 10, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf), ctypes.byref(cyc))
-    src.free(); sink.free()
-
-
-def test_kloop_probe_runs(gpu):
-    """The K-loop diagnostics entry returns a plausible rate and rejects a bad configuration."""
-    import ctypes
-    from ancora_cutile_amd import DevBuf, _lib
-    src = DevBuf.zeros((1 << 22,), np.float32)        # 16 MiB: 8 groups of 2 x 256 x 2048 bf16
-    sink = DevBuf.zeros((512,), np.float32)
-    tf = ctypes.c_double(0)
-    for waves in (8, 4):
-        _lib.api.anc_probe_kloop(waves, 32, 64, 4, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf))
-        assert 300.0 < tf.value < 2500.0
-    with pytest.raises(_lib.AncoraError):
-        _lib.api.anc_probe_kloop(6, 32, 64, 4, src.ptr, src.nbytes, sink.ptr, ctypes.byref(tf))
-    src.free(); sink.free()
