@@ -106,6 +106,8 @@ _PROTOS = {
     "anc_gradnorm_partials": (None, [u64, i64, C.c_int, u64, i64, u64]),
     "anc_gradnorm_partials_multi": (None, [u64, i32, i64, u64, u64]),
     "anc_gradnorm_finalize": (None, [u64, i64, f32, f32, u64, u64]),
+    "anc_gradnorm_static_max_elements": (i64, []),
+    "anc_gradnorm_static": (None, [u64, i64, C.c_int, f32, f32, u64, u64]),
     "anc_adamw": (None, [u64, u64, u64, u64, u64, i64, C.c_int, C.POINTER(AdamWHyper), f32, u32,
                          u64, u64]),
     "anc_adamw_num_blocks": (i64, [i64]),

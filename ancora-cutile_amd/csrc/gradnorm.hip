@@ -15,6 +15,8 @@
 // Stage 2, one block of 1024 lanes: lane t adds partials t, t+1024, ... in order, then
 // the same butterfly, then the 16 wavefront sums in order. The result depends on the
 // tensor sizes only: never on the grid, the launch grouping or the run.
+#include <atomic>
+
 #include "reduce.h"
 
 namespace {
@@ -123,6 +125,66 @@ extern "C" int anc_gradnorm_finalize(uint64_t partials, int64_t n_partials, floa
   AncProfScope prof(ANC_PROF_GN_FINALIZE, anc_stream(stream));
   hipLaunchKernelGGL(k_gn_finalize, dim3(1), dim3(kFinThreads), 0, anc_stream(stream),
                      (const double *)partials, n_partials, max_norm, eps, (anc_step_ctl_t *)ctl);
+  ANC_LAUNCH_CHECK();
+  return ANC_OK;
+}
+
+// ------------------------------------------------------------------ no-allocation variant
+// anc_gradnorm_static keeps the stage-1 partial sums in a file-scope device array instead of a
+// caller-owned buffer, for callers that cannot allocate (HIP graph capture, tight serving loops).
+// Every GPU holds its own copy of the array at its own address; the address is looked up once
+// per device (anc_gradnorm_static_init, called by anc_init, or lazily on a device's first call)
+// and host code only ever uses that looked-up pointer: the array's name is a host-side stand-in,
+// not a device address.
+#define ANC_GN_STATIC_MAX_PARTIALS 262144          /* 2 MiB of fp64 partials: n <= 2^31 elements */
+static __device__ __align__(256) double scratch[ANC_GN_STATIC_MAX_PARTIALS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<double *> g_scratch_ptr[kMaxDevices];
+}  // namespace
+
+// Look up the device address of `scratch` on the current device (once per device).
+int anc_gradnorm_static_init(void) {
+  int dev = 0;
+  ANC_HIP(hipGetDevice(&dev));
+  ANC_REQUIRE(dev >= 0 && dev < kMaxDevices, "anc_gradnorm_static: device index %d beyond %d", dev, kMaxDevices);
+  if (g_scratch_ptr[dev].load(std::memory_order_acquire) != nullptr) return ANC_OK;
+  double *ptr = nullptr;
+  ANC_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+  ANC_REQUIRE(ptr != nullptr, "anc_gradnorm_static: null address for the scratch array");
+  g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  return ANC_OK;
+}
+
+extern "C" int64_t anc_gradnorm_static_max_elements(void) {
+  return (int64_t)ANC_GN_STATIC_MAX_PARTIALS * ANC_GN_CHUNK;
+}
+
+extern "C" int anc_gradnorm_static(uint64_t g, int64_t n, int g_dtype, float max_norm, float eps,
+                                   uint64_t ctl, uint64_t stream) {
+  ANC_REQUIRE(g != 0 && ctl != 0 && n > 0, "anc_gradnorm_static: bad arguments (n=%lld)", (long long)n);
+  ANC_REQUIRE(g_dtype == ANC_F32 || g_dtype == ANC_BF16, "anc_gradnorm_static: bad dtype %d", g_dtype);
+  ANC_REQUIRE((g & 15) == 0 && (ctl & 7) == 0, "anc_gradnorm_static: misaligned pointers");
+  const int64_t chunks = anc_gradnorm_num_partials(n);
+  ANC_REQUIRE(chunks <= ANC_GN_STATIC_MAX_PARTIALS,
+              "anc_gradnorm_static: n=%lld exceeds the built-in scratch (at most %lld elements); use "
+              "anc_gradnorm_partials + anc_gradnorm_finalize with a caller-owned buffer",
+              (long long)n, (long long)anc_gradnorm_static_max_elements());
+  if (int rc = anc_gradnorm_static_init()) return rc;
+  int dev = 0;
+  ANC_HIP(hipGetDevice(&dev));
+  double *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  // Stage 1 overwrites partials [0, chunks) and stage 2 reads exactly those: nothing of an
+  // earlier call is read, so nothing needs clearing.
+  hipStream_t s = anc_stream(stream);
+  if (g_dtype == ANC_BF16)
+    hipLaunchKernelGGL(k_gn_partials<ANC_BF16>, dim3((unsigned)chunks), dim3(kThreads), 0, s, (const void *)g, n, ptr);
+  else
+    hipLaunchKernelGGL(k_gn_partials<ANC_F32>, dim3((unsigned)chunks), dim3(kThreads), 0, s, (const void *)g, n, ptr);
+  ANC_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_gn_finalize, dim3(1), dim3(kFinThreads), 0, s, (const double *)ptr, chunks, max_norm, eps,
+                     (anc_step_ctl_t *)ctl);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }

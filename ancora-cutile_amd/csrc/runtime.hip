@@ -75,6 +75,8 @@ extern "C" int anc_profile_read(float *ms, int64_t *launches) {
 }
 extern "C" int anc_abi_version(void) { return 1; }
 
+int anc_gradnorm_static_init(void);   // gradnorm.hip: per-device address of its built-in scratch
+
 extern "C" int anc_init(int device) {
   int n = 0;
   ANC_HIP(hipGetDeviceCount(&n));
@@ -87,7 +89,7 @@ extern "C" int anc_init(int device) {
                   p.gcnArchName);
     return ANC_ERR_UNSUPPORTED;
   }
-  return ANC_OK;
+  return anc_gradnorm_static_init();
 }
 
 extern "C" int anc_device_info(anc_device_info_t *out) {

@@ -163,6 +163,19 @@ int anc_gradnorm_finalize(uint64_t partials, int64_t n_partials,
                           float max_norm, float eps,
                           uint64_t ctl /* anc_step_ctl_t* */, uint64_t stream);
 
+/* The same norm for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference. One
+ * tensor of n elements; result in ctl bit-identical to anc_gradnorm_partials(g, n, g_dtype, buf, 0)
+ * followed by anc_gradnorm_finalize(buf, anc_gradnorm_num_partials(n), ...). The stage-1 partial
+ * sums live in a 2 MiB array built into the library (one copy per GPU, held until the process
+ * ends), so n is limited to anc_gradnorm_static_max_elements() = 2^31; larger n returns
+ * ANC_ERR_ARG. The call allocates nothing (no hipMalloc/hipFree, no events, and it is not seen
+ * by anc_profile_*). All calls on one GPU share that array: calls that overlap in time on one
+ * GPU (different streams without ordering) race and must be serialised by the caller. */
+int64_t anc_gradnorm_static_max_elements(void);
+int anc_gradnorm_static(uint64_t g, int64_t n, int g_dtype, float max_norm, float eps,
+                        uint64_t ctl /* anc_step_ctl_t* */, uint64_t stream);
+
 /* ---------------------------------------------------------------- AdamW ----
  * Replaces the `_adamw` cuda-tile kernel and its launch tuple
  * (g, m, v, p32, p16, OTM, beta1, beta2, eps, lr, wd, ibc1, ibc2)
