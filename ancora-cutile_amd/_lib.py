@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("ANCORA_OPTIM_LIB") or os.path.join(_HERE, "csrc", "li
 
 F32, BF16 = 0, 1                  # ANC_F32 / ANC_BF16
 FORM_DIV, FORM_IBC = 0, 1         # ANC_ADAMW_FORM_*
-NS_BF16, NS_FP32, NS_BF16_FAST = 0, 1, 2   # ANC_NS_*
+NS_BF16, NS_FP32, NS_BF16_FAST, NS_BF16_X3 = 0, 1, 2, 3   # ANC_NS_*
 GN_CHUNK = 8192                   # ANC_GN_CHUNK
 MUON_MAX_SCALES = 8               # ANC_MUON_MAX_SCALES
 
@@ -137,6 +137,7 @@ _PROTOS = {
                                         C.c_int, C.POINTER(f32), C.c_int, u32, u64, u64]),
     "anc_ns_flops": (None, [i64, i64, i64, C.c_int, C.c_int, C.POINTER(C.c_double),
                             C.POINTER(C.c_double)]),
+    "anc_ns_hard_info": (None, [u64, i64, i64, i64, C.c_int, C.c_int, C.POINTER(i32), C.POINTER(C.c_double), u64]),
     "anc_ns_product_flops": (None, [i64, i64, i64, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "anc_bf16_to_f32": (None, [u64, u64, i64, u64]),
     "anc_f32_to_bf16": (None, [u64, u64, i64, u64]),

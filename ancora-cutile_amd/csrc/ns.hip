@@ -38,6 +38,8 @@
 // banks); the next K tile is fetched into registers while the current one is multiplied.
 // Workgroup ids are remapped so that consecutive tiles -- the tiles of one matrix -- run on
 // the same XCD and share its L2.
+#include <vector>
+
 #include "reduce.h"
 #include "ns_common.h"
 
@@ -77,7 +79,7 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
   const int lrow = tid >> 3, lk = (tid & 7) * 8;     // loader: 8 lanes per 128-byte row
   const int K = p.K;
   const int nk = K / BK;
-  const int total = p.nterms * nk;
+  const int total = anc_ns_terms(p, e) * nk;
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -314,8 +316,13 @@ k_fro_partials(const float *__restrict__ X, int64_t mn, int nchunks, double *__r
 }
 
 // One block per matrix: lane t adds partials t, t+256, ... in order; butterfly; 4 wavefronts in order.
+// pow2 (pair entries only, else null): a matrix whose sum of squares is below 2^-100 (products of
+// its elements would underflow fp32 in the first A = U U^T) gets pow2[e] = 2^k with 2^k ||U|| in
+// [1, 2), every other matrix 1; k_pair_rescale multiplies the pair by it (exact) and the
+// reciprocal carries 2^-k, so the first step sees the same scale*U as without.
 __global__ void __launch_bounds__(kThreads)
-k_fro_finalize(const double *__restrict__ partials, int nchunks, float eps, float *__restrict__ recip) {
+k_fro_finalize(const double *__restrict__ partials, int nchunks, float eps, float *__restrict__ recip,
+               float *__restrict__ pow2) {
   __shared__ double wave_sum[kThreads / 64];
   const double *p = partials + (int64_t)blockIdx.x * nchunks;
   double acc = 0.0;
@@ -327,7 +334,42 @@ k_fro_finalize(const double *__restrict__ partials, int nchunks, float eps, floa
     double t = wave_sum[0];
 #pragma unroll
     for (int w = 1; w < kThreads / 64; ++w) t = t + wave_sum[w];
-    recip[blockIdx.x] = 1.0f / ((float)sqrt(t) + eps);
+    float r = 1.0f / ((float)sqrt(t) + eps);
+    if (pow2 != nullptr) {
+      float sc = 1.0f;
+      if (t > 0.0 && t < 0x1p-100) {
+        const int k = -ilogb(sqrt(t));
+        sc = ldexpf(1.0f, k);
+        r = ldexpf(r, -k);
+      }
+      pow2[blockIdx.x] = sc;
+    }
+    recip[blockIdx.x] = r;
+  }
+}
+
+// Multiply the bf16 pair of every matrix whose pow2 is not 1 by it; blocks of the others return
+// at once. One block per 4096 elements.
+__global__ void __launch_bounds__(kThreads)
+k_pair_rescale(uint16_t *__restrict__ Uh, uint16_t *__restrict__ Ul, const float *__restrict__ pow2, int blocks_per) {
+  const int e = (int)blockIdx.x / blocks_per;
+  const float sc = pow2[e];
+  if (sc == 1.0f) return;
+  const int64_t o = (int64_t)blockIdx.x * 4096 + threadIdx.x * 16;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    uint16_t *p = (h ? Ul : Uh) + o;
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+      anc_u32x4 w = *(const anc_u32x4 *)(p + 8 * v);
+      uint32_t q[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float lo = __uint_as_float(q[i] << 16) * sc, hi = __uint_as_float(q[i] & 0xFFFF0000u) * sc;
+        q[i] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
+      }
+      *(anc_u32x4 *)(p + 8 * v) = anc_u32x4{q[0], q[1], q[2], q[3]};
+    }
   }
 }
 
@@ -362,6 +404,42 @@ k_ns_prep(float *__restrict__ X, const float *__restrict__ recip, int64_t mn, in
   anc_st_stream((anc_u32x4 *)(Xl + o), lo);
 }
 
+// ------------------------------------------------------------------ conditioning proxy
+// ||offdiag(A)||_F^2 of the first iteration's A = X X^T (||X||_F = 1, so tr A = 1): 1/N for a
+// matrix with independent entries whatever its row scaling, N/r - N/M for one whose mass sits
+// in r directions that are spread over the rows (outlier columns). Read from Fh (bf16, zero
+// diagonal). kCondParts blocks per matrix, each over M*M/kCondParts consecutive elements: lane t
+// takes the 8-element vectors t, t+256, ..., adds their squares left to right in fp32, widens to
+// fp64; butterfly over the wavefront; the 4 wavefront sums in order. The consumers add the
+// kCondParts partial sums in order (anc_ns_terms).
+struct NsCondArgs {
+  int n;
+  int blocks[kMaxGroups];
+  const uint16_t *Fh[kMaxGroups];
+  double *out[kMaxGroups];
+  int M[kMaxGroups];
+};
+__global__ void __launch_bounds__(kThreads) k_ns_cond(NsCondArgs a) {
+  __shared__ double wave_sum[kThreads / 64];
+  int b = (int)blockIdx.x, q = 0;
+  while (q + 1 < a.n && b >= a.blocks[q]) { b -= a.blocks[q]; ++q; }
+  const int64_t per = (int64_t)a.M[q] * a.M[q] / kCondParts;
+  const uint16_t *src = a.Fh[q] + (int64_t)b * per;          // b = e * kCondParts + part
+  double acc = 0.0;
+  for (int64_t v = threadIdx.x; v < per / kRun; v += kThreads) acc = acc + (double)run_sumsq<ANC_BF16>(src, v * kRun, per);
+  acc = anc_wave_sum_f64(acc);
+  if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double t = wave_sum[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) t = t + wave_sum[w];
+    a.out[q][b] = t;
+  }
+}
+// A matrix is "hard" when N * ||offdiag(A0)||_F^2 exceeds this (1.0 for independent entries).
+constexpr double kCondTau = 2.5;
+
 // ------------------------------------------------------------------------- workspace
 struct Carve {
   uint64_t base;
@@ -384,10 +462,25 @@ struct Carve {
 struct SplitPlan {
   int x_from;    // first iteration whose A and B X products add the residual of X
   int fb_from;   // first iteration whose A A and B X products add the residuals of F and Boff
+  unsigned gram_hard;   // bit k: in iteration k (< x_from) the A = X X^T product of a hard matrix
+                        // adds the residual of X
 };
+// Hard matrices: inputs whose Frobenius mass sits in a few directions spread over all rows (a
+// gradient with a few outlier columns: the transposed iterate of a tall weight with outlier
+// rows). Rounding X to bf16 then costs the small directions their signal in A = X X^T while the
+// large ones converge: 1% of the columns x100 gives 2.2e-3 at 1024x3072 and 3.8e-3 at 1024x1024
+// without the terms below, 1.2e-3 and 8e-4 with them. Row outliers, whose mass lands on the exact
+// fp32 diagonal of A, need nothing (5e-4 .. 7e-4).
 SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
-  SplitPlan sp{steps, steps};
+  SplitPlan sp{steps, steps, 0u};
+  if (mode == ANC_NS_BF16_X3) {
+    // every product with the residuals of both operands' bf16 roundings, in every iteration:
+    // about 1e-5 on every input tried, three times the matrix-core work
+    sp.x_from = sp.fb_from = 0;
+    return sp;
+  }
   if (mode != ANC_NS_BF16) return sp;
+  sp.gram_hard = N < 2 * M ? 0x6u : 0x4u;       // iterations 1 and 2, or 2 alone
   // The first iterations are insensitive (the singular values are still far below 1, so
   // B X is a small correction to a X); residuals start at a fixed iteration index.
   if (M >= 1024) {
@@ -407,6 +500,8 @@ struct Plan {
   uint16_t *Fl, *Bl;
   double *partials;
   float *recip;
+  float *pow2;           // (E) power-of-two pre-scale of tiny inputs, pair entries
+  double *cond;          // (E, kCondParts) conditioning proxy, bf16 modes
   // bf16 modes
   uint16_t *Xh[2], *Xl[2];
   float *A32, *dA, *dB;
@@ -424,6 +519,7 @@ Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int ste
   pl.split = pl.sp.x_from < steps;
   pl.partials = c.take<double>(E * pl.nchunks);
   pl.recip = c.take<float>(E);
+  pl.pow2 = c.take<float>(E);
   if (mode == ANC_NS_FP32) {
     pl.Af = c.take<float>(E * M * M);
     pl.Bf = c.take<float>(E * M * M);
@@ -442,6 +538,7 @@ Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int ste
     }
     pl.dA = c.take<float>(E * M);
     pl.dB = c.take<float>(E * M);
+    pl.cond = c.take<double>(E * kCondParts);
   }
   pl.bytes = c.off;
   return pl;
@@ -453,7 +550,7 @@ int check_shape(int64_t E, int64_t M, int64_t N, int mode, const char *who) {
               (long long)M, (long long)N);
   ANC_REQUIRE(M <= N, "%s: M=%lld > N=%lld; pass tall matrices transposed", who, (long long)M,
               (long long)N);
-  ANC_REQUIRE(mode == ANC_NS_BF16 || mode == ANC_NS_FP32 || mode == ANC_NS_BF16_FAST,
+  ANC_REQUIRE(mode == ANC_NS_BF16 || mode == ANC_NS_FP32 || mode == ANC_NS_BF16_FAST || mode == ANC_NS_BF16_X3,
               "%s: unknown mode %d", who, mode);
   ANC_REQUIRE(E * (M / 128) * (N / 128) < (1ll << 30) && E * M * N < (1ll << 40),
               "%s: batch too large", who);
@@ -485,9 +582,14 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
   int nxt[kMaxGroups];
   int64_t Es[kMaxGroups];
   for (int q = 0; q < n; ++q) { curH[q] = cp[q].inH; curL[q] = cp[q].inL; nxt[q] = cp[q].nxt; Es[q] = cp[q].E; }
+  bool want_cond = false;      // some later iteration gates a product on the proxy
+  for (int q = 0; q < n; ++q)
+    for (int k = 1; k < steps && k < 32; ++k)
+      if (k < cp[q].pl.sp.x_from && ((cp[q].pl.sp.gram_hard >> k) & 1u)) want_cond = true;
   for (int k = 0; k < steps; ++k) {
     const bool last = k + 1 == steps;
     NsGemm ga[kMaxGroups], gb[kMaxGroups], gx[kMaxGroups];
+    bool any_gated = false;
     for (int q = 0; q < n; ++q) {
       const Plan &pl = cp[q].pl;
       const int64_t M = cp[q].M, N = cp[q].N, mn = M * N;
@@ -505,10 +607,17 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       // A = X X^T
       ga[q] = g;
       ga[q].A[0] = curH[q]; ga[q].B[0] = curH[q]; ga[q].nterms = 1;
-      if (split) {
+      const bool gated = !split && k < 32 && ((pl.sp.gram_hard >> k) & 1u);
+      if (split || gated) {
         ga[q].A[1] = curH[q]; ga[q].B[1] = curL[q];
         ga[q].A[2] = curL[q]; ga[q].B[2] = curH[q];
-        ga[q].nterms = 3;
+        if (split) ga[q].nterms = 3;
+      }
+      if (gated) {
+        ga[q].cond = pl.cond;
+        ga[q].cond_thresh = kCondTau / (double)N;
+        ga[q].nterms_hard = 3;
+        any_gated = true;
       }
       ga[q].K = (int)N; ga[q].strideA = mn; ga[q].strideB = mn; ga[q].tiles_m = tM; ga[q].tiles_n = tM; ga[q].lower = 1;
       // B = b A + c A A
@@ -540,6 +649,22 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       else hipLaunchKernelGGL(k_ns_gemm<EPI_GRAM>, dim3(g_sym), dim3(kGemmThreads), 0, s, ga[0]);
     }
     ANC_LAUNCH_CHECK();
+    if (k == 0 && want_cond) {
+      // the proxy of every problem that gates a later product, from the Fh this launch wrote
+      NsCondArgs ca{};
+      int blocks = 0;
+      for (int q = 0; q < n; ++q) {
+        if (cp[q].pl.sp.gram_hard == 0u) continue;
+        ca.Fh[ca.n] = cp[q].pl.Fh; ca.out[ca.n] = cp[q].pl.cond; ca.M[ca.n] = (int)cp[q].M;
+        ca.blocks[ca.n] = (int)(cp[q].E * kCondParts);
+        blocks += ca.blocks[ca.n];
+        ++ca.n;
+      }
+      AncProfScope prof(ANC_PROF_NS_FRO, s);
+      hipLaunchKernelGGL(k_ns_cond, dim3((unsigned)blocks), dim3(kThreads), 0, s, ca);
+      ANC_LAUNCH_CHECK();
+    }
+    (void)any_gated;
     {
       AncProfScope prof(ANC_PROF_NS_BMAT, s);
       if (big) { if (int rc = anc_ns_gemm_big_multi(EPI_BMAT, gb, Es, n, s)) return rc; }
@@ -615,6 +740,37 @@ extern "C" int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, 
   return ANC_OK;
 }
 
+// How many matrices of the last chain call on this workspace took the extra terms of the
+// conditioning gate, and the matrix-core work one such matrix adds to anc_ns_flops' `executed`.
+// Synchronises `stream`, then reads the proxy's partial sums back and takes the kernels' decision.
+extern "C" int anc_ns_hard_info(uint64_t workspace, int64_t E, int64_t M, int64_t N, int mode, int steps,
+                                int32_t *n_hard, double *extra_flops_per_matrix, uint64_t stream) {
+  mode &= ~ANC_NS_TILE128;
+  if (int rc = check_shape(E, M, N, mode, "anc_ns_hard_info")) return rc;
+  ANC_REQUIRE(n_hard != nullptr && extra_flops_per_matrix != nullptr && workspace != 0 && steps >= 0,
+              "anc_ns_hard_info: bad arguments");
+  *n_hard = 0;
+  *extra_flops_per_matrix = 0.0;
+  if (mode == ANC_NS_FP32) return ANC_OK;
+  const Plan pl = make_plan(workspace, E, M, N, mode, steps);
+  int gated_iters = 0;
+  for (int k = 1; k < steps && k < 32; ++k)
+    if (k < pl.sp.x_from && ((pl.sp.gram_hard >> k) & 1u)) ++gated_iters;
+  if (gated_iters == 0) return ANC_OK;
+  const double tM = (double)M / BM;
+  *extra_flops_per_matrix = gated_iters * 2.0 * (tM * (tM + 1) / 2) * (2.0 * BM * BN) * (double)N;
+  std::vector<double> host((size_t)(E * kCondParts));
+  ANC_HIP(hipStreamSynchronize(anc_stream(stream)));
+  ANC_HIP(hipMemcpy(host.data(), pl.cond, host.size() * sizeof(double), hipMemcpyDeviceToHost));
+  const double thresh = kCondTau / (double)N;
+  for (int64_t e = 0; e < E; ++e) {
+    double t = host[(size_t)(e * kCondParts)];
+    for (int i = 1; i < kCondParts; ++i) t = t + host[(size_t)(e * kCondParts + i)];
+    if (t > thresh) ++*n_hard;
+  }
+  return ANC_OK;
+}
+
 extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int steps,
                               const float *coef, float eps, int mode, uint64_t workspace,
                               int64_t workspace_bytes, uint64_t stream) {
@@ -637,7 +793,7 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
                      pl.nchunks, pl.partials); }
   ANC_LAUNCH_CHECK();
   { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s, pl.partials, pl.nchunks,
-                     eps, pl.recip); }
+                     eps, pl.recip, (float *)nullptr); }
   ANC_LAUNCH_CHECK();
   const int64_t total8 = E * mn / 8;
   const unsigned prep_grid = (unsigned)((total8 + kThreads - 1) / kThreads);
@@ -709,7 +865,10 @@ extern "C" int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partia
               (long long)workspace_bytes, (long long)pl.bytes);
   hipStream_t s = anc_stream(stream);
   { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s,
-                     (const double *)fro_partials, (int)n_partials, eps, pl.recip); }
+                     (const double *)fro_partials, (int)n_partials, eps, pl.recip, pl.pow2); }
+  ANC_LAUNCH_CHECK();
+  { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_pair_rescale, dim3((unsigned)(E * (M * N / 4096))), dim3(kThreads), 0, s,
+                     (uint16_t *)Uh, (uint16_t *)Ul, pl.pow2, (int)(M * N / 4096)); }
   ANC_LAUNCH_CHECK();
   ChainProb cp{pl, (const uint16_t *)Uh, (const uint16_t *)Ul, 0, pl.recip, (float *)X32_out, E, M, N};
   return run_bf16_chain(&cp, 1, steps, coef, force_small, s);
@@ -723,7 +882,7 @@ static int pair_multi_impl(const char *who, const anc_ns_problem_t *probs, int32
                            const uint64_t *desc_tables, const NsUpdate *upd, int steps, const float *coef,
                            float eps, int mode, uint64_t stream) {
   ANC_REQUIRE(probs != nullptr && n_probs >= 1 && n_probs <= kMaxGroups, "%s: 1..%d problems", who, kMaxGroups);
-  ANC_REQUIRE(mode == ANC_NS_BF16 || mode == ANC_NS_BF16_FAST, "%s: bf16 modes only", who);
+  ANC_REQUIRE(mode == ANC_NS_BF16 || mode == ANC_NS_BF16_FAST || mode == ANC_NS_BF16_X3, "%s: bf16 modes only", who);
   ANC_REQUIRE(steps >= 2 && steps <= 64 && coef != nullptr, "%s: steps=%d: 2..64", who, steps);
   hipStream_t s = anc_stream(stream);
   ChainProb cp[kMaxGroups];
@@ -753,7 +912,10 @@ static int pair_multi_impl(const char *who, const anc_ns_problem_t *probs, int32
     ANC_REQUIRE(b.workspace_bytes >= pl.bytes, "%s: workspace holds %lld bytes, %lld needed", who,
                 (long long)b.workspace_bytes, (long long)pl.bytes);
     { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)b.E), dim3(kThreads), 0, s,
-                       (const double *)b.fro_partials, (int)b.n_partials, eps, pl.recip); }
+                       (const double *)b.fro_partials, (int)b.n_partials, eps, pl.recip, pl.pow2); }
+    ANC_LAUNCH_CHECK();
+    { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_pair_rescale, dim3((unsigned)(b.E * (b.M * b.N / 4096))), dim3(kThreads), 0, s,
+                       (uint16_t *)b.Uh, (uint16_t *)b.Ul, pl.pow2, (int)(b.M * b.N / 4096)); }
     ANC_LAUNCH_CHECK();
     cp[q] = ChainProb{pl, (const uint16_t *)b.Uh, (const uint16_t *)b.Ul, 0, pl.recip, (float *)b.X32_out, b.E, b.M, b.N,
                       desc_tables ? (const anc_muon_desc_t *)desc_tables[order[q]] : nullptr};

@@ -35,6 +35,7 @@ __device__ __forceinline__ void anc_pk_pair(float a, float b, uint32_t &hi, uint
 }
 
 constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int kCondParts = 8;            // partial sums per matrix of the conditioning proxy
 constexpr int PITCH = BK + 8;            // bf16 elements per LDS row: 144 bytes
 constexpr int kGemmThreads = 256;
 constexpr int kXcds = 8;
@@ -79,11 +80,28 @@ struct NsGemm {
   const anc_muon_desc_t *upd;  // BX, last step only: if set, matrix e is the Newton-Schulz result of the
                              // weight upd[e] and the epilogue applies W -= lr*O to it (p32, p16) instead
                              // of writing X32
+  const double *cond;        // null, or (E, kCondParts) partial sums of the conditioning proxy (see
+                             // k_ns_cond): a matrix whose sum exceeds cond_thresh multiplies
+                             // nterms_hard terms instead of nterms (its list is a prefix of the hard one)
+  double cond_thresh;
+  int nterms_hard;
   const float *scale;        // (E) or null. The operands are an unnormalised iterate U and the step
                              // acts on X = scale*U: GRAM multiplies its accumulator by scale^2, BX
                              // multiplies the accumulator and the epilogue's X by scale.
 };
 
+
+// Number of accumulation terms of matrix e: p.nterms, or p.nterms_hard for a matrix that the
+// conditioning proxy marks as hard. The partial sums are added in a fixed order, so every
+// workgroup of every launch takes the same decision for a matrix.
+__device__ __forceinline__ int anc_ns_terms(const NsGemm &p, int e) {
+  if (p.cond == nullptr) return p.nterms;
+  const double *c = p.cond + (int64_t)e * kCondParts;
+  double s = c[0];
+#pragma unroll
+  for (int i = 1; i < kCondParts; ++i) s = s + c[i];
+  return s > p.cond_thresh ? p.nterms_hard : p.nterms;
+}
 
 // Up to 8 independent problems of the same kind (the same product of different shape groups)
 // in one launch: tiles[k] workgroups belong to problem k. One launch over all groups keeps the

@@ -260,7 +260,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / NWN, wn = wave % NWN;
-  const int K = p.K, nk = K / TK, total = p.nterms * nk;
+  const int K = p.K, nk = K / TK, total = anc_ns_terms(p, e) * nk;
 
   // ---- DMA addressing: this wavefront moves IA*RPI rows of the A tile and IB*RPI rows of the B
   //      tile, RPI rows per instruction; lane -> (row lane/CPR, physical chunk lane%CPR). The

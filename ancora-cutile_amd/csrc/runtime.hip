@@ -73,7 +73,7 @@ extern "C" int anc_profile_read(float *ms, int64_t *launches) {
   g_prof_recs.clear();
   return ANC_OK;
 }
-extern "C" int anc_abi_version(void) { return 1; }
+extern "C" int anc_abi_version(void) { return 2; }
 
 int anc_gradnorm_static_init(void);   // gradnorm.hip: per-device address of its built-in scratch
 

@@ -17,7 +17,7 @@ import ctypes
 import numpy as np
 
 from . import _lib
-from ._lib import api, NS_BF16, NS_FP32, NS_BF16_FAST
+from ._lib import api, NS_BF16, NS_FP32, NS_BF16_FAST, NS_BF16_X3
 from .devbuf import DevBuf
 
 NTM, NTN, NTK = 128, 128, 64                       # ancora/kernels/muon_ns.py:20
@@ -30,7 +30,7 @@ PE_SCHEDULE = [(4.0848, -6.8946, 2.9270),
                (2.8769, -3.1427, 1.2046),
                (2.8366, -3.0525, 1.2012)]
 
-MODES = {"bf16": NS_BF16, "bf16_fast": NS_BF16_FAST, "fp32": NS_FP32,
+MODES = {"bf16": NS_BF16, "bf16_fast": NS_BF16_FAST, "bf16_x3": NS_BF16_X3, "fp32": NS_FP32,
          # same arithmetic forced onto the 128x128-tile kernel (ANC_NS_TILE128), for tests
          "bf16_tile128": NS_BF16 | 0x100, "bf16_fast_tile128": NS_BF16_FAST | 0x100}
 
@@ -111,6 +111,16 @@ def ns_flops(E, M, N, steps=5, mode="bf16"):
     ex, de = ctypes.c_double(0), ctypes.c_double(0)
     api.anc_ns_flops(E, M, N, int(steps), MODES[mode], ctypes.byref(ex), ctypes.byref(de))
     return ex.value, de.value
+
+
+def ns_hard_info(workspace_ptr, E, M, N, steps=5, mode="bf16", si=0):
+    """(n_hard, extra_flops_per_matrix) of the last chain call that used this workspace: how many
+    of its E matrices took the extra terms of the conditioning gate, and the matrix-core work
+    each adds to `ns_flops`' executed count. Synchronises stream `si`."""
+    n, ex = ctypes.c_int32(0), ctypes.c_double(0)
+    api.anc_ns_hard_info(int(workspace_ptr), int(E), int(M), int(N), MODES[mode], int(steps),
+                         ctypes.byref(n), ctypes.byref(ex), int(si))
+    return n.value, ex.value
 
 
 def ns_product_flops(E, M, N, k, product, steps=5, mode="bf16"):

@@ -59,6 +59,17 @@ def synth(shapes, seed=0):
     return params, grads
 
 
+def kernel_source_sha16():
+    """Hash of the Newton-Schulz kernel sources: ties a recorded counter figure to the code it was
+    measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in ("ns_common.h", "ns.hip", "ns_gemm_big.hip"):
+        with open(os.path.join(ROOT, "ancora-cutile_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def cpu_baseline(shapes, lr_adam=3e-4):
     """Numpy restatement of the reference host path (Muon.step + host_ns, AdamW test-oracle
     formula) timed on a bounded sample: one matrix of each Newton-Schulz shape and a 16M-element
@@ -309,7 +320,7 @@ def main():
         return side_workload(args)
     from ancora_cutile_amd import HybridOptimizer, DevBuf, PE_SCHEDULE, _lib
     from ancora_cutile_amd.hybrid import resident_is_muon
-    from ancora_cutile_amd.muon_ns import ns_flops, ns_product_flops
+    from ancora_cutile_amd.muon_ns import ns_flops, ns_product_flops, ns_hard_info
     from ancora_cutile_amd.shapes import qwen3_shapes, moe_shapes
 
     _lib.init(0)
@@ -364,11 +375,15 @@ def main():
     e0, e1 = _lib.Event(), _lib.Event()
     t0 = time.perf_counter()
     e0.record(0)
+    skipped = 0
     for _ in range(args.steps):
         opt.step(gdev, 0)
+        skipped += int(opt.last_skipped)
     e1.record(0)
     e1.sync()
     _lib.api.anc_device_sync()
+    if skipped:       # a skipped step returns early from every kernel and would time as falsely fast
+        sys.exit(f"bench.py: the guard skipped {skipped} of {args.steps} timed steps (non-finite gradient norm)")
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ev_ms = e0.elapsed_ms(e1) / args.steps
     ms_per_step = max(wall_ms, ev_ms)
@@ -388,10 +403,13 @@ def main():
     launches = {k: v[1] // prof_steps for k, v in prof.items() if v[1]}
 
     executed = dense = last_bx = 0.0
+    hard = 0           # matrices that took the extra terms of the conditioning gate in the last step
     for b in opt.muon.engine.batches:
         ex, de = ns_flops(b.E, b.M, b.Nn, 5, "bf16")
-        executed += ex
+        nh, extra = ns_hard_info(b.ws.buf.ptr, b.E, b.M, b.Nn, 5, "bf16")
+        executed += ex + nh * extra
         dense += de
+        hard += nh
         last_bx += ns_product_flops(b.E, b.M, b.Nn, 4, 2, 5, "bf16")
     # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
     # last X = a X + B X) also reads and writes the weights
@@ -415,13 +433,20 @@ def main():
     elem_moved = 14.0 if upd_fused else 26.0
     elem_gbps = elem_bytes * n_muon / (elem_ms * 1e-3) / 1e9
 
-    # HBM bytes per k_ns_gemm_big launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE on this
-    # same workload (two counter runs scaled by the copy kernel; summary under profiles/)
-    traffic = None
+    # HBM bytes per k_ns_gemm_big launch: NOT measured by this run (hardware counters need the
+    # profiler). The figure comes from two rocprofv3 --pmc runs of this same command (FETCH_SIZE,
+    # WRITE_SIZE, scaled by the copy kernel; summary under profiles/) and is reported only while
+    # the kernel sources still have the hash those runs were taken with; otherwise null.
+    traffic, traffic_note = None, "not measured in this run"
     tpath = os.path.join(ROOT, "profiles", "ns_gemm_traffic.json")
     if args.workload == "qwen3" and args.layers == 28 and os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+            tj = json.load(f)
+        if tj.get("source_sha16") == kernel_source_sha16():
+            traffic = tj.get("hbm_bytes_per_launch")
+            traffic_note = "static: rocprofv3 FETCH_SIZE + WRITE_SIZE runs recorded in " + tj.get("source", "profiles/")
+        else:
+            traffic_note = "profiles/ns_gemm_traffic.json was taken with other kernel sources: dropped"
 
     out = {
         "metric": METRIC if args.workload == "qwen3" else "MoE-16L Muon+AdamW step ms",
@@ -437,6 +462,7 @@ def main():
                    "layers": 16 if args.workload == "moe" else args.layers},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
+                     "traffic_source": traffic_note, "gated_hard_matrices": hard,
                      "kernel": "k_ns_gemm_big (gram, bmat, bx launches of the Newton-Schulz chain)",
                      "timed": "HIP events around each launch, chains serialised on one stream"
                               + ("; the last of the 15 launches also carries the fused weight update" if upd_fused else ""),
@@ -466,7 +492,7 @@ def main():
         "streams": "serial" if args.serial else "one: the Newton-Schulz chains of all shape groups advance together (grouped launches)",
         "copy_kernel_gbps": round(copy_gbps, 1),
         "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
-        "device": {"name": info["name"], "arch": info["arch"], "cus": info["cu_count"],
+        "device": {"name": info["name"] or info["arch"].split(":")[0], "arch": info["arch"], "cus": info["cu_count"],
                    "clock_khz": info["clock_khz"]},
     }
     opt.free()

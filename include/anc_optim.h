@@ -369,7 +369,22 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *                     residuals of X, A, B as extra accumulation terms.
  *   ANC_NS_BF16_FAST  as ANC_NS_BF16 without the residual terms (15 GEMM passes);
  *                     no accuracy bar of its own (about 2.2e-3 on 1024x1024).
+ *   ANC_NS_BF16_X3    every product also multiplies the bf16 residuals of both operands (three
+ *                     accumulation terms per product in every iteration): about 1e-5 from the
+ *                     fp32 chain on every input tried, ill-conditioned ones included, for three
+ *                     times the matrix-core work of ANC_NS_BF16_FAST.
  *   ANC_NS_FP32       every product in fp32 (validation mode).
+ *
+ * Conditioning gate (ANC_NS_BF16 only). After the first A = X X^T the chain measures
+ * N * ||offdiag(A)||_F^2 per matrix (1 for independent entries whatever the row scaling; N/r - N/M
+ * when the Frobenius mass sits in r directions spread over all rows, e.g. a few outlier columns).
+ * A matrix above 2.5 adds the residual of X to A = X X^T in iteration 2 (N >= 2M) or iterations 1
+ * and 2 (N < 2M): with 1 % of the columns scaled x100 that is 1.2e-3 / 8e-4 instead of 2.2e-3
+ * (1024x3072) / 3.8e-3 (1024x1024). The decision depends on the matrix alone (fixed-order sums),
+ * never on the batch. Accuracy bar of ANC_NS_BF16: 2e-3 relative Frobenius on inputs with
+ * independent entries, with row or column outliers up to x100; spectra spread over more than two
+ * decades (condition number >= 1e2 with a log-uniform spectrum) reach 2.5e-3 .. 4e-3 and need
+ * ANC_NS_BF16_X3.
  *
  * M and N must be multiples of 128 (the reference's tile alignment,
  * ancora/optim/muon.py:98). workspace must hold anc_ns_workspace_bytes(E,M,N,mode)
@@ -377,6 +392,7 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
 #define ANC_NS_BF16 0
 #define ANC_NS_FP32 1
 #define ANC_NS_BF16_FAST 2
+#define ANC_NS_BF16_X3 3
 /* Flag OR-ed into a bf16 mode: use the 128x128-tile GEMM kernel even where the 256x256-tile
  * kernel applies. Both produce the same bits; the flag exists so that tests can show it. */
 #define ANC_NS_TILE128 0x100
@@ -394,7 +410,11 @@ int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N,
  * X1 = s (a U + B U)). The fp32 result goes to X32_out, which may overlay the input pair
  * (Uh at X32_out, Ul right behind it: the same 4 bytes per element); steps >= 2. bf16
  * modes only. Results differ from anc_ns_batched on the same data only by where the bf16
- * rounding of the first operand falls (before instead of after the scaling). */
+ * rounding of the first operand falls (before instead of after the scaling). The first products
+ * run on the unnormalised values: a matrix whose sum of squares is below 2^-100 (||U||_F < 9e-16,
+ * where products of two elements would underflow fp32) is first multiplied in place, Uh and Ul,
+ * by the power of two that brings its norm into [1, 2), exactly, and its scale carries the
+ * inverse; every other matrix is left as it is. */
 int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partials, int64_t n_partials,
                         uint64_t X32_out, int64_t E, int64_t M, int64_t N,
                         int steps, const float *coef, float eps, int mode,
@@ -435,6 +455,11 @@ int anc_muon_ns_update_multi(const anc_ns_problem_t *problems, int32_t n_problem
  * `dense` is steps*(4 M^2 N + 2 M^3) per matrix. Roofline figures use `executed`. */
 int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
                  double *executed, double *dense);
+/* Of the E matrices of the last chain call that used `workspace`: how many took the extra
+ * terms of the conditioning gate, and the matrix-core work each of them adds to anc_ns_flops'
+ * `executed`. Synchronises `stream` and reads 64 bytes per matrix back. */
+int anc_ns_hard_info(uint64_t workspace, int64_t E, int64_t M, int64_t N, int mode, int steps,
+                     int32_t *n_hard, double *extra_flops_per_matrix, uint64_t stream);
 /* Executed matrix-core work of one product of one iteration of that chain: iteration k in
  * 0..steps-1, product 0 (A = X X^T), 1 (B = b A + c A A) or 2 (X = a X + B X). */
 int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, int mode, int k, int product,

@@ -77,7 +77,7 @@ def test_config4_moe_family_small(gpu):
                 continue
             _, u = muon_momentum(np.zeros_like(W[e]), G[e], clip=clip)
             want = muon_update(W[e], ns_any_shape(u, PE_SCHEDULE, 5), 0.02)
-            assert rel_fro(W[e] - got[e], W[e] - want) < 2.5e-3, (n, e)
+            assert rel_fro(W[e] - got[e], W[e] - want) < 2e-3, (n, e)
     for n in r["adamw"]:
         wd = 0.0 if params[n].ndim == 1 else 0.1
         want, _, _ = adamw_step_div(params[n], 0 * params[n], 0 * params[n], g[n], 3e-4, 0.9, 0.95, 1e-8,
@@ -131,4 +131,205 @@ def test_config5_flat_buffer_guard_and_update(gpu):
                                     0.95, 1e-8, 0.1, 1000, clip=c["clip_scale"])
         assert max_ulp(P[lo:hi], pw) == 0 and max_ulp(M_[lo:hi], mw) == 0 and max_ulp(V[lo:hi], vw) == 0
         assert bits_equal(P16[lo:hi], bf16_sr_bits(pw, sr_seed_base(11, 1000), first_index=lo))
+    gdev.free(); guard.free(); opt.free()
+
+
+def _zero_idle(rng, gb, g, params, idle_per_tensor=4):
+    """Config 4's sparsity: `idle_per_tensor` of the experts of every stacked tensor get an all-zero
+    gradient. Returns {name: sorted idle expert indices}."""
+    idle = {}
+    for n, p in params.items():
+        if p.ndim == 3:
+            idx = np.sort(rng.choice(p.shape[0], idle_per_tensor, replace=False))
+            g[n][idx] = 0
+            gb[n][idx] = 0
+            idle[n] = [int(i) for i in idx]
+    return idle
+
+
+def test_config4_moe_family_real_width(gpu):
+    """Config 4 at its real width: one dense layer (FFN 3072) and one MoE layer (16 experts of
+    1024x1024 per tensor, stacked [16,1024,1024]; router 1024x16 on AdamW), hidden 1024, 4 of 16
+    experts idle. 59 Muon matrices in three Newton-Schulz shape groups, all on the 256x256-tile
+    kernels, the (1024,1024) group with its residual-term iterations. Every expert of one stacked
+    tensor, three of each other and every 2-D projection against the numpy oracle at 2e-3."""
+    from ancora_cutile_amd import HybridOptimizer, resident_is_muon, PE_SCHEDULE as PE
+    from ancora_cutile_amd.shapes import moe_shapes
+    shapes = moe_shapes(layers=2, hidden=1024, dense_ffn=3072, experts=16, expert_ffn=1024, vocab=2048)
+    rng = np.random.default_rng(44)
+    params = {n: ((1 + 0.05 * rng.standard_normal(s)) if len(s) == 1 else 0.02 * rng.standard_normal(s))
+              .astype(np.float32) for n, s in shapes.items()}
+    gb, g = {}, {}
+    for n, p in params.items():
+        gb[n], g[n] = bf16_grad(rng, p.shape, 1e-3)
+    idle = _zero_idle(rng, gb, g, params)
+    opt = HybridOptimizer(params, is_muon=resident_is_muon, muon_kw=dict(schedule=PE),
+                          adamw_kw=dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.1),
+                          max_grad_norm=1.0, grad_dtype=np.uint16)
+    r = opt.routing()
+    assert "layer1.ffn.router" in r["adamw"] and len(r["muon"]) == 7 + 4 + 3
+    assert sorted((b.M, b.Nn, b.E) for b in opt.muon.engine.batches) == [(1024, 1024, 52), (1024, 2048, 4), (1024, 3072, 3)]
+    opt.step(gb, 0)
+    clip = opt.last_ctl["clip_scale"]
+    order = opt.muon_names + opt.adamw_names
+    assert opt.last_ctl["sumsq"] == gn.gradnorm_fixed([gb[n] for n in order])
+    mm, am = opt.muon.master(), opt.adamw.master()
+    worst = 0.0
+    for n in r["muon"]:
+        W = params[n].reshape((-1,) + params[n].shape[-2:])
+        G = g[n].reshape(W.shape)
+        got = mm[n].reshape(W.shape)
+        if W.shape[0] == 1:
+            picks = [0]
+        elif n.endswith("ffn.down_proj"):
+            picks = list(range(W.shape[0]))
+        else:
+            live = [e for e in range(W.shape[0]) if e not in idle[n]]
+            picks = sorted(set(idle[n] + live[:2] + live[-1:]))
+        for e in picks:
+            if not G[e].any():
+                assert e in idle[n] and bits_equal(got[e], W[e])        # idle expert: untouched at step 1
+                continue
+            _, u = muon_momentum(np.zeros_like(W[e]), G[e], clip=clip)
+            want = muon_update(W[e], ns_any_shape(u, PE_SCHEDULE, 5), 0.02)
+            err = rel_fro(W[e] - got[e], W[e] - want)
+            worst = max(worst, err)
+            assert err < 2e-3, (n, e, err)
+    print(f"\nconfig 4 at width 1024: worst update-direction error {worst:.3e}")
+    for n in r["adamw"]:
+        wd = 0.0 if params[n].ndim == 1 else 0.1
+        want, _, _ = adamw_step_div(params[n], 0 * params[n], 0 * params[n], g[n], 3e-4, 0.9, 0.95, 1e-8,
+                                    wd, 1, clip=clip)
+        assert max_ulp(am[n], want) == 0, n
+    opt.free()
+
+
+def test_config4_expert_optimizer_e16_1024(gpu):
+    """The reference's expert probe size (tests/kernels/_probe_expert_muon_ns.py:24-54: E=16 of
+    1024x1024, distinct experts) through the MoE layer's own optimizer class: three stacked tensors,
+    4 idle experts each, Polar-Express. Per expert: cos > 0.99 and rel < 0.05 (the reference's bars:
+    no cross-matrix leak) and the 2e-3 bar against the oracle; idle experts untouched; the transposed
+    bf16 copy the backward reads equals the transpose of the new bf16 weights; router on AdamW."""
+    from ancora_cutile_amd import DevBuf, PE_SCHEDULE as PE
+    from ancora_cutile_amd.moe import ExpertOptimizer
+    from oracle.adamw_ref import adamw_step_ibc
+    E, H = 16, 1024
+    rng = np.random.default_rng(45)
+    weights = {n: (0.02 * rng.standard_normal((E, H, H))).astype(np.float32) for n in ExpertOptimizer.NAMES}
+    router = (0.02 * rng.standard_normal((H, E))).astype(np.float32)
+    gb, g = {}, {}
+    for n in weights:
+        gb[n], g[n] = bf16_grad(rng, (E, H, H), 1e-3)
+    idle = _zero_idle(rng, gb, g, weights)
+    rgrad = (1e-3 * rng.standard_normal((H, E))).astype(np.float32)
+    opt = ExpertOptimizer(weights, router=router, optimizer="muon")
+    gdev = {n: DevBuf(gb[n].reshape(E * H, H)) for n in weights}
+    rdev = DevBuf(rgrad.reshape(-1, 64))
+    opt.step(gdev, 0, lr=1e-3, muon_lr=0.02, router_grad=rdev, schedule=PE)
+    gpu.stream_sync(0)
+    got = opt.master()
+    for n in weights:
+        s = opt.st[n]
+        p16 = s["p16"].to_numpy().reshape(E, H, H)
+        p16T = s["p16T"].to_numpy().reshape(E, H, H)
+        for e in range(E):
+            assert bits_equal(p16T[e], np.ascontiguousarray(p16[e].T)), (n, e)
+            if e in idle[n]:
+                assert bits_equal(got[n][e], weights[n][e]), (n, e)
+                continue
+            if n != "up_proj" and e not in (0, 7, 15):
+                continue
+            _, u = muon_momentum(np.zeros((H, H), np.float32), g[n][e])
+            o_ref = host_ns(u, PE_SCHEDULE, 5)
+            o_got = (weights[n][e].astype(np.float64) - got[n][e]) / 0.02
+            cos = float(np.sum(o_got * o_ref) / (np.linalg.norm(o_got) * np.linalg.norm(o_ref)))
+            assert cos > 0.99 and rel_fro(o_got, o_ref) < 0.05, (n, e)            # reference bars
+            assert rel_fro(o_got, o_ref) < 2e-3, (n, e, rel_fro(o_got, o_ref))
+    b1, b2 = 0.9, 0.999
+    want, _, _ = adamw_step_ibc(router, 0 * router, 0 * router, rgrad, 1e-3, b1, b2, 1e-8, 0.0,
+                                1.0 / (1.0 - b1), 1.0 / (1.0 - b2))
+    assert max_ulp(got["router"], want) <= 1
+    for b in list(gdev.values()) + [rdev]:
+        b.free()
+    opt.free()
+
+
+def _tiled(base, n, scale_step):
+    """n-element fp32 array made of copies of `base`, copy k scaled by 1 + k*scale_step: cheap to
+    build at 1.2e9 elements, different bits in every copy."""
+    out = np.empty(n, np.float32)
+    B = base.size
+    for k, lo in enumerate(range(0, n, B)):
+        hi = min(n, lo + B)
+        np.multiply(base[:hi - lo], np.float32(1.0 + k * scale_step), out=out[lo:hi])
+    return out
+
+
+def _block(buf, lo, hi):
+    """Elements [lo, hi) of a (R, 64) device buffer, lo and hi multiples of 64."""
+    return buf.at_pos(lo // 64).view(((hi - lo) // 64, 64)).to_numpy().ravel()
+
+
+def test_config5_flat_buffer_full_size(gpu):
+    """Config 5 at its real size, one flat 1.2e9-element buffer (fp32 master, m, v: 4.8 GB each,
+    byte offsets beyond 2^32 from element 2^30 on; bf16 gradient and weights 2.4 GB), step 1000.
+    Gradient with 0.01 % Inf/NaN: the guard skips, the master (all of it), the bf16 weights (all)
+    and sampled blocks of m and v keep their bits. Clean gradient: sum of squares bit-equal to the
+    fixed-order oracle, norm within 1 ulp of the fp64 closed form; m, v, master 0 ulp and stochastic
+    bf16 bits equal on blocks at the start, across elements 2^29 and 2^30 (byte offsets 2^31 and
+    2^32 of the fp32 arrays), deep in the upper part and at the very end."""
+    from ancora_cutile_amd import AdamW, StepGuard, DevBuf
+    from ancora_cutile_amd.adamw import sr_seed_base
+    n = 1_200_000_000
+    B = 1 << 24
+    rng = np.random.default_rng(55)
+    p = _tiled(rng.standard_normal(B, dtype=np.float32), n, 2.0 ** -12)
+    m0 = _tiled(1e-3 * rng.standard_normal(B, dtype=np.float32), n, 2.0 ** -11)
+    v0 = _tiled(1e-6 * rng.random(B, dtype=np.float32), n, 2.0 ** -10)
+    gbase = bf16_rne_bits(1e-3 * rng.standard_normal(B, dtype=np.float32))
+    gbits = np.empty(n, np.uint16)
+    for k, lo in enumerate(range(0, n, B)):
+        hi = min(n, lo + B)
+        gbits[lo:hi] = gbase[:hi - lo] ^ np.uint16(0x8000 if k & 1 else 0)      # alternate the sign per copy
+    opt = AdamW({"flat": p}, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.1, sr=True, seed=11,
+                grad_dtype=np.uint16)
+    s = opt.st["flat"]
+    s["m"].upload(m0.reshape(-1, 64))
+    s["v"].upload(v0.reshape(-1, 64))
+    opt.t = 999
+    guard = StepGuard(1.0)
+    spans = [(0, 8192), ((1 << 29) - 4096, (1 << 29) + 4096), ((1 << 30) - 4096, (1 << 30) + 4096),
+             (1_150_000_000 // 64 * 64, 1_150_000_000 // 64 * 64 + 8192), (n - 4096 * 3, n), (n - 64, n)]
+    # -- 0.01 % non-finite: skipped, nothing written
+    idx = rng.choice(n, n // 10000, replace=False)
+    saved = gbits[idx].copy()
+    gbits[idx] = rng.choice(np.array([0x7F80, 0xFF80, 0x7FC0], np.uint16), idx.size)
+    gdev = DevBuf(gbits)
+    guard.compute([gdev], 0)
+    opt.step({"flat": gdev}, 0, guard=guard)
+    assert guard.read(0)["skip"] and opt.t == 999 and opt.last_skipped
+    assert bits_equal(s["p32"].to_numpy().ravel(), p) and not s["p16"].to_numpy().any()
+    for lo, hi in spans:
+        assert bits_equal(_block(s["m"], lo, hi), m0[lo:hi]) and bits_equal(_block(s["v"], lo, hi), v0[lo:hi])
+    # -- clean gradient: the update
+    gbits[idx] = saved
+    gdev.upload(gbits)
+    guard.compute([gdev], 0)
+    opt.step({"flat": gdev}, 0, guard=guard)
+    c = guard.read(0)
+    assert not c["skip"] and opt.t == 1000
+    parts = np.concatenate([gn.chunk_partials(gbits[lo:lo + B]) for lo in range(0, n, B)])   # B % 8192 == 0
+    assert c["sumsq"] == gn.finalize_fixed(parts)
+    f64 = sum(gn.gradnorm_f64([gbits[lo:lo + B]]) for lo in range(0, n, B))
+    assert max_ulp(np.float32(c["norm"]), np.float32(gn.control(f64)["norm"])) <= 1
+    for lo, hi in spans:
+        gseg = bits_to_f32(gbits[lo:hi])
+        pw, mw, vw = adamw_step_div(p[lo:hi], m0[lo:hi], v0[lo:hi], gseg, 3e-4, 0.9, 0.95, 1e-8, 0.1, 1000,
+                                    clip=c["clip_scale"])
+        assert max_ulp(_block(s["p32"], lo, hi), pw) == 0, lo
+        assert max_ulp(_block(s["m"], lo, hi), mw) == 0 and max_ulp(_block(s["v"], lo, hi), vw) == 0, lo
+        assert bits_equal(_block(s["p16"], lo, hi), bf16_sr_bits(pw, sr_seed_base(11, 1000), first_index=lo)), lo
+    # every element was updated: the master moved everywhere the gradient or the decay is non-zero
+    P = s["p32"].to_numpy().ravel()
+    assert np.count_nonzero(P != p) > 0.999 * n
     gdev.free(); guard.free(); opt.free()

@@ -38,7 +38,7 @@ def test_config1_minimal_hybrid_step(gpu):
     # the update direction (W0 - W1)/lr is the orthogonalised momentum: 2e-3 bar
     upd_got = (params["layer0.q_proj"].astype(np.float64) - mm) / 0.02
     upd_ref = (params["layer0.q_proj"].astype(np.float64) - mr.w["layer0.q_proj"]) / 0.02
-    assert rel_fro(upd_got, upd_ref) < 2.5e-3       # 2e-3 chain + fp32 rounding of W - lr*O
+    assert rel_fro(upd_got, upd_ref) < 2e-3
     assert bits_equal(opt.muon.momentum_buffers()["layer0.q_proj"], mr.buf["layer0.q_proj"])
     w = opt.weights()
     assert np.array_equal(w["embed"], bits_to_f32(bf16_rne_bits(am["embed"])).reshape(1024, 1024))
@@ -172,7 +172,7 @@ def test_expert_optimizer(gpu, Ie):
         _, u = muon_momentum(np.zeros((K, N), np.float32), G[n][0])
         want = muon_update(W[n][0], ns_any_shape(u, PE_SCHEDULE, 5), 0.02)
         step = 0.02 * shape_scale(K, N)
-        assert rel_fro((W[n][0] - m[n][0]) / step, (W[n][0] - want) / step) < 2.5e-3
+        assert rel_fro((W[n][0] - m[n][0]) / step, (W[n][0] - want) / step) < 2e-3
         s = opt.st[n]
         p16 = s["p16"].to_numpy().reshape(E, K, N)
         assert np.array_equal(s["p16T"].to_numpy().reshape(E, N, K), p16.transpose(0, 2, 1))

@@ -44,9 +44,14 @@ def test_bf16_mode_within_2e3(gpu, M, N, sched):
     schedule = PE_SCHEDULE if sched == "pe" else None
     X = rng.standard_normal((2, M, N)).astype(np.float32)
     got = run_ns(X, schedule=schedule, mode="bf16")
-    tol = TOL_BF16 if sched == "pe" else 6e-3      # Keller amplifies rounding ~2x more (no bar set)
+    # Keller's quintic amplifies operand rounding about twice as much as the Polar-Express schedule
+    # every BASELINE configuration uses: default mode held to 5e-3, the bar itself in bf16_x3 below
+    tol = TOL_BF16 if sched == "pe" else 5e-3
     for e in range(2):
         assert rel_fro(got[e], host_ns(X[e], schedule, 5)) < tol
+    if sched == "keller" and M in (256, 1024):
+        got = run_ns(X[:1], schedule=None, mode="bf16_x3")
+        assert rel_fro(got[0], host_ns(X[0], None, 5)) < 2e-4
 
 
 def test_reference_probe_inputs(gpu):
@@ -60,9 +65,13 @@ def test_reference_probe_inputs(gpu):
         X = bits_to_f32(bf16_rne_bits(X)).reshape(X.shape)
         got = run_ns(X[None], schedule=None)[0]
         want = ns5_ref(X, 5)
-        assert rel_fro(got, want) < 0.05
+        assert rel_fro(got, want) < 0.05                   # the reference-held leg (Keller)
         sg, sw = np.linalg.svd(got, compute_uv=False), np.linalg.svd(want, compute_uv=False)
         assert abs(sg.min() - sw.min()) < 0.03 and abs(sg.max() - sw.max()) < 0.03
+        pe = run_ns(X[None], schedule=PE_SCHEDULE)[0]      # the bar of this build
+        err = rel_fro(pe, host_ns(X, PE_SCHEDULE, 5))
+        print(f"probe input {X.shape}: Polar-Express chain {err:.3e}")
+        assert err < TOL_BF16
 
 
 def test_polar_express_orthogonalises_better_than_keller(gpu):
@@ -180,6 +189,46 @@ def test_pair_entry_folds_the_normalisation(gpu, M, N, mode):
     U.free(); fro.free()
 
 
+def _pair_run(X, eps, mode="bf16", nper=4):
+    """X (E,M,N) fp32 -> anc_ns_batched_pair on its exact bf16 pair and fp64 sums of squares."""
+    from ancora_cutile_amd import DevBuf
+    from ancora_cutile_amd.muon_ns import ns_batched_pair
+    E, M, N = X.shape
+    hi = bf16_rne_bits(X).reshape(E, M, N)
+    lo = bf16_rne_bits(X - bits_to_f32(hi).reshape(E, M, N)).reshape(E, M, N)
+    U = DevBuf(np.concatenate([hi.reshape(-1), lo.reshape(-1)]).view(np.float32))
+    parts = (X.astype(np.float64) ** 2).reshape(E, nper, -1).sum(axis=2)
+    fro = DevBuf(np.ascontiguousarray(parts))
+    ns_batched_pair(U, fro, nper, E, M, N, 0, steps=5, eps=eps, schedule=PE_SCHEDULE, mode=mode)
+    got = U.to_numpy().reshape(E, M, N)
+    U.free(); fro.free()
+    return got
+
+
+@pytest.mark.parametrize("M,N", [(256, 512), (1024, 1024)])
+def test_pair_entry_tiny_inputs_do_not_underflow(gpu, M, N):
+    """The fused-prologue entry multiplies unnormalised values, and products of elements below
+    about 1e-19 underflow fp32. Such a matrix is pre-scaled by an exact power of two on the device:
+    with eps = 0 the result for X * 2^-90 (elements ~1e-30) has the bits of the result for X, and a
+    normal matrix in the same batch is untouched. With the reference's eps = 1e-7 a tiny gradient
+    gives the tiny, nearly linear result of the fp32 chain (evaluated in fp64 to keep the oracle's
+    own norm from underflowing)."""
+    rng = np.random.default_rng(M + N)
+    X = (1e-3 * rng.standard_normal((2, M, N))).astype(np.float32)
+    tiny = X.copy()
+    tiny[1] *= np.float32(2.0 ** -90)
+    a, b = _pair_run(X, 0.0), _pair_run(tiny, 0.0)
+    assert bits_equal(a, b)
+    assert rel_fro(a[1], host_ns(X[1], PE_SCHEDULE, 5, eps=0.0)) < TOL_BF16
+    got = _pair_run(tiny, 1e-7)[1].astype(np.float64)
+    Y = tiny[1].astype(np.float64)
+    Y = Y / (np.linalg.norm(Y) + 1e-7)
+    for (ca, cb, cc) in PE_SCHEDULE:
+        A = Y @ Y.T
+        Y = ca * Y + (cb * A + cc * (A @ A)) @ Y
+    assert np.linalg.norm(Y) > 0 and rel_fro(got, Y) < TOL_BF16
+
+
 def test_grouped_launch_equals_per_batch_bits(gpu):
     """anc_ns_batched_pair_multi (one launch per product over several shape groups) gives each
     batch the bits of anc_ns_batched_pair on that batch alone; batch order does not matter."""
@@ -216,3 +265,71 @@ def test_grouped_launch_equals_per_batch_bits(gpu):
         for t in bufs:
             for b in t:
                 b.free()
+
+
+def _outlier_cols(rng, M, N, frac=0.01, scale=100.0):
+    X = rng.standard_normal((M, N)).astype(np.float32)
+    X[:, rng.choice(N, max(1, int(N * frac)), replace=False)] *= np.float32(scale)
+    return X
+
+
+def _log_spectrum(rng, M, N, cond):
+    U, _ = np.linalg.qr(rng.standard_normal((M, M)))
+    V, _ = np.linalg.qr(rng.standard_normal((N, M)))
+    return ((U * np.logspace(0, -np.log10(cond), M)) @ V.T).astype(np.float32)
+
+
+def _hard_count(E, M, N, mode="bf16"):
+    from ancora_cutile_amd import muon_ns
+    return muon_ns.ns_hard_info(muon_ns._SHARED_WS.buf.ptr, E, M, N, 5, mode)
+
+
+@pytest.mark.parametrize("M,N", [(256, 256), (1024, 1024), (1024, 2048), (1024, 3072)])
+def test_outlier_columns_take_the_gate_and_meet_the_bar(gpu, M, N):
+    """1 % of the columns scaled x100 (what the transposed iterate of a tall weight with outlier
+    rows looks like): the conditioning proxy marks the matrix, the extra A = X X^T terms bring it
+    inside 2e-3. A Gaussian matrix and one with outlier ROWS in the same batch are not marked and
+    keep the bits they have in a batch of their own."""
+    rng = np.random.default_rng(M + N + 1)
+    cols = _outlier_cols(rng, M, N)
+    gauss = rng.standard_normal((M, N)).astype(np.float32)
+    rows = rng.standard_normal((M, N)).astype(np.float32)
+    rows[rng.choice(M, max(1, M // 100), replace=False)] *= np.float32(100.0)
+    X = np.stack([gauss, cols, rows])
+    got = run_ns(X)
+    n_hard, extra = _hard_count(3, M, N)
+    assert n_hard == 1 and extra > 0
+    errs = [rel_fro(got[e], host_ns(X[e], PE_SCHEDULE, 5)) for e in range(3)]
+    print(f"({M},{N}) gaussian {errs[0]:.3e}  outlier columns {errs[1]:.3e}  outlier rows {errs[2]:.3e}")
+    assert max(errs) < TOL_BF16
+    alone = run_ns(X[:1])
+    assert _hard_count(1, M, N)[0] == 0
+    assert bits_equal(alone[0], got[0])
+    assert bits_equal(run_ns(X[1:2])[0], got[1]) and _hard_count(1, M, N)[0] == 1
+    fast = run_ns(X[1:2], mode="bf16_fast")          # no residual terms, no gate
+    assert _hard_count(1, M, N, "bf16_fast") == (0, 0.0)
+    assert rel_fro(fast[0], host_ns(X[1], PE_SCHEDULE, 5)) > errs[1]
+
+
+@pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 1536)])
+def test_wide_spectrum_inputs_default_bound_and_x3_mode(gpu, M, N):
+    """Singular values spread log-uniformly over three decades (condition number 1e3). The default
+    bf16 mode does NOT meet 2e-3 here: its error is pinned between 2e-3 and 4.5e-3 so that a
+    regression, or a fix, shows. The three-term mode meets the bar with a wide margin."""
+    rng = np.random.default_rng(N)
+    X = _log_spectrum(rng, M, N, 1e3)
+    want = host_ns(X, PE_SCHEDULE, 5)
+    err = rel_fro(run_ns(X[None])[0], want)
+    err3 = rel_fro(run_ns(X[None], mode="bf16_x3")[0], want)
+    print(f"({M},{N}) cond 1e3: bf16 {err:.3e}, bf16_x3 {err3:.3e}")
+    assert 2e-3 < err < 4.5e-3
+    assert err3 < 2e-4
+
+
+def test_x3_mode_on_every_shape_class(gpu):
+    rng = np.random.default_rng(77)
+    for (M, N) in ((128, 256), (512, 512), (1024, 3072)):
+        X = np.stack([rng.standard_normal((M, N)).astype(np.float32), _outlier_cols(rng, M, N)])
+        got = run_ns(X, mode="bf16_x3")
+        for e in range(2):
+            assert rel_fro(got[e], host_ns(X[e], PE_SCHEDULE, 5)) < 1e-4, (M, N, e)

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} declared in include/anc_optim.h but not exported"
     assert sorted(_lib.EXPORTS) == names, "ctypes prototypes and header disagree"
     _lib.load()
-    assert _lib.api.anc_abi_version() == 1
+    assert _lib.api.anc_abi_version() == 2
 
 
 def test_struct_sizes_match_header():
