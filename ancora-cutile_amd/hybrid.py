@@ -57,7 +57,15 @@ class HybridOptimizer:
         if no_decay is None:
             no_decay = lambda n, p: (p.ndim == 1)          # noqa: E731  don't decay 1-D gains/biases
 
-        self.muon_names = [n for n, p in params.items() if is_muon(n, p)]
+        # A matrix the predicate sends to Muon but whose dims are not multiples of 128 (the (H, E)
+        # router of a MoE model under `default_is_muon`) cannot enter the batched chain; the
+        # reference runs its Newton-Schulz on the host for those (`_ns_ok`,
+        # ancora/optim/muon.py:37-41), here it goes to AdamW, as in the resident models
+        # (ancora/kernels/moe.py:603-604).
+        def _aligned(p):
+            return p.shape[-2] % NTM == 0 and p.shape[-1] % NTM == 0
+        self.muon_names = [n for n, p in params.items() if is_muon(n, p) and _aligned(p)]
+        self.misaligned_to_adamw = [n for n, p in params.items() if is_muon(n, p) and not _aligned(p)]
         self.adamw_names = [n for n in params if n not in self.muon_names]
         self.muon = Muon({n: params[n] for n in self.muon_names}, grad_dtype=grad_dtype, **muon_kw)
         self.adamw = AdamW({n: params[n] for n in self.adamw_names},
@@ -135,10 +143,16 @@ class HybridOptimizer:
     def save(self, path):
         """Checkpoint to one uncompressed .npz (plain arrays, no pickle): a run resumed with
         `load` continues bit for bit. The reference keeps optimizer state in memory only."""
-        np.savez(path, **self.state_dict())
+        np.savez(self._npz(path), **self.state_dict())
+
+    @staticmethod
+    def _npz(path):
+        """np.savez appends '.npz' to a name without it; `load` must look for the same file."""
+        path = str(path)
+        return path if path.endswith(".npz") else path + ".npz"
 
     def load(self, path, stream_int=0):
-        with np.load(path, allow_pickle=False) as z:
+        with np.load(self._npz(path), allow_pickle=False) as z:
             self.load_state_dict({k: z[k] for k in z.files}, stream_int)
 
     def weights(self):

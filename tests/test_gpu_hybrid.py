@@ -200,7 +200,7 @@ def test_checkpoint_resume_is_bitwise(gpu, tmp_path):
     a = HybridOptimizer(params, **kw)
     for g in grads[:2]:
         a.step(g, 0)
-    path = str(tmp_path / "opt.npz")
+    path = str(tmp_path / "opt")              # no extension: save and load agree on "opt.npz"
     a.save(path)
     for g in grads[2:]:
         a.step(g, 0)
@@ -213,6 +213,28 @@ def test_checkpoint_resume_is_bitwise(gpu, tmp_path):
     for k in sa:
         assert np.atleast_1d(sa[k]).tobytes() == np.atleast_1d(sb[k]).tobytes(), k
     a.free(); b.free()
+
+
+def test_default_predicate_with_a_misaligned_router(gpu):
+    """`HybridOptimizer(model.params())` on a MoE parameter set with the default predicate
+    (tests/training/test_moe_pipeline.py:36): the (H, E) router is 2-D, so the predicate names it
+    for Muon, but it is not 128-aligned; it goes to AdamW instead of raising, and the step runs."""
+    from ancora_cutile_amd import HybridOptimizer
+    rng = np.random.default_rng(8)
+    params = {"embed": (0.02 * rng.standard_normal((256, 128))).astype(np.float32),
+              "layer1.ffn.router": (0.02 * rng.standard_normal((128, 16))).astype(np.float32),
+              "layer1.ffn.gate_proj": (0.02 * rng.standard_normal((4, 128, 128))).astype(np.float32),
+              "layer1.q_proj": (0.02 * rng.standard_normal((128, 256))).astype(np.float32)}
+    opt = HybridOptimizer(params)
+    assert opt.routing() == {"muon": ["layer1.q_proj"],
+                             "adamw": ["embed", "layer1.ffn.router", "layer1.ffn.gate_proj"]}
+    assert opt.misaligned_to_adamw == ["layer1.ffn.router"]
+    grads = {n: (1e-2 * rng.standard_normal(p.shape)).astype(np.float32) for n, p in params.items()}
+    opt.step(grads, 0)
+    ar = AdamWRef({n: params[n] for n in opt.adamw_names}, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.01)
+    ar.step(grads)
+    assert max_ulp(opt.adamw.master()["layer1.ffn.router"], ar.st["layer1.ffn.router"]["p"]) == 0
+    opt.free()
 
 
 @pytest.mark.parametrize("sr", [False, True])
