@@ -12,6 +12,10 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
     python3 -m ancora_cutile_amd.prof_target dw T K N1[,N2,..] [calls]   weight-gradient GEMM of up to 8
                                       weights (K, Ni) that share the activations, T tokens
 
+    python3 -m ancora_cutile_amd.prof_target copy [GiB] [reps]          streaming-kernel shapes
+                                      (anc_copy_shape): TB/s of each, the reference points for
+                                      the elementwise optimizer kernels
+
 Each target allocates its operands, runs the kernel(s) `calls` times on the null stream and
 synchronises; nothing is checked here (parity lives in tests/).
 """
@@ -130,6 +134,28 @@ def main(argv):
         gms, rms = pr["dw_gemm"][0] / calls, pr["dw_reduce"][0] / calls
         print(f"dW of one layer (7 weights, T={T}, 1 segment, 480 workgroups): gemm {gms * 1e3:.1f} us "
               f"({fl / gms / 1e9:.1f} TFLOP/s), finish {rms * 1e3:.1f} us, together {fl / (gms + rms) / 1e9:.1f} TFLOP/s")
+    elif what == "copy":
+        gib = float(argv[1]) if len(argv) > 1 else 1.0
+        reps = int(argv[2]) if len(argv) > 2 else 5
+        nb = int(gib * (1 << 30)) // (1 << 20) * (1 << 20)
+        a, b = DevBuf.empty((nb // 4,), np.float32), DevBuf.empty((nb // 4,), np.float32)
+        a.fill_zero(0)
+        b.fill_zero(0)
+        names = ("copy 4x16B nt", "copy 4x16B plain", "copy 8x16B nt", "copy persistent 2048 wg", "copy 1024-lane wg",
+                 "read only", "write only", "AdamW mix 4R+4W (14+14 B/elem)", "momentum mix 2R+3W (6+8 B/elem)")
+        e0, e1 = _lib.Event(), _lib.Event()
+        moved = ctypes.c_int64(0)
+        print(f"two buffers of {nb / 2 ** 30:.2f} GiB, {reps} launches each, HIP events around the launches")
+        for shape, name in enumerate(names):
+            _lib.api.anc_copy_shape(b.ptr, a.ptr, nb, shape, ctypes.byref(moved), 0)
+            e0.record(0)
+            for _ in range(reps):
+                _lib.api.anc_copy_shape(b.ptr, a.ptr, nb, shape, ctypes.byref(moved), 0)
+            e1.record(0)
+            e1.sync()
+            ms = e0.elapsed_ms(e1) / reps
+            print(f"  shape {shape}  {name:34s} {moved.value / 1e9:7.3f} GB in {ms * 1e3:8.1f} us = "
+                  f"{moved.value / ms / 1e9:6.3f} TB/s = {moved.value / ms / 1e9 / 8 * 100:5.1f} % of 8 TB/s")
     else:
         raise SystemExit(__doc__)
     _lib.api.anc_device_sync()

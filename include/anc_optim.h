@@ -89,6 +89,17 @@ int anc_event_elapsed_ms(uint64_t start, uint64_t stop, float *ms);
 /* Plain streaming copy kernel of n_bytes (multiple of 16): the calibration
  * reference for HBM traffic counters and the measured copy ceiling. */
 int anc_copy_kernel(uint64_t dst, uint64_t src, int64_t n_bytes, uint64_t stream);
+/* The same streaming traffic in other kernel shapes, to establish what an elementwise kernel can
+ * reach on this memory system (no reference counterpart; the reference's own method is a timed
+ * copy beside its AdamW kernel, tests/hardware/_probe_adamw_bw.py:24-25,58-91). shape: 0 as
+ * anc_copy_kernel; 1 ordinary instead of non-temporal accesses; 2 eight 16-byte accesses in
+ * flight per lane; 3 2048 persistent workgroups, grid-stride; 4 1024 lanes per workgroup; 5 read
+ * only; 6 write only; 7 AdamW's access mix without its arithmetic (four read streams of 2+4+4+4
+ * and four write streams of 4+4+4+2 bytes per element, same block and lane layout); 8 the Muon
+ * momentum kernel's mix (read 2+4, write 4+2+2). n_bytes (a multiple of 1 MiB) is the size of
+ * each of the two buffers; *bytes_moved receives the bytes read plus written. */
+int anc_copy_shape(uint64_t dst, uint64_t src, int64_t n_bytes, int shape, int64_t *bytes_moved,
+                   uint64_t stream);
 
 /* ------------------------------------------------------------- profiling ----
  * Per-kernel timing with HIP events on the launch stream, for the benchmarks (the
