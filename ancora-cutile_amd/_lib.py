@@ -113,6 +113,9 @@ _PROTOS = {
                          u64, u64]),
     "anc_adamw_num_blocks": (i64, [i64]),
     "anc_adamw_multi": (None, [u64, i32, i64, C.POINTER(AdamWHyper), u64, u64]),
+    "anc_adamw_rows": (None, [u64, i64, u64, u64, u64, u64, u64, u64, i64, i64, u64, i32,
+                              C.POINTER(AdamWHyper), f32, u32, u64, u64]),
+    "anc_embed_dw_scatter": (None, [u64, u64, u64, u64, u64, u64, u64, i64, i64, i64, u64]),
     "anc_cast_bf16": (None, [u64, u64, i64, C.c_int, u32, u64]),
     "anc_muon_momentum": (None, [u64, u64, u64, i64, i64, f32, C.c_int, C.c_int, C.c_int,
                                  C.c_int, u64, u64]),

@@ -188,6 +188,72 @@ k_cast_bf16(const float *__restrict__ p32, uint16_t *__restrict__ p16, int64_t n
   }
 }
 
+
+// ---- row-sparse AdamW, dense-equivalent ---------------------------------------------------
+// For a (V, H) tensor whose gradient touches few rows per step (an input embedding that is not
+// tied to the output head). A dense step on a row with zero gradient still moves it (m and v decay,
+// the bias-corrected momentum and the weight decay keep updating p), so skipping untouched rows
+// changes the result; instead every row remembers the last step it is current for, and when it is
+// next needed the steps it missed are replayed on it, each with g = 0 and that step's own scalars
+// (bias corrections, learning rate, rounding seed) from a per-step table, through the same
+// per-element routine as the dense kernel. The state of a row that is current is therefore
+// bit-identical to what the dense kernel would hold. A row is brought up to date (a) before the
+// forward pass gathers it (anc_adamw_rows with grads = 0: replay through step t_now) and (b) by
+// the step itself (replay through t_now - 1, then step t_now with its gradient row).
+struct RowStep { float bc1, bc2, lr; uint32_t seed_base; };   // entry s: counted step s (1-based)
+
+template <int FORM, int SR>
+__global__ void __launch_bounds__(kThreads)
+k_adamw_rows(const int32_t *__restrict__ rows, const float *__restrict__ grads, float *__restrict__ m,
+             float *__restrict__ v, float *__restrict__ p32, uint16_t *__restrict__ p16,
+             int32_t *__restrict__ last, int H, int64_t V, const RowStep *__restrict__ table, int t_now,
+             anc_adamw_hyper_t h, float wd, uint32_t seed, const anc_step_ctl_t *__restrict__ ctl) {
+  float clip;
+  if (!load_ctl(ctl, clip)) return;                      // skipped step: nothing is touched
+  const int64_t row = rows != nullptr ? (int64_t)rows[blockIdx.x] : (int64_t)blockIdx.x;
+  if (row < 0 || row >= V) return;
+  const int k0 = last[row];
+  __syncthreads();                                       // every lane has read `last` before lane 0 rewrites it
+  const bool with_step = grads != nullptr;
+  const int t_replay = with_step ? t_now - 1 : t_now;    // replay (g = 0) through this step
+  if (k0 >= t_now || (!with_step && k0 >= t_replay)) return;
+  for (int c = (int)threadIdx.x * kVec; c < H; c += kSlab) {
+    const int64_t e = row * H + c;
+    const anc_f32x4 m4 = *(const anc_f32x4 *)(m + e), v4 = *(const anc_f32x4 *)(v + e), p4 = *(const anc_f32x4 *)(p32 + e);
+    float mm[4] = {m4.x, m4.y, m4.z, m4.w}, vv[4] = {v4.x, v4.y, v4.z, v4.w}, pp[4] = {p4.x, p4.y, p4.z, p4.w};
+    anc_adamw_hyper_t hs = h;
+    uint32_t seed_step = 0;
+    for (int s = k0 + 1; s <= t_replay; ++s) {
+      const RowStep rs = table[s];
+      hs.bc1 = rs.bc1; hs.bc2 = rs.bc2; hs.lr = rs.lr;
+      seed_step = rs.seed_base;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) adamw_elem<FORM>(0.0f, mm[k], vv[k], pp[k], hs, wd, 1.0f);
+    }
+    if (with_step) {
+      const RowStep rs = table[t_now];
+      hs.bc1 = rs.bc1; hs.bc2 = rs.bc2; hs.lr = rs.lr;
+      seed_step = rs.seed_base;
+      const anc_f32x4 g4 = *(const anc_f32x4 *)(grads + (int64_t)blockIdx.x * H + c);
+      const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) adamw_elem<FORM>(gg[k], mm[k], vv[k], pp[k], hs, wd, clip);
+    }
+    uint32_t hb[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint64_t i = (uint64_t)(e + k);
+      hb[k] = SR ? anc_bf16_sr_bits(pp[k], (uint32_t)(i >> 6), (uint32_t)(i & 63u), seed_step + seed)
+                 : anc_bf16_rne_bits(pp[k]);
+    }
+    *(anc_f32x4 *)(m + e) = anc_f32x4{mm[0], mm[1], mm[2], mm[3]};
+    *(anc_f32x4 *)(v + e) = anc_f32x4{vv[0], vv[1], vv[2], vv[3]};
+    *(anc_f32x4 *)(p32 + e) = anc_f32x4{pp[0], pp[1], pp[2], pp[3]};
+    *(anc_u32x2 *)(p16 + e) = anc_u32x2{(hb[0] & 0xFFFFu) | (hb[1] << 16), (hb[2] & 0xFFFFu) | (hb[3] << 16)};
+  }
+  if (threadIdx.x == 0) last[row] = t_now;
+}
+
 int check_hyper(const anc_adamw_hyper_t *h, const char *who) {
   ANC_REQUIRE(h != nullptr, "%s: null hyper-parameter block", who);
   ANC_REQUIRE(h->form == ANC_ADAMW_FORM_DIV || h->form == ANC_ADAMW_FORM_IBC,
@@ -257,6 +323,35 @@ extern "C" int anc_adamw_multi(uint64_t desc_table, int32_t n_tensors, int64_t t
     constexpr int f = decltype(F)::value, s = decltype(S)::value;
     hipLaunchKernelGGL((k_adamw_multi<f, s>), dim3((unsigned)total_blocks), dim3(kThreads), 0,
                        anc_stream(stream), tab, (int)n_tensors, hh, c);
+  });
+  ANC_LAUNCH_CHECK();
+  return ANC_OK;
+}
+
+// Row-sparse AdamW on a (V, H) tensor (see k_adamw_rows). rows: n_rows distinct row indices
+// (int32, device) or 0 for "every row, in order" (n_rows = V). grads: (n_rows, H) fp32, row i the
+// gradient of rows[i], or 0 to bring the rows up to date through step t_now without a step.
+// step_table: device array of {bc1, bc2, lr, seed_base} per counted step, entries 1 .. t_now.
+extern "C" int anc_adamw_rows(uint64_t rows, int64_t n_rows, uint64_t grads, uint64_t m, uint64_t v,
+                              uint64_t p32, uint64_t p16, uint64_t last_step, int64_t V, int64_t H,
+                              uint64_t step_table, int32_t t_now, const anc_adamw_hyper_t *h, float wd,
+                              uint32_t seed, uint64_t ctl, uint64_t stream) {
+  if (int rc = check_hyper(h, "anc_adamw_rows")) return rc;
+  ANC_REQUIRE(m && v && p32 && p16 && last_step && step_table, "anc_adamw_rows: null device pointer");
+  ANC_REQUIRE(V > 0 && H > 0 && H % 64 == 0 && n_rows > 0 && n_rows < (1ll << 31) && (rows != 0 || n_rows == V),
+              "anc_adamw_rows: V=%lld, H=%lld (multiple of 64), n_rows=%lld", (long long)V, (long long)H,
+              (long long)n_rows);
+  ANC_REQUIRE(t_now >= 1, "anc_adamw_rows: t_now=%d: steps count from 1", t_now);
+  ANC_REQUIRE(((m | v | p32 | grads | step_table) & 15) == 0 && (p16 & 7) == 0 && ((rows | last_step) & 3) == 0,
+              "anc_adamw_rows: misaligned pointers");
+  const anc_adamw_hyper_t hh = *h;
+  AncProfScope prof(ANC_PROF_ADAMW, anc_stream(stream));
+  dispatch_form_sr(hh.form, hh.sr, [&](auto F, auto S) {
+    constexpr int f = decltype(F)::value, s = decltype(S)::value;
+    hipLaunchKernelGGL((k_adamw_rows<f, s>), dim3((unsigned)n_rows), dim3(kThreads), 0, anc_stream(stream),
+                       (const int32_t *)rows, (const float *)grads, (float *)m, (float *)v, (float *)p32,
+                       (uint16_t *)p16, (int32_t *)last_step, (int)H, V, (const RowStep *)step_table, (int)t_now, hh,
+                       wd, seed, (const anc_step_ctl_t *)ctl);
   });
   ANC_LAUNCH_CHECK();
   return ANC_OK;

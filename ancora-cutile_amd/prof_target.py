@@ -12,6 +12,9 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
     python3 -m ancora_cutile_amd.prof_target dw T K N1[,N2,..] [calls]   weight-gradient GEMM of up to 8
                                       weights (K, Ni) that share the activations, T tokens
 
+    python3 -m ancora_cutile_amd.prof_target embed [V] [H] [TOKENS] [steps]  sorted-scatter embedding
+                                      gradient + row-sparse AdamW step beside the dense AdamW sweep
+                                      of the same table (prints us per call from HIP events)
     python3 -m ancora_cutile_amd.prof_target copy [GiB] [reps]          streaming-kernel shapes
                                       (anc_copy_shape): TB/s of each, the reference points for
                                       the elementwise optimizer kernels
@@ -134,6 +137,50 @@ def main(argv):
         gms, rms = pr["dw_gemm"][0] / calls, pr["dw_reduce"][0] / calls
         print(f"dW of one layer (7 weights, T={T}, 1 segment, 480 workgroups): gemm {gms * 1e3:.1f} us "
               f"({fl / gms / 1e9:.1f} TFLOP/s), finish {rms * 1e3:.1f} us, together {fl / (gms + rms) / 1e9:.1f} TFLOP/s")
+    elif what == "embed":
+        from .adamw import AdamW
+        from .embed import IdGroups, RowSparseAdamW, embed_dw_scatter
+        from .bf16 import bf16_bits
+        V = int(argv[1]) if len(argv) > 1 else 151936
+        H = int(argv[2]) if len(argv) > 2 else 1024
+        T = int(argv[3]) if len(argv) > 3 else 8192
+        steps = int(argv[4]) if len(argv) > 4 else 20
+        rng = np.random.default_rng(0)
+        W = (0.02 * rng.standard_normal((V, H))).astype(np.float32)
+        sparse = RowSparseAdamW(W, sr=True, seed=1)
+        dense = AdamW({"embed": W}, sr=True, seed=1, grad_dtype=np.float32)
+        dy = DevBuf(bf16_bits((1e-2 * rng.standard_normal((T, H))).astype(np.float32)))
+        compact = DevBuf.zeros((T, H), np.float32)
+        gdense = DevBuf.zeros((V, H), np.float32)
+        e = [_lib.Event() for _ in range(4)]
+        t_sc = t_sp = t_de = t_cu = 0.0
+        uniq = 0
+        for it in range(steps + 1):
+            ids = np.minimum((V * rng.random(T) ** 2).astype(np.int32), V - 1)      # skewed token ids
+            grp = IdGroups(ids)
+            e[0].record(0)
+            sparse.catch_up(ids, 0)
+            e[1].record(0)
+            embed_dw_scatter(grp, dy, 0, compact=compact)
+            e[2].record(0)
+            sparse.step(grp.gid, grp.n_groups, compact, 0)
+            e[3].record(0)
+            e[3].sync()
+            if it:                                          # first round warms up
+                t_cu += e[0].elapsed_ms(e[1]); t_sc += e[1].elapsed_ms(e[2]); t_sp += e[2].elapsed_ms(e[3])
+                uniq += grp.n_groups
+            e[0].record(0)
+            dense.launch({"embed": gdense}, 0)
+            e[1].record(0)
+            e[1].sync()
+            if it:
+                t_de += e[0].elapsed_ms(e[1])
+            grp.free()
+        print(f"(V, H) = ({V}, {H}), {T} tokens per step, {uniq / steps:.0f} distinct rows on average, {steps} steps")
+        print(f"  catch-up of the rows the forward gathers  {t_cu / steps * 1e3:8.1f} us (includes the upload of the row list)")
+        print(f"  sorted-scatter gradient rows              {t_sc / steps * 1e3:8.1f} us")
+        print(f"  row-sparse AdamW step                     {t_sp / steps * 1e3:8.1f} us (includes the 16-byte step-table upload)")
+        print(f"  dense AdamW sweep of the same table       {t_de / steps * 1e3:8.1f} us ({28.0 * V * H / (t_de / steps) / 1e9:.2f} TB/s)")
     elif what == "copy":
         gib = float(argv[1]) if len(argv) > 1 else 1.0
         reps = int(argv[2]) if len(argv) > 2 else 5

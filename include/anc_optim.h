@@ -244,6 +244,38 @@ int64_t anc_adamw_num_blocks(int64_t n);   /* blocks one tensor of n elements oc
 int anc_adamw_multi(uint64_t desc_table, int32_t n_tensors, int64_t total_blocks,
                     const anc_adamw_hyper_t *h, uint64_t ctl, uint64_t stream);
 
+/* Row-sparse AdamW on a (V, H) tensor whose gradient touches few rows per step (an input
+ * embedding not tied to the output head), with the results of the dense kernel: ranked "next" in
+ * the survey of the path; the reference has only the dense kernel (ancora/optim/adamw.py:92-97). A
+ * dense step moves rows with zero gradient too (moment decay, bias-corrected momentum, weight
+ * decay), so each row carries the last counted step it is current for (last_step, int32[V], zero
+ * at the start) and the steps it missed are replayed on it, with g = 0 and that step's own
+ * scalars from step_table (device array of {float bc1, bc2, lr; uint32 seed_base} per counted
+ * step, entries 1 .. t_now, bc as in anc_adamw_hyper_t for the chosen form), before anything else
+ * is done to it. m, v, p32 and p16 of a current row are bit-identical to anc_adamw's.
+ *   grads != 0: rows[i]'s gradient is row i of grads, (n_rows, H) fp32: replay through t_now - 1,
+ *               then step t_now (clip scale and skip flag from ctl as in anc_adamw).
+ *   grads == 0: replay through t_now (what the forward must call for the rows it is about to
+ *               gather; with rows == 0 and n_rows == V: every row, e.g. before a checkpoint).
+ * rows: distinct int32 indices on the device. beta1, beta2, omb1, omb2, eps, form and sr are taken
+ * from h; bc1, bc2, lr and seed_base of h are ignored (the table carries them per step). */
+int anc_adamw_rows(uint64_t rows, int64_t n_rows, uint64_t grads, uint64_t m, uint64_t v,
+                   uint64_t p32, uint64_t p16, uint64_t last_step, int64_t V, int64_t H,
+                   uint64_t step_table, int32_t t_now, const anc_adamw_hyper_t *h, float wd,
+                   uint32_t seed, uint64_t ctl, uint64_t stream);
+
+/* Input-embedding weight gradient by deterministic sorted scatter: replaces `_embed_dw_scatter`
+ * (ancora/kernels/fused.py:387-408, launched at ancora/model/resident_moe_model.py:333-334) with
+ * the group arrays of `build_id_groups` (fused.py:411-424): cnt, start, gid (int32[M], groups
+ * padded with cnt = 0) and srt (int32[M], the stable argsort of the token ids). dy: (M, H) bf16.
+ *   out != 0:     out[gid[g]] += sum_r f32(dy[srt[start[g] + r]]), out (V, H) fp32 (the reference)
+ *   compact != 0: compact[g]   = that sum, (M, H) fp32: the gradient rows anc_adamw_rows takes
+ * Rows of a group are added in sorted order starting from zero, one writer per element, no
+ * atomics: bit-identical to the sequential fp32 sum, and from run to run. H % 64 == 0. */
+int anc_embed_dw_scatter(uint64_t cnt, uint64_t start, uint64_t gid, uint64_t srt, uint64_t dy,
+                         uint64_t out, uint64_t compact, int64_t M, int64_t V, int64_t H,
+                         uint64_t stream);
+
 /* p16 = bf16(p32): replaces `_cast_bf16` (ancora/kernels/fused.py:285-290). */
 int anc_cast_bf16(uint64_t p32, uint64_t p16, int64_t n, int sr, uint32_t seed,
                   uint64_t stream);

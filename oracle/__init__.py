@@ -32,6 +32,9 @@ How each function is pinned (see tests/test_oracle_*.py):
                                     (tests/kernels/test_gpu_quant.py:45-47,68)
   gemm_dw                           (gemm_ref.py) the reference's own checker, an fp64 library
                                     matrix product of the bf16 inputs (tests/kernels/test_gemm_bwd.py:40-44)
+  id_groups / embed_dw_rows /       (embed_ref.py) defining properties of the group arrays (permutation,
+  embed_dw_scatter                  stability, counts), an exact integer case, the reference-held gate
+                                    against an fp64 scatter-add (tests/kernels/test_embed_dw_scatter.py:55-61,91)
 No function of the optimizer step is "parity unpinned". quant_mxfp8_w has three edge behaviours
 that no reference-held vector fixes (blocks with amax < 2**-120, bf16 subnormal inputs,
 non-finite inputs): they are parity unpinned and listed in the header of quant_ref.py.
