@@ -8,15 +8,17 @@
 // (`x_row_major`: the A tile is then [tokens][128 columns] and its fragments come from transposing
 // LDS reads, like B's), or x^T (K, T) for a caller that keeps the activations transposed.
 //
-// A single weight is 50-200 tiles, far fewer than the 512 a launch needs to fill 256 CUs, and the
-// backward pass produces one layer's gradients at a time. So the token axis is cut into S
-// segments: segment s of every tile is its own workgroup and leaves an fp32 partial tile in the
-// workspace; a second, HBM-bound kernel adds the S partials in ascending order (and the old dW
-// when accumulating) and can emit the bf16 copy the optimizer step reads. S is the caller's
-// (`segments`: a caller that collects a whole layer's 7 weights into one call fills the CUs with
-// S = 1 and saves the partials' traffic) or, by default, a function of the problem's shape alone;
-// either way the result's bits do not depend on what shares the launch: one workgroup owns one
-// (tile, segment) and its whole K loop, K tiles in ascending order, no atomics.
+// By default one workgroup owns one output tile and runs the whole token axis, tokens in ascending
+// order, one accumulator per element: fixed tiles, no split-K, so a gradient's bits are a function
+// of x and dy alone, whatever shares the call and however the caller groups its calls. A single
+// weight is only 50-200 tiles, far fewer than the 512 a launch needs to fill 256 CUs: a caller
+// fills the GPU by handing over the 7 weights of a layer in one call (480 tiles at Qwen3-0.6B
+// shapes). A caller that cannot do that may opt into cutting the token axis into S segments
+// (`segments` > 1, or -1 for a rule that depends on the problem's shape alone): segment s of every
+// tile is then its own workgroup and leaves an fp32 partial tile in the workspace, and a second,
+// HBM-bound kernel adds the S partials in ascending order (and the old dW when accumulating) and
+// can emit the bf16 copy the optimizer step reads. That split is deterministic, but the bits then
+// depend on S (not on what else is in the call).
 #include "reduce.h"
 #include "ns_common.h"
 
@@ -126,9 +128,11 @@ extern "C" int anc_gemm_dw_multi(const anc_dw_problem_t *probs, int32_t n_probs,
   for (int q = 0; q < n_probs; ++q) {
     const anc_dw_problem_t &b = probs[q];
     if (int rc = check_dw(b, "anc_gemm_dw_multi")) return rc;
-    const int S = b.segments > 0 ? b.segments : dw_segments(b.T, b.K, b.N);
-    ANC_REQUIRE(b.segments >= 0 && S <= 256 && b.T % ((int64_t)S * 32) == 0,
-                "anc_gemm_dw_multi: segments=%d must be 0 (shape rule) or divide T=%lld into multiples of 32 tokens",
+    // 0 or 1: no split of the token axis (the default: fixed tiles, no split-K, bits a function of
+    // the inputs alone); -1: the shape rule; S > 1: S segments
+    const int S = b.segments > 0 ? b.segments : b.segments == 0 ? 1 : dw_segments(b.T, b.K, b.N);
+    ANC_REQUIRE(b.segments >= -1 && S <= 256 && b.T % ((int64_t)S * 32) == 0,
+                "anc_gemm_dw_multi: segments=%d must be 0 or 1 (none), -1 (shape rule) or divide T=%lld into multiples of 32 tokens",
                 (int)b.segments, (long long)b.T);
     // One segment and no grad-norm sums wanted: the GEMM's epilogue finishes the gradient itself
     // (old dW or 0 + product, bf16 copy), no partial tile and no second kernel. Same bits as

@@ -8,10 +8,11 @@ call (`gemm_dW`), the activations are passed as they lie (`x`) or transposed (`x
 that keeps them so), and the call can also leave the bf16 copy of the finished gradient, which is
 what `HybridOptimizer(grad_dtype=np.uint16)` reads.
 
-The token axis is cut into `segments` pieces so that a call fills the GPU (512 workgroups of
-128x256 outputs). By default every problem gets the number of pieces its shape needs to do that
-alone; a caller that hands over the 7 weights of a whole layer in one call passes `segments=1`
-(480 workgroups at Qwen3-0.6B shapes) and saves the partial tiles' traffic.
+By default the token axis is not cut (fixed tiles, no split-K): a gradient's bits do not depend on
+how the caller groups its calls. A call fills the GPU when it carries about 500 tiles of 128x256
+outputs, which the 7 weights of a layer handed over in one call do (480 at Qwen3-0.6B shapes); a
+caller that must launch weight by weight can opt into `segments` (an int, "shape" or "fill"), a
+deterministic split of the token axis whose number of pieces then enters the bits.
 """
 import ctypes
 
@@ -67,10 +68,10 @@ def gemm_dW(problems, si=0, segments=None):
     g16: DevBuf or None; accumulate: bool; gn_partials: int device address or None (where the
     grad-norm partial sums of this gradient go, `StepGuard.partials_ptr`); segments: int, optional}.
     dW (+)= x^T dy for each, 8 per launch. `segments` (argument, or per problem) fixes the number
-    of token segments; None / 0 = the shape rule (a function of T, K, N alone); "fill" = per
-    launch, the largest power of two that keeps the launch within the 512 workgroups the GPU runs
-    at once (so it depends on what shares the call). The result's bits depend on the number of
-    segments and on nothing else. Asynchronous on stream `si`."""
+    of token segments: None / 1 = none (the default); "shape" = the library's rule (a function of
+    T, K, N alone); "fill" = per launch, the largest power of two that keeps the launch within the
+    512 workgroups the GPU runs at once (so it depends on what shares the call). The result's bits
+    depend on the number of segments and on nothing else. Asynchronous on stream `si`."""
     _lib.init()
     runs, cur = [], []
     for p in problems:                       # a native call takes one activation layout
@@ -92,12 +93,15 @@ def gemm_dW(problems, si=0, segments=None):
         arr = (DwProblem * len(group))()
         for k, p in enumerate(group):
             T, K, N = int(p["T"]), int(p["K"]), int(p["N"])
-            S = int(p.get("segments") or fill or (0 if segments == "fill" else segments) or 0)
+            S = p.get("segments") or fill or (None if segments == "fill" else segments) or 1
+            if S == "shape":
+                S = dw_info(T, K, N)[1]
+            S = int(S)
             gn = int(p.get("gn_partials") or 0)
             if S == 1 and gn == 0:                 # finished by the GEMM's epilogue: no partial tiles
                 ws_ptr = ws_bytes = 0
             else:
-                ws = p["workspace"].ensure(S * K * N * 4 if S > 0 else dw_workspace_bytes(T, K, N))
+                ws = p["workspace"].ensure(S * K * N * 4)
                 ws_ptr, ws_bytes = ws.ptr, ws.nbytes
             g16 = p.get("g16")
             x = p.get("x")

@@ -187,19 +187,38 @@ def side_workload(args):
         layers = 28
         per_layer = [p for probs in calls for p in probs]
 
+        side = [_lib.stream_create() for _ in calls] if args.dw_launch == "group" else []
+        main_st = _lib.stream_create() if args.dw_launch == "group" else 0
+        fork, joins = _lib.Event(), [_lib.Event() for _ in calls]
+
         def step():
             for _ in range(layers):
                 if args.dw_launch == "layer":
                     gemm_dW(per_layer, 0, segments=1)
+                elif args.dw_launch == "group":
+                    # one call per group of weights, no token segments (the bits of `layer`); the four
+                    # calls of a layer go to four streams, as a backward pass that keeps its
+                    # weight-gradient GEMMs off the critical path would issue them
+                    fork.record(main_st)
+                    for st, ev, probs in zip(side, joins, calls):
+                        fork.wait_on(st)
+                        gemm_dW(probs, st, segments=1)
+                        ev.record(st)
+                    for ev in joins:
+                        ev.wait_on(main_st)
+                elif args.dw_launch == "group-serial":
+                    for probs in calls:
+                        gemm_dW(probs, 0, segments=1)
                 else:
                     for probs in calls:
-                        gemm_dW(probs, 0, segments="fill" if args.dw_launch == "group-fill" else None)
+                        gemm_dW(probs, 0, segments="fill" if args.dw_launch == "group-fill" else "shape")
         for _ in range(max(1, args.warmup // 2)):
             step()
-        e0.record(0)
+        _lib.api.anc_device_sync()
+        e0.record(main_st)
         for _ in range(args.steps):
             step()
-        e1.record(0)
+        e1.record(main_st)
         e1.sync()
         ms = e0.elapsed_ms(e1) / args.steps
         _lib.profile_enable(True)
@@ -231,7 +250,9 @@ def side_workload(args):
                "config": {"workload": "qwen3-0.6b-weight-gradients", "tokens": T, "weights": 7 * layers,
                           "params": nparams, "launch": args.dw_launch,
                           "launches_per_layer": 1 if args.dw_launch == "layer" else 4,
-                          "token_segments": {"layer": 1, "group": "shape rule", "group-fill": "per launch, <= 512 workgroups"}[args.dw_launch],
+                          "token_segments": {"layer": 1, "group": 1, "group-serial": 1, "group-split": "shape rule",
+                                             "group-fill": "per launch, <= 512 workgroups"}[args.dw_launch],
+                          "streams": 4 if args.dw_launch == "group" else 1,
                           "accumulate": True, "bf16_copy": True,
                           "activations": "x (T,K) as they lie" if args.dw_acts == "x" else "x^T (K,T), transposed by the caller"},
                "roofline": {"bound": "mfma", "achieved": round(gtf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
@@ -302,8 +323,10 @@ def main():
     ap.add_argument("--tokens", type=int, default=8192, help="tokens per micro-batch of --workload dw")
     ap.add_argument("--dw-acts", default="x", choices=("x", "xT"),
                     help="--workload dw: activations as they lie (T,K), or transposed by the caller")
-    ap.add_argument("--dw-launch", default="layer", choices=("layer", "group", "group-fill"),
-                    help="--workload dw: one call per layer (7 weights, 1 token segment) or 4 calls per layer")
+    ap.add_argument("--dw-launch", default="layer", choices=("layer", "group", "group-serial", "group-split", "group-fill"),
+                    help="--workload dw: one call per layer (7 weights); or 4 calls per layer: `group` on four "
+                         "streams, `group-serial` on one, both without token segments (same bits as `layer`); "
+                         "`group-split` / `group-fill` cut the token axis (shape rule / per launch): other bits")
     ap.add_argument("--workload", default="qwen3", choices=("qwen3", "moe", "ns", "adamw", "dw"),
                     help="qwen3: the headline hybrid step (default). moe: the 16-layer MoE family "
                          "(config 4). ns: the 196-matrix Newton-Schulz stress, bf16 and fp32 modes "

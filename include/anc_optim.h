@@ -351,17 +351,21 @@ int anc_transpose_bf16(uint64_t X, uint64_t XT, int64_t E, int64_t M, int64_t N,
  * the producer of the fp32 gradients the optimizer step reads. xT is the activation matrix, either
  * transposed, (K, T) bf16 row-major, or as it lies, x (T, K), with x_row_major = 1; dy is (T, N) bf16; dW (K, N) fp32 is overwritten, or added onto when
  * `accumulate` is set (micro-batch accumulation in place); g16, if not 0, receives the bf16 copy
- * (RNE) of the final dW, the format the step reads. fp32 accumulation in a fixed order: the token
- * axis is cut into S equal pieces, each tile of each piece is one workgroup's whole K loop, and
- * the pieces are added in ascending order, so the bits depend on S but not on what else is in the
- * call. S = `segments` if > 0 (T must be a multiple of 32 S; a call that carries a whole layer's
- * weights fills the GPU with S = 1), else anc_gemm_dw_info's shape rule, which makes a problem
- * fill the GPU by itself. T % 32, K % 128, N % 256 == 0 (the reference: all % 64); pointers
- * 16-byte aligned; workspace of S * K * N * 4 bytes per problem (the partial tiles;
- * anc_gemm_dw_workspace_bytes(T, K, N) for the shape rule), not shared between the problems of a
- * call. g16 16-byte aligned. With S = 1 and gn_partials = 0 the GEMM's epilogue adds onto dW and
- * writes g16 itself: no second kernel runs and no workspace is needed (workspace may be 0); the
- * bits are those of the two-kernel route. */
+ * (RNE) of the final dW, the format the step reads.
+ * Accumulation order. segments = 0 or 1 (the default): one workgroup owns one 128x256 output tile
+ * and runs the whole token axis in ascending order with one fp32 accumulator per element: fixed
+ * tiles, no split-K, the bits of dW are a function of x, dy (and the old dW) alone, independent of
+ * what else is in the call and of how the caller groups its calls; the GEMM's epilogue adds onto
+ * the old dW and writes g16 itself, no workspace is needed (with gn_partials set a second kernel
+ * finishes the gradient and needs workspace K*N*4). A call fills the GPU when it carries about 500
+ * tiles: the 7 weights of a Qwen3-0.6B layer in one call are 480. segments > 1, or -1 for
+ * anc_gemm_dw_info's shape rule (the smallest power of two that gives the problem 256 workgroups
+ * by itself): the token axis is cut into S equal pieces (T a multiple of 32 S), each piece of each
+ * tile is one workgroup's whole K loop leaving an fp32 partial tile, and a second kernel adds the
+ * pieces in ascending order: deterministic, but the bits then DEPEND ON S (and on nothing else);
+ * workspace of S*K*N*4 bytes per problem (anc_gemm_dw_workspace_bytes for the shape rule), not
+ * shared between the problems of a call.
+ * T % 32, K % 128, N % 256 == 0 (the reference: all % 64); pointers and g16 16-byte aligned. */
 typedef struct {
   uint64_t xT, dy, dW, g16, workspace;
   int64_t  T, K, N, workspace_bytes;
@@ -377,7 +381,7 @@ typedef struct {
 } anc_dw_problem_t;
 int64_t anc_gemm_dw_workspace_bytes(int64_t T, int64_t K, int64_t N);
 int anc_gemm_dw_multi(const anc_dw_problem_t *problems, int32_t n_problems, uint64_t stream);
-/* FLOPs of one problem (2 T K N, all executed) and its number of token segments. */
+/* FLOPs of one problem (2 T K N, all executed) and the segment count of the shape rule (segments = -1). */
 int anc_gemm_dw_info(int64_t T, int64_t K, int64_t N, double *flops, int32_t *segments);
 
 /* MXFP8 re-quantisation of bf16 weights (E, K, N) after the step: per block of 32 consecutive K

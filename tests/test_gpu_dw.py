@@ -40,8 +40,9 @@ def _free(p):
 @pytest.mark.parametrize("T,K,N", [(512, 1024, 1024), (256, 1024, 3072), (64, 128, 256), (2048, 128, 256),
                                    (4096, 256, 512), (96, 384, 768)])
 def test_matches_fp64_product(gpu, T, K, N):
-    """The first two shapes are the reference's (test_gemm_bwd.py:49-50); the others reach one and
-    many token segments, a single tile, and a token count that is not a multiple of 64."""
+    """The first two shapes are the reference's (test_gemm_bwd.py:49-50); the others reach a single
+    tile and a token count that is not a multiple of 64. Default: the token axis is not cut; then the
+    opt-in shape rule (one to many token segments) on the same inputs."""
     from ancora_cutile_amd.grads import gemm_dW, dw_info
     x, dy = _inputs(T, K, N, T + K + N)
     p = _problem(x, dy, T, K, N, emit=True) if T % 64 == 0 else None
@@ -58,6 +59,11 @@ def test_matches_fp64_product(gpu, T, K, N):
     assert bits_equal(p["g16"].to_numpy(), bf16_rne_bits(got).reshape(K, N))
     fl, seg = dw_info(T, K, N)
     assert fl == 2.0 * T * K * N and seg >= 1 and T % (32 * seg) == 0
+    gemm_dW([p], segments="shape")
+    split = p["dW"].to_numpy()
+    assert rel_fro(split, want) < 2e-5
+    if seg == 1:
+        assert bits_equal(split, got)
     _free(p)
 
 
