@@ -348,27 +348,24 @@ k_fro_finalize(const double *__restrict__ partials, int nchunks, float eps, floa
   }
 }
 
-// Multiply the bf16 pair of every matrix whose pow2 is not 1 by it; blocks of the others return
-// at once. One block per 4096 elements.
+// Multiply the bf16 pair of every matrix whose pow2 is not 1 by it (exact). One workgroup per
+// matrix: it returns at once unless its matrix is one of the rare tiny ones.
 __global__ void __launch_bounds__(kThreads)
-k_pair_rescale(uint16_t *__restrict__ Uh, uint16_t *__restrict__ Ul, const float *__restrict__ pow2, int blocks_per) {
-  const int e = (int)blockIdx.x / blocks_per;
-  const float sc = pow2[e];
+k_pair_rescale(uint16_t *__restrict__ Uh, uint16_t *__restrict__ Ul, const float *__restrict__ pow2, int64_t mn) {
+  const float sc = pow2[blockIdx.x];
   if (sc == 1.0f) return;
-  const int64_t o = (int64_t)blockIdx.x * 4096 + threadIdx.x * 16;
+  for (int64_t o = (int64_t)threadIdx.x * 8; o < mn; o += (int64_t)kThreads * 8) {
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    uint16_t *p = (h ? Ul : Uh) + o;
-#pragma unroll
-    for (int v = 0; v < 2; ++v) {
-      anc_u32x4 w = *(const anc_u32x4 *)(p + 8 * v);
+    for (int h = 0; h < 2; ++h) {
+      uint16_t *p = (h ? Ul : Uh) + (int64_t)blockIdx.x * mn + o;
+      anc_u32x4 w = *(const anc_u32x4 *)p;
       uint32_t q[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float lo = __uint_as_float(q[i] << 16) * sc, hi = __uint_as_float(q[i] & 0xFFFF0000u) * sc;
         q[i] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xFFFF0000u);
       }
-      *(anc_u32x4 *)(p + 8 * v) = anc_u32x4{q[0], q[1], q[2], q[3]};
+      *(anc_u32x4 *)p = anc_u32x4{q[0], q[1], q[2], q[3]};
     }
   }
 }
@@ -480,7 +477,10 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
     return sp;
   }
   if (mode != ANC_NS_BF16) return sp;
-  sp.gram_hard = N < 2 * M ? 0x6u : 0x4u;       // iterations 1 and 2, or 2 alone
+  // N < 2M: iterations 1 and 2 (3 and 4 carry the terms for every matrix). N >= 3M: iteration 2.
+  // In between nothing: there the outlier-column case meets the bar without (1.6e-3 at 1024x2048)
+  // and the term would buy 6 %.
+  sp.gram_hard = N < 2 * M ? 0x6u : N >= 3 * M ? 0x4u : 0u;
   // The first iterations are insensitive (the singular values are still far below 1, so
   // B X is a small correction to a X); residuals start at a fixed iteration index.
   if (M >= 1024) {
@@ -867,8 +867,8 @@ extern "C" int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partia
   { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)E), dim3(kThreads), 0, s,
                      (const double *)fro_partials, (int)n_partials, eps, pl.recip, pl.pow2); }
   ANC_LAUNCH_CHECK();
-  { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_pair_rescale, dim3((unsigned)(E * (M * N / 4096))), dim3(kThreads), 0, s,
-                     (uint16_t *)Uh, (uint16_t *)Ul, pl.pow2, (int)(M * N / 4096)); }
+  { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_pair_rescale, dim3((unsigned)E), dim3(kThreads), 0, s,
+                     (uint16_t *)Uh, (uint16_t *)Ul, pl.pow2, M * N); }
   ANC_LAUNCH_CHECK();
   ChainProb cp{pl, (const uint16_t *)Uh, (const uint16_t *)Ul, 0, pl.recip, (float *)X32_out, E, M, N};
   return run_bf16_chain(&cp, 1, steps, coef, force_small, s);
@@ -914,8 +914,8 @@ static int pair_multi_impl(const char *who, const anc_ns_problem_t *probs, int32
     { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_fro_finalize, dim3((unsigned)b.E), dim3(kThreads), 0, s,
                        (const double *)b.fro_partials, (int)b.n_partials, eps, pl.recip, pl.pow2); }
     ANC_LAUNCH_CHECK();
-    { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_pair_rescale, dim3((unsigned)(b.E * (b.M * b.N / 4096))), dim3(kThreads), 0, s,
-                       (uint16_t *)b.Uh, (uint16_t *)b.Ul, pl.pow2, (int)(b.M * b.N / 4096)); }
+    { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_pair_rescale, dim3((unsigned)b.E), dim3(kThreads), 0, s,
+                       (uint16_t *)b.Uh, (uint16_t *)b.Ul, pl.pow2, b.M * b.N); }
     ANC_LAUNCH_CHECK();
     cp[q] = ChainProb{pl, (const uint16_t *)b.Uh, (const uint16_t *)b.Ul, 0, pl.recip, (float *)b.X32_out, b.E, b.M, b.N,
                       desc_tables ? (const anc_muon_desc_t *)desc_tables[order[q]] : nullptr};

@@ -425,9 +425,9 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  * Conditioning gate (ANC_NS_BF16 only). After the first A = X X^T the chain measures
  * N * ||offdiag(A)||_F^2 per matrix (1 for independent entries whatever the row scaling; N/r - N/M
  * when the Frobenius mass sits in r directions spread over all rows, e.g. a few outlier columns).
- * A matrix above 2.5 adds the residual of X to A = X X^T in iteration 2 (N >= 2M) or iterations 1
- * and 2 (N < 2M): with 1 % of the columns scaled x100 that is 1.2e-3 / 8e-4 instead of 2.2e-3
- * (1024x3072) / 3.8e-3 (1024x1024). The decision depends on the matrix alone (fixed-order sums),
+ * A matrix above 2.5 adds the residual of X to A = X X^T in iteration 2 (N >= 3M) or iterations 1
+ * and 2 (N < 2M; nothing in between, where the case meets the bar without): with 1 % of the
+ * columns scaled x100 that is 1.2e-3 / 8e-4 instead of 2.2e-3 (1024x3072) / 3.8e-3 (1024x1024). The decision depends on the matrix alone (fixed-order sums),
  * never on the batch. Accuracy bar of ANC_NS_BF16: 2e-3 relative Frobenius on inputs with
  * independent entries, with row or column outliers up to x100; spectra spread over more than two
  * decades (condition number >= 1e2 with a log-uniform spectrum) reach 2.5e-3 .. 4e-3 and need

@@ -298,17 +298,19 @@ def test_outlier_columns_take_the_gate_and_meet_the_bar(gpu, M, N):
     X = np.stack([gauss, cols, rows])
     got = run_ns(X)
     n_hard, extra = _hard_count(3, M, N)
-    assert n_hard == 1 and extra > 0
+    gated = N < 2 * M or N >= 3 * M               # 2M <= N < 3M meets the bar without the extra terms
+    assert (n_hard == 1 and extra > 0) if gated else (n_hard == 0 and extra == 0)
     errs = [rel_fro(got[e], host_ns(X[e], PE_SCHEDULE, 5)) for e in range(3)]
     print(f"({M},{N}) gaussian {errs[0]:.3e}  outlier columns {errs[1]:.3e}  outlier rows {errs[2]:.3e}")
     assert max(errs) < TOL_BF16
     alone = run_ns(X[:1])
     assert _hard_count(1, M, N)[0] == 0
     assert bits_equal(alone[0], got[0])
-    assert bits_equal(run_ns(X[1:2])[0], got[1]) and _hard_count(1, M, N)[0] == 1
+    assert bits_equal(run_ns(X[1:2])[0], got[1]) and _hard_count(1, M, N)[0] == int(gated)
     fast = run_ns(X[1:2], mode="bf16_fast")          # no residual terms, no gate
     assert _hard_count(1, M, N, "bf16_fast") == (0, 0.0)
-    assert rel_fro(fast[0], host_ns(X[1], PE_SCHEDULE, 5)) > errs[1]
+    if gated:
+        assert rel_fro(fast[0], host_ns(X[1], PE_SCHEDULE, 5)) > errs[1]
 
 
 @pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 1536)])
