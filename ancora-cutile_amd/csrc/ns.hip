@@ -694,11 +694,23 @@ extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int m
   return make_plan(0, E, M, N, mode, 64).bytes;
 }
 
+// FLOPs of the output tiles a symmetric M x M product really multiplies, per unit of K: the tiles
+// on or below the diagonal, 256x256 where the 256-tile kernel runs (dims multiples of 256 and the
+// 128-tile kernel not forced), else 128x128. A diagonal tile is multiplied in full, so the count is
+// 10/16 of the dense product at M = 1024 with 256-tiles and 36/64 with 128-tiles; the matrix-
+// instruction counter of the profiler reads exactly this.
+static double sym_tile_flops(int64_t M, int64_t N, bool force_small) {
+  const double ts = (!force_small && M % 256 == 0 && N % 256 == 0) ? 256.0 : 128.0;
+  const double t = (double)M / ts;
+  return t * (t + 1) / 2 * 2.0 * ts * ts;
+}
+
 // Matrix-core work of one chain call: `executed` counts the tiles and terms actually
 // multiplied (symmetric products compute the lower tiles only; residual terms count),
 // `dense` is the textbook steps*(4 M^2 N + 2 M^3) per matrix.
 extern "C" int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
                             double *executed, double *dense) {
+  const bool force_small = (mode & ANC_NS_TILE128) != 0;
   mode &= ~ANC_NS_TILE128;
   if (int rc = check_shape(E, M, N, mode, "anc_ns_flops")) return rc;
   ANC_REQUIRE(executed != nullptr && dense != nullptr && steps >= 0, "anc_ns_flops: bad arguments");
@@ -706,13 +718,13 @@ extern "C" int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode
   *dense = e * steps * (4.0 * m * m * n + 2.0 * m * m * m);
   if (mode == ANC_NS_FP32) { *executed = *dense; return ANC_OK; }
   const SplitPlan sp = split_plan(M, N, mode, steps);
-  const double tM = m / BM, tN = n / BN, tile = 2.0 * BM * BN;
+  const double sym = sym_tile_flops(M, N, force_small);
   double ex = 0.0;
   for (int k = 0; k < steps; ++k) {
     const bool sx = k >= sp.x_from, sfb = k >= sp.fb_from;
-    ex += tM * (tM + 1) / 2 * (sx ? 3 : 1) * tile * n;                   // A = X X^T
-    ex += tM * (tM + 1) / 2 * (sfb ? 3 : 1) * tile * m;                  // B = b A + c A A
-    ex += tM * tN * (1 + (sx ? 1 : 0) + (sfb ? 1 : 0)) * tile * m;       // X = a X + B X
+    ex += sym * (sx ? 3 : 1) * n;                                        // A = X X^T
+    ex += sym * (sfb ? 3 : 1) * m;                                       // B = b A + c A A
+    ex += 2.0 * m * n * (1 + (sx ? 1 : 0) + (sfb ? 1 : 0)) * m;          // X = a X + B X
   }
   *executed = e * ex;
   return ANC_OK;
@@ -720,6 +732,7 @@ extern "C" int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode
 
 extern "C" int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, int mode, int k, int product,
                                     double *executed) {
+  const bool force_small = (mode & ANC_NS_TILE128) != 0;
   mode &= ~ANC_NS_TILE128;
   if (int rc = check_shape(E, M, N, mode, "anc_ns_product_flops")) return rc;
   ANC_REQUIRE(executed != nullptr && steps > 0 && k >= 0 && k < steps && product >= 0 && product <= 2,
@@ -731,11 +744,11 @@ extern "C" int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, 
   }
   const SplitPlan sp = split_plan(M, N, mode, steps);
   const bool sx = k >= sp.x_from, sfb = k >= sp.fb_from;
-  const double tM = m / BM, tN = n / BN, tile = 2.0 * BM * BN;
+  const double sym = sym_tile_flops(M, N, force_small);
   double ex;
-  if (product == 0)      ex = tM * (tM + 1) / 2 * (sx ? 3 : 1) * tile * n;
-  else if (product == 1) ex = tM * (tM + 1) / 2 * (sfb ? 3 : 1) * tile * m;
-  else                   ex = tM * tN * (1 + (sx ? 1 : 0) + (sfb ? 1 : 0)) * tile * m;
+  if (product == 0)      ex = sym * (sx ? 3 : 1) * n;
+  else if (product == 1) ex = sym * (sfb ? 3 : 1) * m;
+  else                   ex = 2.0 * m * n * (1 + (sx ? 1 : 0) + (sfb ? 1 : 0)) * m;
   *executed = (double)E * ex;
   return ANC_OK;
 }
@@ -745,6 +758,7 @@ extern "C" int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, 
 // Synchronises `stream`, then reads the proxy's partial sums back and takes the kernels' decision.
 extern "C" int anc_ns_hard_info(uint64_t workspace, int64_t E, int64_t M, int64_t N, int mode, int steps,
                                 int32_t *n_hard, double *extra_flops_per_matrix, uint64_t stream) {
+  const bool force_small = (mode & ANC_NS_TILE128) != 0;
   mode &= ~ANC_NS_TILE128;
   if (int rc = check_shape(E, M, N, mode, "anc_ns_hard_info")) return rc;
   ANC_REQUIRE(n_hard != nullptr && extra_flops_per_matrix != nullptr && workspace != 0 && steps >= 0,
@@ -757,8 +771,7 @@ extern "C" int anc_ns_hard_info(uint64_t workspace, int64_t E, int64_t M, int64_
   for (int k = 1; k < steps && k < 32; ++k)
     if (k < pl.sp.x_from && ((pl.sp.gram_hard >> k) & 1u)) ++gated_iters;
   if (gated_iters == 0) return ANC_OK;
-  const double tM = (double)M / BM;
-  *extra_flops_per_matrix = gated_iters * 2.0 * (tM * (tM + 1) / 2) * (2.0 * BM * BN) * (double)N;
+  *extra_flops_per_matrix = gated_iters * 2.0 * sym_tile_flops(M, N, force_small) * (double)N;
   std::vector<double> host((size_t)(E * kCondParts));
   ANC_HIP(hipStreamSynchronize(anc_stream(stream)));
   ANC_HIP(hipMemcpy(host.data(), pl.cond, host.size() * sizeof(double), hipMemcpyDeviceToHost));

@@ -425,7 +425,7 @@ def main():
     kind_ms = {k: v[0] / prof_steps for k, v in prof.items() if v[1]}
     launches = {k: v[1] // prof_steps for k, v in prof.items() if v[1]}
 
-    executed = dense = last_bx = 0.0
+    executed = dense = last_bx = lower128 = 0.0
     hard = 0           # matrices that took the extra terms of the conditioning gate in the last step
     for b in opt.muon.engine.batches:
         ex, de = ns_flops(b.E, b.M, b.Nn, 5, "bf16")
@@ -433,6 +433,9 @@ def main():
         executed += ex + nh * extra
         dense += de
         hard += nh
+        ex128, _ = ns_flops(b.E, b.M, b.Nn, 5, "bf16_tile128")    # the same chain counted in 128x128 tiles
+        nh128, extra128 = ns_hard_info(b.ws.buf.ptr, b.E, b.M, b.Nn, 5, "bf16_tile128")
+        lower128 += ex128 + nh128 * extra128
         last_bx += ns_product_flops(b.E, b.M, b.Nn, 4, 2, 5, "bf16")
     # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
     # last X = a X + B X) also reads and writes the weights
@@ -495,6 +498,11 @@ def main():
                                                      "avg_launch_ms": round(pure_ms / max(1, pure_launches), 4)},
                      "avg_launch_ms": round(gemm_ms / max(1, gemm_launches), 4),
                      "executed_tflop_per_step": round(executed / 1e12, 3),
+                     "executed_counts": "what the kernels multiply: residual and gated terms, and of the symmetric "
+                                        "products the 256x256 tiles on or below the diagonal, each in full "
+                                        "(= the profiler's matrix-instruction count)",
+                     "lower_triangle_128_tflop_per_step": round(lower128 / 1e12, 3),
+                     "frac_on_lower_triangle_128": round(lower128 / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4) if gemm_ms else 0.0,
                      "dense_tflop_per_step": round(dense / 1e12, 3)},
         "adamw_hbm": {"bound": "hbm", "achieved": round(adamw_gbps, 1), "peak": PEAK_HBM_GBPS,
                       "unit": "GB/s", "frac": round(adamw_gbps / PEAK_HBM_GBPS, 4),

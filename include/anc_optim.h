@@ -498,8 +498,12 @@ int anc_muon_ns_update_multi(const anc_ns_problem_t *problems, int32_t n_problem
                              uint32_t seed_base, uint64_t ctl, uint64_t stream);
 
 /* Matrix-core FLOPs of one anc_ns_batched call: `executed` counts the tiles and terms the
- * kernels really multiply (lower-triangle tiles of the symmetric products, residual terms),
- * `dense` is steps*(4 M^2 N + 2 M^3) per matrix. Roofline figures use `executed`. */
+ * kernels really multiply (residual terms; of the symmetric products the tiles on or below the
+ * diagonal, each in full: 256x256 tiles where dims are multiples of 256, i.e. 10/16 of the dense
+ * product at M = 1024, else, or with ANC_NS_TILE128 in `mode`, 128x128 tiles, 36/64; the
+ * profiler's matrix-instruction counter reads this number), `dense` is steps*(4 M^2 N + 2 M^3)
+ * per matrix. Roofline figures use `executed`; matrices that take the conditioning gate add
+ * anc_ns_hard_info's extra work. */
 int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
                  double *executed, double *dense);
 /* Of the E matrices of the last chain call that used `workspace`: how many took the extra

@@ -127,3 +127,23 @@ def test_bf16_host_helpers_match_oracle():
     x = np.random.default_rng(0).standard_normal(1000).astype(np.float32)
     assert np.array_equal(bf16_bits(x), bf16_rne_bits(x))
     assert np.array_equal(bits_f32(bf16_bits(x)), bits_to_f32(bf16_rne_bits(x)))
+
+
+def test_flop_accounting_matches_the_tiles_the_kernels_multiply():
+    """Host arithmetic only. (1024, 3072), 5 steps, no residual terms: per step the symmetric
+    products multiply 10 lower 256x256 tiles (36 lower 128x128 tiles on the small-tile kernel) over
+    K = N and K = M, the third product all of 2 M^2 N."""
+    from ancora_cutile_amd.muon_ns import ns_flops, ns_product_flops
+    M, N, E = 1024, 3072, 3
+    ex, de = ns_flops(E, M, N, 5, "bf16_fast")
+    assert de == E * 5 * (4.0 * M * M * N + 2.0 * M ** 3)
+    assert ex == E * 5 * (10 * 2 * 256 * 256 * (N + M) + 2.0 * M * M * N)
+    ex128, _ = ns_flops(E, M, N, 5, "bf16_fast_tile128")
+    assert ex128 == E * 5 * (36 * 2 * 128 * 128 * (N + M) + 2.0 * M * M * N)
+    assert ns_flops(E, 384, 768, 5, "bf16_fast")[0] == E * 5 * (6 * 2 * 128 * 128 * (768 + 384) + 2.0 * 384 * 384 * 768)
+    assert sum(ns_product_flops(E, M, N, k, p, 5, "bf16_fast") for k in range(5) for p in range(3)) == ex
+    # 1024 x 1024: iterations 3 and 4 carry the residual of X (3 terms in A = X X^T, 2 in X = a X + B X)
+    ex_sq, _ = ns_flops(1, M, M, 5, "bf16")
+    sym = 10 * 2 * 256 * 256 * M
+    assert ex_sq == 3 * (2 * sym + 2.0 * M ** 3) + 2 * (3 * sym + sym + 2 * 2.0 * M ** 3)
+    assert ns_flops(1, M, M, 5, "fp32")[0] == ns_flops(1, M, M, 5, "fp32")[1]
