@@ -12,7 +12,7 @@ from .muon_ns import (newton_schulz_resident, newton_schulz_resident_e, ns_fp32_
                       set_polar_express, PE_SCHEDULE, A_COEF, B_COEF, C_COEF, NTM, NTN, NTK)
 from .muon import (Muon, DeviceMuon, MuonScratch, ResidentMuon, BatchedProjMuon,  # noqa: F401
                    newton_schulz5)
-from .moe import ExpertMuonScratch, ExpertOptimizer                          # noqa: F401
+from .moe import ExpertMuonScratch, ExpertOptimizer, GroupedMoEFFNOptim                          # noqa: F401
 from .hybrid import HybridOptimizer, default_is_muon, resident_is_muon       # noqa: F401
 from .quant import Mxfp8WeightCache, quant_mxfp8_w                          # noqa: F401
 from .grads import gemm_dW, transpose_acts, DwWorkspace                       # noqa: F401

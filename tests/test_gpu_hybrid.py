@@ -298,3 +298,79 @@ def test_fused_update_equals_separate_update_kernel(gpu, sr):
         for k in ("buf", "p32", "p16", "G"):
             if w[k] is not None:
                 w[k].free()
+
+
+class _StubMoELayer:
+    """What `GroupedMoEFFN` carries when its optimizer methods run: masters in `w`, packed bf16
+    forward weights and their transposes, fp32 gradient buffers, router buffers."""
+
+    def __init__(self, E, H, rng, optimizer, device_route):
+        from ancora_cutile_amd import DevBuf
+        from ancora_cutile_amd.bf16 import bf16_bits
+        self.E, self.H, self.Ie, self.optimizer, self.device_route = E, H, H, optimizer, device_route
+        self.w = {k: (0.02 * rng.standard_normal((E, H, H))).astype(np.float32)
+                  for k in ("gate_proj", "up_proj", "down_proj")}
+        self.w["router"] = (0.02 * rng.standard_normal((H, E))).astype(np.float32)
+        for attr, key in (("Wg", "gate_proj"), ("Wu", "up_proj"), ("Wd", "down_proj")):
+            setattr(self, attr, DevBuf(bf16_bits(self.w[key]).reshape(E * H, H)))
+            setattr(self, attr + "T", DevBuf.zeros((E * H, H), np.uint16))
+            setattr(self, "d" + attr, DevBuf.zeros((E * H, H), np.float32))
+        self.Wr_dev = DevBuf(self.w["router"].reshape(-1))
+        self.G_router_dev = DevBuf.zeros((H * E,), np.float32)
+        self.Gr_acc = DevBuf.zeros((H * E,), np.float32)
+        self.G_router = np.zeros((H, E), np.float32)
+        self._muon_lr = 0.02
+
+
+@pytest.mark.parametrize("optimizer", ["muon", "adamw"])
+@pytest.mark.parametrize("device_route", [True, False])
+def test_grouped_moe_ffn_optimizer_methods(gpu, optimizer, device_route):
+    """`init_adamw` / `step` under the reference's names (ancora/kernels/moe.py:525-609) on a layer
+    object's own buffers: experts bit-equal to `ExpertOptimizer` on the same data, the bf16 forward
+    weights updated in place, their transposes refreshed, the router against the oracle."""
+    from ancora_cutile_amd import DevBuf, GroupedMoEFFNOptim, ExpertOptimizer
+    from oracle.adamw_ref import adamw_step_ibc
+
+    class Layer(_StubMoELayer, GroupedMoEFFNOptim):
+        pass
+
+    E, H = 4, 256
+    rng = np.random.default_rng(21)
+    layer = Layer(E, H, rng, optimizer, device_route)
+    layer.init_adamw(0, betas=(0.9, 0.999), eps=1e-8, wd=0.01)
+    ref = ExpertOptimizer({k: layer.w[k] for k in ExpertOptimizer.NAMES}, router=None, optimizer=optimizer,
+                          betas=(0.9, 0.999), eps=1e-8, wd=0.01)
+    router0 = layer.w["router"].copy()
+    rm = np.zeros_like(router0); rv = np.zeros_like(router0); rw = router0.copy()
+    names = (("Wg", "gate_proj"), ("Wu", "up_proj"), ("Wd", "down_proj"))
+    for t in (1, 2):
+        g = {key: (1e-2 * rng.standard_normal((E * H, H))).astype(np.float32) for _, key in names}
+        gr = (1e-2 * rng.standard_normal((H, E))).astype(np.float32)
+        gdev = {}
+        for attr, key in names:
+            getattr(layer, "d" + attr).upload(g[key])
+            gdev[key] = DevBuf(g[key])
+        layer.Gr_acc.upload(gr.reshape(-1))
+        layer.G_router = gr
+        layer.step(0, lr=1e-3)
+        ref.step(gdev, 0, lr=1e-3, muon_lr=0.02)
+        gpu.stream_sync(0)
+        assert layer._wq_dirty_mx and layer._t == t
+        rw, rm, rv = adamw_step_ibc(rw, rm, rv, gr, 1e-3, 0.9, 0.999, 1e-8, 0.0 if device_route else 0.01,
+                                    1.0 / (1.0 - 0.9 ** t), 1.0 / (1.0 - 0.999 ** t))
+        for b in gdev.values():
+            b.free()
+    state = layer._muon if optimizer == "muon" else layer._eopt
+    for attr, key in names:
+        want = ref.st[key]
+        assert bits_equal(state[attr]["p32"].to_numpy().ravel(), want["p32"].to_numpy().ravel()), attr
+        p16 = getattr(layer, attr).to_numpy()
+        assert bits_equal(p16.ravel(), want["p16"].to_numpy().ravel()), attr          # forward weights, in place
+        p16T = getattr(layer, attr + "T").to_numpy().reshape(E, H, H)
+        assert all(bits_equal(p16T[e], np.ascontiguousarray(p16.reshape(E, H, H)[e].T)) for e in range(E)), attr
+    if device_route:
+        assert max_ulp(layer.Wr_dev.to_numpy().reshape(H, E), rw) <= 1
+        assert bits_equal(layer.G_router_dev.to_numpy(), layer.Gr_acc.to_numpy())
+    else:
+        assert np.abs(layer.w["router"] - rw).max() < 1e-7
+    layer.free_optim(); ref.free()
