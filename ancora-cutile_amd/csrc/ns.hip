@@ -434,8 +434,6 @@ __global__ void __launch_bounds__(kThreads) k_ns_cond(NsCondArgs a) {
     a.out[q][b] = t;
   }
 }
-// A matrix is "hard" when N * ||offdiag(A0)||_F^2 exceeds this (1.0 for independent entries).
-constexpr double kCondTau = 2.5;
 
 // ------------------------------------------------------------------------- workspace
 struct Carve {
@@ -457,19 +455,36 @@ struct Carve {
 //   X, F, B in last three 1024x1024 7e-5                                          256x256 3e-4
 // The plan depends on (M, N, steps) only, never on the batch.
 struct SplitPlan {
-  int x_from;    // first iteration whose A and B X products add the residual of X
+  int x_from;    // first iteration whose A and B X products add the residual of X for every matrix
   int fb_from;   // first iteration whose A A and B X products add the residuals of F and Boff
-  unsigned gram_hard;   // bit k: in iteration k (< x_from) the A = X X^T product of a hard matrix
-                        // adds the residual of X
+  // Conditioning gates. In iteration k < x_from with gate_tau[k] > 0, a matrix whose proxy
+  // N * ||offdiag(A0)||_F^2 exceeds gate_tau[k] adds the residual of X to A = X X^T and, with bit k
+  // of gate_bx set, to X = a X + B X as well.
+  static constexpr int kGateIters = 8;
+  float gate_tau[kGateIters];
+  unsigned gate_bx;
+  bool gated(int k) const { return k >= 0 && k < kGateIters && k < x_from && gate_tau[k] > 0.0f; }
+  bool any_gate(int steps) const {
+    for (int k = 0; k < steps; ++k) if (gated(k)) return true;
+    return false;
+  }
 };
-// Hard matrices: inputs whose Frobenius mass sits in a few directions spread over all rows (a
-// gradient with a few outlier columns: the transposed iterate of a tall weight with outlier
-// rows). Rounding X to bf16 then costs the small directions their signal in A = X X^T while the
-// large ones converge: 1% of the columns x100 gives 2.2e-3 at 1024x3072 and 3.8e-3 at 1024x1024
-// without the terms below, 1.2e-3 and 8e-4 with them. Row outliers, whose mass lands on the exact
-// fp32 diagonal of A, need nothing (5e-4 .. 7e-4).
+// The proxy is 1.0 for a matrix with independent entries whatever its row scaling (1.2 with 1 %
+// of the rows x100), 1.7 for columns scaled over 0.1..3, about 100 with 1 % of the columns x100.
+//   kTauHard: inputs whose Frobenius mass sits in a few directions spread over all rows (a
+//     gradient with a few outlier columns: the transposed iterate of a tall weight with outlier
+//     rows). Rounding X to bf16 then costs the small directions their signal in A = X X^T while the
+//     large ones converge: 1% of the columns x100 gives 2.2e-3 at 1024x3072 and 3.8e-3 at
+//     1024x1024 without the extra terms of iterations 1-2, 1.2e-3 and 8e-4 with them. Row outliers,
+//     whose mass lands on the exact fp32 diagonal of A, need nothing (5e-4 .. 7e-4).
+//   kTauPlain: N < 2M runs the residual of X in both X-products of the last two iterations; a
+//     matrix with independent entries needs them in the last one only (1.66e-3 against 1.41e-3 at
+//     1024x1024, 5.3e-4 either way with outlier rows), the column-scaled case needs both (1.85e-3
+//     against 2.09e-3). So the first of the two is gated low.
+constexpr float kTauHard = 2.5f, kTauPlain = 1.3f;
 SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
-  SplitPlan sp{steps, steps, 0u};
+  SplitPlan sp{};
+  sp.x_from = sp.fb_from = steps;
   if (mode == ANC_NS_BF16_X3) {
     // every product with the residuals of both operands' bf16 roundings, in every iteration:
     // about 1e-5 on every input tried, three times the matrix-core work
@@ -477,16 +492,25 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
     return sp;
   }
   if (mode != ANC_NS_BF16) return sp;
-  // N < 2M: iterations 1 and 2 (3 and 4 carry the terms for every matrix). N >= 3M: iteration 2.
-  // In between nothing: there the outlier-column case meets the bar without (1.6e-3 at 1024x2048)
-  // and the term would buy 6 %.
-  sp.gram_hard = N < 2 * M ? 0x6u : N >= 3 * M ? 0x4u : 0u;
   // The first iterations are insensitive (the singular values are still far below 1, so
   // B X is a small correction to a X); residuals start at a fixed iteration index.
   if (M >= 1024) {
-    if (N < 2 * M) sp.x_from = steps - 2 < 3 ? steps - 2 : 3;
+    if (N < 2 * M) {
+      sp.x_from = steps - 2 < 3 ? steps - 2 : 3;
+      sp.gate_tau[1] = sp.gate_tau[2] = kTauHard;
+      if (steps == 5) {                       // the schedule the low gate was measured on
+        sp.gate_tau[3] = kTauPlain;
+        sp.gate_bx = 1u << 3;
+        sp.x_from = 4;
+      }
+    } else if (N >= 3 * M) {
+      // iteration 2 alone. In between (2M <= N < 3M) nothing: there the outlier-column case meets
+      // the bar without (1.6e-3 at 1024x2048) and the term would buy 6 %.
+      sp.gate_tau[2] = kTauHard;
+    }
   } else {
     sp.x_from = sp.fb_from = steps - 3 < 2 ? steps - 3 : 2;
+    sp.gate_tau[1] = kTauHard;
   }
   if (sp.x_from < 0) sp.x_from = 0;
   if (sp.fb_from < 0) sp.fb_from = 0;
@@ -583,13 +607,10 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
   int64_t Es[kMaxGroups];
   for (int q = 0; q < n; ++q) { curH[q] = cp[q].inH; curL[q] = cp[q].inL; nxt[q] = cp[q].nxt; Es[q] = cp[q].E; }
   bool want_cond = false;      // some later iteration gates a product on the proxy
-  for (int q = 0; q < n; ++q)
-    for (int k = 1; k < steps && k < 32; ++k)
-      if (k < cp[q].pl.sp.x_from && ((cp[q].pl.sp.gram_hard >> k) & 1u)) want_cond = true;
+  for (int q = 0; q < n; ++q) want_cond = want_cond || cp[q].pl.sp.any_gate(steps);
   for (int k = 0; k < steps; ++k) {
     const bool last = k + 1 == steps;
     NsGemm ga[kMaxGroups], gb[kMaxGroups], gx[kMaxGroups];
-    bool any_gated = false;
     for (int q = 0; q < n; ++q) {
       const Plan &pl = cp[q].pl;
       const int64_t M = cp[q].M, N = cp[q].N, mn = M * N;
@@ -607,7 +628,7 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       // A = X X^T
       ga[q] = g;
       ga[q].A[0] = curH[q]; ga[q].B[0] = curH[q]; ga[q].nterms = 1;
-      const bool gated = !split && k < 32 && ((pl.sp.gram_hard >> k) & 1u);
+      const bool gated = pl.sp.gated(k);           // implies !split
       if (split || gated) {
         ga[q].A[1] = curH[q]; ga[q].B[1] = curL[q];
         ga[q].A[2] = curL[q]; ga[q].B[2] = curH[q];
@@ -615,9 +636,8 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       }
       if (gated) {
         ga[q].cond = pl.cond;
-        ga[q].cond_thresh = kCondTau / (double)N;
+        ga[q].cond_thresh = (double)pl.sp.gate_tau[k] / (double)N;
         ga[q].nterms_hard = 3;
-        any_gated = true;
       }
       ga[q].K = (int)N; ga[q].strideA = mn; ga[q].strideB = mn; ga[q].tiles_m = tM; ga[q].tiles_n = tM; ga[q].lower = 1;
       // B = b A + c A A
@@ -633,6 +653,12 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       gx[q] = g;
       gx[q].A[0] = pl.Bh; gx[q].B[0] = curH[q]; gx[q].nterms = 1;
       if (split) { gx[q].A[gx[q].nterms] = pl.Bh; gx[q].B[gx[q].nterms] = curL[q]; ++gx[q].nterms; }
+      if (gated && ((pl.sp.gate_bx >> k) & 1u) && !split_fb) {
+        gx[q].A[1] = pl.Bh; gx[q].B[1] = curL[q];
+        gx[q].cond = pl.cond;
+        gx[q].cond_thresh = (double)pl.sp.gate_tau[k] / (double)N;
+        gx[q].nterms_hard = 2;
+      }
       if (split_fb) { gx[q].A[gx[q].nterms] = pl.Bl; gx[q].B[gx[q].nterms] = curH[q]; ++gx[q].nterms; }
       gx[q].K = (int)M; gx[q].strideA = M * M; gx[q].strideB = mn; gx[q].tiles_m = tM; gx[q].tiles_n = tN; gx[q].lower = 0;
       gx[q].Xh = curH[q]; gx[q].Xl = curL[q];
@@ -654,7 +680,7 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       NsCondArgs ca{};
       int blocks = 0;
       for (int q = 0; q < n; ++q) {
-        if (cp[q].pl.sp.gram_hard == 0u) continue;
+        if (!cp[q].pl.sp.any_gate(steps)) continue;
         ca.Fh[ca.n] = cp[q].pl.Fh; ca.out[ca.n] = cp[q].pl.cond; ca.M[ca.n] = (int)cp[q].M;
         ca.blocks[ca.n] = (int)(cp[q].E * kCondParts);
         blocks += ca.blocks[ca.n];
@@ -664,7 +690,6 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       hipLaunchKernelGGL(k_ns_cond, dim3((unsigned)blocks), dim3(kThreads), 0, s, ca);
       ANC_LAUNCH_CHECK();
     }
-    (void)any_gated;
     {
       AncProfScope prof(ANC_PROF_NS_BMAT, s);
       if (big) { if (int rc = anc_ns_gemm_big_multi(EPI_BMAT, gb, Es, n, s)) return rc; }
@@ -753,33 +778,36 @@ extern "C" int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, 
   return ANC_OK;
 }
 
-// How many matrices of the last chain call on this workspace took the extra terms of the
-// conditioning gate, and the matrix-core work one such matrix adds to anc_ns_flops' `executed`.
-// Synchronises `stream`, then reads the proxy's partial sums back and takes the kernels' decision.
+// Of the last chain call on this workspace: how many matrices took extra terms through a
+// conditioning gate, and the matrix-core work all of them together add to anc_ns_flops' `executed`.
+// Synchronises `stream`, then reads the proxy's partial sums back and takes the kernels' decisions.
 extern "C" int anc_ns_hard_info(uint64_t workspace, int64_t E, int64_t M, int64_t N, int mode, int steps,
-                                int32_t *n_hard, double *extra_flops_per_matrix, uint64_t stream) {
+                                int32_t *n_gated, double *extra_flops, uint64_t stream) {
   const bool force_small = (mode & ANC_NS_TILE128) != 0;
   mode &= ~ANC_NS_TILE128;
   if (int rc = check_shape(E, M, N, mode, "anc_ns_hard_info")) return rc;
-  ANC_REQUIRE(n_hard != nullptr && extra_flops_per_matrix != nullptr && workspace != 0 && steps >= 0,
+  ANC_REQUIRE(n_gated != nullptr && extra_flops != nullptr && workspace != 0 && steps >= 0,
               "anc_ns_hard_info: bad arguments");
-  *n_hard = 0;
-  *extra_flops_per_matrix = 0.0;
+  *n_gated = 0;
+  *extra_flops = 0.0;
   if (mode == ANC_NS_FP32) return ANC_OK;
   const Plan pl = make_plan(workspace, E, M, N, mode, steps);
-  int gated_iters = 0;
-  for (int k = 1; k < steps && k < 32; ++k)
-    if (k < pl.sp.x_from && ((pl.sp.gram_hard >> k) & 1u)) ++gated_iters;
-  if (gated_iters == 0) return ANC_OK;
-  *extra_flops_per_matrix = gated_iters * 2.0 * sym_tile_flops(M, N, force_small) * (double)N;
+  if (!pl.sp.any_gate(steps)) return ANC_OK;
   std::vector<double> host((size_t)(E * kCondParts));
   ANC_HIP(hipStreamSynchronize(anc_stream(stream)));
   ANC_HIP(hipMemcpy(host.data(), pl.cond, host.size() * sizeof(double), hipMemcpyDeviceToHost));
-  const double thresh = kCondTau / (double)N;
+  const double gram_extra = 2.0 * sym_tile_flops(M, N, force_small) * (double)N;     // two more terms
+  const double bx_extra = 2.0 * (double)M * (double)M * (double)N;                   // one more term
   for (int64_t e = 0; e < E; ++e) {
     double t = host[(size_t)(e * kCondParts)];
     for (int i = 1; i < kCondParts; ++i) t = t + host[(size_t)(e * kCondParts + i)];
-    if (t > thresh) ++*n_hard;
+    bool any = false;
+    for (int k = 0; k < steps; ++k) {
+      if (!pl.sp.gated(k) || !(t > (double)pl.sp.gate_tau[k] / (double)N)) continue;
+      any = true;
+      *extra_flops += gram_extra + (((pl.sp.gate_bx >> k) & 1u) ? bx_extra : 0.0);
+    }
+    if (any) ++*n_gated;
   }
   return ANC_OK;
 }

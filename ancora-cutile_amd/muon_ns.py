@@ -114,9 +114,9 @@ def ns_flops(E, M, N, steps=5, mode="bf16"):
 
 
 def ns_hard_info(workspace_ptr, E, M, N, steps=5, mode="bf16", si=0):
-    """(n_hard, extra_flops_per_matrix) of the last chain call that used this workspace: how many
-    of its E matrices took the extra terms of the conditioning gate, and the matrix-core work
-    each adds to `ns_flops`' executed count. Synchronises stream `si`."""
+    """(n_gated, extra_flops) of the last chain call that used this workspace: how many of its E
+    matrices took extra terms through a conditioning gate, and the matrix-core work they add,
+    all together, to `ns_flops`' executed count. Synchronises stream `si`."""
     n, ex = ctypes.c_int32(0), ctypes.c_double(0)
     api.anc_ns_hard_info(int(workspace_ptr), int(E), int(M), int(N), MODES[mode], int(steps),
                          ctypes.byref(n), ctypes.byref(ex), int(si))

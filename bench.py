@@ -430,12 +430,12 @@ def main():
     for b in opt.muon.engine.batches:
         ex, de = ns_flops(b.E, b.M, b.Nn, 5, "bf16")
         nh, extra = ns_hard_info(b.ws.buf.ptr, b.E, b.M, b.Nn, 5, "bf16")
-        executed += ex + nh * extra
+        executed += ex + extra
         dense += de
         hard += nh
         ex128, _ = ns_flops(b.E, b.M, b.Nn, 5, "bf16_tile128")    # the same chain counted in 128x128 tiles
         nh128, extra128 = ns_hard_info(b.ws.buf.ptr, b.E, b.M, b.Nn, 5, "bf16_tile128")
-        lower128 += ex128 + nh128 * extra128
+        lower128 += ex128 + extra128
         last_bx += ns_product_flops(b.E, b.M, b.Nn, 4, 2, 5, "bf16")
     # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
     # last X = a X + B X) also reads and writes the weights

@@ -422,16 +422,25 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *                     times the matrix-core work of ANC_NS_BF16_FAST.
  *   ANC_NS_FP32       every product in fp32 (validation mode).
  *
- * Conditioning gate (ANC_NS_BF16 only). After the first A = X X^T the chain measures
- * N * ||offdiag(A)||_F^2 per matrix (1 for independent entries whatever the row scaling; N/r - N/M
- * when the Frobenius mass sits in r directions spread over all rows, e.g. a few outlier columns).
- * A matrix above 2.5 adds the residual of X to A = X X^T in iteration 2 (N >= 3M) or iterations 1
- * and 2 (N < 2M; nothing in between, where the case meets the bar without): with 1 % of the
- * columns scaled x100 that is 1.2e-3 / 8e-4 instead of 2.2e-3 (1024x3072) / 3.8e-3 (1024x1024). The decision depends on the matrix alone (fixed-order sums),
- * never on the batch. Accuracy bar of ANC_NS_BF16: 2e-3 relative Frobenius on inputs with
- * independent entries, with row or column outliers up to x100; spectra spread over more than two
- * decades (condition number >= 1e2 with a log-uniform spectrum) reach 2.5e-3 .. 4e-3 and need
- * ANC_NS_BF16_X3.
+ * Conditioning gates (ANC_NS_BF16 only). After the first A = X X^T the chain measures
+ * N * ||offdiag(A)||_F^2 per matrix: 1.0 for independent entries whatever the row scaling (1.2 with
+ * 1 % of the rows x100), 1.7 for columns scaled over 0.1..3, N/r - N/M when the Frobenius mass sits in
+ * r directions spread over all rows (about 100 with 1 % of the columns x100). Later products of a
+ * matrix add the residual of X (three accumulation terms in A = X X^T, two in X = a X + B X)
+ * according to it:
+ *   N >= 3M:  above 2.5, A = X X^T of iteration 2 (1 % of the columns x100 at 1024x3072: 1.15e-3
+ *             instead of 2.2e-3);
+ *   N < 2M:   above 2.5, A = X X^T of iterations 1 and 2 (1024x1024: 8e-4 instead of 3.8e-3); above
+ *             1.3, both X-products of iteration 3 (5-step chains; every matrix has them in
+ *             iteration 4): a matrix with independent entries or outlier rows does without
+ *             (1.66e-3 / 5e-4 at 1024x1024), the column-scaled case needs them (1.85e-3);
+ *   2M <= N < 3M: no gate (1.6e-3 on the outlier-column case as it is).
+ * The decision depends on the matrix alone (fixed-order sums), never on the batch. Accuracy bar of
+ * ANC_NS_BF16 with the Polar-Express schedule: 2e-3 relative Frobenius on inputs with independent
+ * entries, with row or column outliers up to x100 on 1 % of the rows or columns, with columns
+ * scaled over a factor 30; spectra spread over two decades or more (condition number >= 1e2 with
+ * a log-uniform spectrum) reach 2.5e-3 .. 4e-3 and need ANC_NS_BF16_X3. Keller coefficients
+ * amplify operand rounding about twice as much (4.5e-3 at 1024x1024).
  *
  * M and N must be multiples of 128 (the reference's tile alignment,
  * ancora/optim/muon.py:98). workspace must hold anc_ns_workspace_bytes(E,M,N,mode)
@@ -506,11 +515,11 @@ int anc_muon_ns_update_multi(const anc_ns_problem_t *problems, int32_t n_problem
  * anc_ns_hard_info's extra work. */
 int anc_ns_flops(int64_t E, int64_t M, int64_t N, int steps, int mode,
                  double *executed, double *dense);
-/* Of the E matrices of the last chain call that used `workspace`: how many took the extra
- * terms of the conditioning gate, and the matrix-core work each of them adds to anc_ns_flops'
- * `executed`. Synchronises `stream` and reads 64 bytes per matrix back. */
+/* Of the E matrices of the last chain call that used `workspace`: how many took extra terms
+ * through a conditioning gate, and the matrix-core work they add, all together, to
+ * anc_ns_flops' `executed`. Synchronises `stream` and reads 64 bytes per matrix back. */
 int anc_ns_hard_info(uint64_t workspace, int64_t E, int64_t M, int64_t N, int mode, int steps,
-                     int32_t *n_hard, double *extra_flops_per_matrix, uint64_t stream);
+                     int32_t *n_gated, double *extra_flops, uint64_t stream);
 /* Executed matrix-core work of one product of one iteration of that chain: iteration k in
  * 0..steps-1, product 0 (A = X X^T), 1 (B = b A + c A A) or 2 (X = a X + B X). */
 int anc_ns_product_flops(int64_t E, int64_t M, int64_t N, int steps, int mode, int k, int product,

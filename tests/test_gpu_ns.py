@@ -45,8 +45,8 @@ def test_bf16_mode_within_2e3(gpu, M, N, sched):
     X = rng.standard_normal((2, M, N)).astype(np.float32)
     got = run_ns(X, schedule=schedule, mode="bf16")
     # Keller's quintic amplifies operand rounding about twice as much as the Polar-Express schedule
-    # every BASELINE configuration uses: default mode held to 5e-3, the bar itself in bf16_x3 below
-    tol = TOL_BF16 if sched == "pe" else 5e-3
+    # every BASELINE configuration uses: default mode held to 5.5e-3, the bar itself in bf16_x3 below
+    tol = TOL_BF16 if sched == "pe" else 5.5e-3
     for e in range(2):
         assert rel_fro(got[e], host_ns(X[e], schedule, 5)) < tol
     if sched == "keller" and M in (256, 1024):
@@ -72,6 +72,9 @@ def test_reference_probe_inputs(gpu):
         err = rel_fro(pe, host_ns(X, PE_SCHEDULE, 5))
         print(f"probe input {X.shape}: Polar-Express chain {err:.3e}")
         assert err < TOL_BF16
+        # the column-scaled square input sits above the low gate and keeps the residual terms of
+        # iteration 3; a Gaussian one does without (test_bf16_mode_within_2e3 holds it to the bar)
+        assert _hard_count(1, *X.shape)[0] == (1 if X.shape == (1024, 1024) else 0)
 
 
 def test_polar_express_orthogonalises_better_than_keller(gpu):
