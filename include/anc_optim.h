@@ -245,8 +245,8 @@ int anc_adamw_multi(uint64_t desc_table, int32_t n_tensors, int64_t total_blocks
                     const anc_adamw_hyper_t *h, uint64_t ctl, uint64_t stream);
 
 /* Row-sparse AdamW on a (V, H) tensor whose gradient touches few rows per step (an input
- * embedding not tied to the output head), with the results of the dense kernel: ranked "next" in
- * the survey of the path; the reference has only the dense kernel (ancora/optim/adamw.py:92-97). A
+ * embedding not tied to the output head), with the results of the dense kernel. The
+ * reference has only the dense kernel (ancora/optim/adamw.py:92-97). A
  * dense step moves rows with zero gradient too (moment decay, bias-corrected momentum, weight
  * decay), so each row carries the last counted step it is current for (last_step, int32[V], zero
  * at the start) and the steps it missed are replayed on it, with g = 0 and that step's own
