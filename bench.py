@@ -309,7 +309,7 @@ def side_workload(args):
                "adamw_kernel": {"ms": round(a_ms, 3), "gbps": round(28.0 * n / (a_ms * 1e-3) / 1e9, 1)},
                "gradnorm_kernel": {"ms": round(g_ms, 3), "gbps": round(2.0 * n / (g_ms * 1e-3) / 1e9, 1)},
                "clip_scale": guard.read(0)["clip_scale"]}
-    out["device"] = {"name": info["name"], "arch": info["arch"], "cus": info["cu_count"]}
+    out["device"] = {"name": info["name"] or info["arch"].split(":")[0], "arch": info["arch"], "cus": info["cu_count"]}
     print(json.dumps(out), flush=True)
 
 
