@@ -625,6 +625,11 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       g.Bl = split_fb ? pl.Bl : nullptr;
       g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
       g.scale = (k == 0) ? cp[q].scale0 : nullptr;
+      // 256-tile kernels: everything the chain itself writes (F, B, every iterate after the input)
+      // is in panel layout; the input pair is row-major as the caller left it
+      g.f_panel = big ? 1 : 0;
+      g.x_panel = (big && k > 0) ? 1 : 0;
+      g.y_panel = big ? 1 : 0;
       // A = X X^T
       ga[q] = g;
       ga[q].A[0] = curH[q]; ga[q].B[0] = curH[q]; ga[q].nterms = 1;

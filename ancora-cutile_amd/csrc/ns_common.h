@@ -88,6 +88,13 @@ struct NsGemm {
   const float *scale;        // (E) or null. The operands are an unnormalised iterate U and the step
                              // acts on X = scale*U: GRAM multiplies its accumulator by scale^2, BX
                              // multiplies the accumulator and the epilogue's X by scale.
+  // Panel layout of a bf16 matrix with R rows: element (r, c) at ((c / 32) * R + r) * 32 + c % 32,
+  // i.e. 32-column panels, each (R, 32) row-major. The K tile of a product is one panel, so the
+  // rows a tile fetches are one contiguous block instead of 64-byte pieces of rows that lie a
+  // whole row pitch apart. 256-tile kernel only; R = M for every matrix of the chain.
+  int f_panel;               // Fh, Fl, Bh, Bl are in panel layout (GRAM, BMAT write them so; BMAT, BX read them so)
+  int x_panel;               // the input iterate (operands X of GRAM and BX, Xh/Xl of the BX epilogue)
+  int y_panel;               // the output iterate Yh/Yl of BX
 };
 
 

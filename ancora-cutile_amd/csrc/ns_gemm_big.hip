@@ -110,8 +110,10 @@ __device__ __forceinline__ void mfma8(const Frags &f, f32x16 (&acc)[4][2]) {
 // its 2 column blocks in accumulator layout (element r: row 8*(r/4) + 4*(lane/32) + r%4, column
 // bj*32 + lane%32), packed two per dword: v[bj][i] = elements r = 2i (low half), 2i+1 (high).
 // Row-major output: out[row*ld + col]; transposed: outT[col*ldT + row].
+// With pstride > 0 the output is in panel layout: `out` addresses the slab's first row in its
+// first 32-column panel, rows lie 32 elements apart and the second panel pstride elements further.
 __device__ __forceinline__ void stage_rows(unsigned char *region, const uint32_t (&v)[2][8], int lane,
-                                           uint16_t *out, int64_t ld) {
+                                           uint16_t *out, int64_t ld, int64_t pstride = 0) {
   uint16_t *t = (uint16_t *)region;                 // [32][72]
 #pragma unroll
   for (int bj = 0; bj < 2; ++bj)
@@ -125,7 +127,8 @@ __device__ __forceinline__ void stage_rows(unsigned char *region, const uint32_t
   for (int p = 0; p < 4; ++p) {
     const int idx = p * 64 + lane, row = idx >> 3, c8 = (idx & 7) * 8;
     const anc_u32x4 q = *(const anc_u32x4 *)(t + row * 72 + c8);
-    epi_st((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
+    if (pstride > 0) epi_st((anc_u32x4 *)(out + (int64_t)(c8 >> 5) * pstride + row * 32 + (c8 & 31)), q);
+    else epi_st((anc_u32x4 *)(out + (int64_t)row * ld + c8), q);
   }
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_wave_barrier();
@@ -268,18 +271,31 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   //      the swizzle: 128-byte rows use chunk ^ ((row>>1)&7), which alternates with the parity
   //      of the instruction index (RPI = 8); 64-byte rows use chunk ^ ((row>>2)&3), the same
   //      for every instruction (RPI = 16).
+  // Panel layout (see NsGemm): rows of a tile lie 64 bytes apart, consecutive K tiles one panel
+  // (rows_of_the_matrix * 64 bytes) apart; a (k, n) tile is one 2 KiB block per 32 columns.
   const int ldA = p.ldA > 0 ? p.ldA : K;
+  constexpr bool PLAINV0 = (VAR == VAR_PLAIN);
+  const bool a_pan = !PLAINV0 && (EPI == EPI_GRAM ? p.x_panel != 0 : p.f_panel != 0);
+  const bool b_pan = !PLAINV0 && (EPI == EPI_BMAT ? p.f_panel != 0 : p.x_panel != 0);
+  const int64_t panel = (int64_t)p.M * 64;          // bytes per panel (every matrix of the chain has M rows)
+  const int rpA = a_pan ? 64 : ldA * 2;             // bytes between consecutive rows of the A operand
+  const int rpB = b_pan ? 64 : K * 2;               // the same for an "NT" B operand
   const int lrow = lane / CPR, pchunk = lane % CPR;
   const int key0 = (TK == 64) ? (lrow >> 1) : ((lrow >> 2) & 3);
-  const uint32_t voff0 = (uint32_t)(lrow * ldA * 2 + ((pchunk ^ key0) * 16));
-  const uint32_t voff1 = (uint32_t)(lrow * ldA * 2 + ((pchunk ^ key0 ^ (TK == 64 ? 4 : 0)) * 16));
+  const uint32_t voff0 = (uint32_t)(lrow * rpA + ((pchunk ^ key0) * 16));
+  const uint32_t voff1 = (uint32_t)(lrow * rpA + ((pchunk ^ key0 ^ (TK == 64 ? 4 : 0)) * 16));
+  const uint32_t voffN0 = (uint32_t)(lrow * rpB + ((pchunk ^ key0) * 16));
+  const uint32_t voffN1 = (uint32_t)(lrow * rpB + ((pchunk ^ key0 ^ (TK == 64 ? 4 : 0)) * 16));
   // (k, m) A tile (AT): TK rows of TM*2 = 256 bytes, four rows per DMA instruction; lane -> (row
   // lane/16, physical chunk lane%16), chunk index XORed with 4*(row&3) as for the B tile.
   static_assert(!AT || (TM == 128 && IA * NWAVES * 4 == TK), "(k,m) tile layout");
-  const uint32_t voffAT = (uint32_t)((lane >> 4) * ldA * 2 + (((lane & 15) ^ ((lane >> 4) << 2)) * 16));
-  const int64_t ubaseA = AT ? ((int64_t)e * p.strideA + (int64_t)tm * TM + (int64_t)(wave * IA * 4) * ldA) * 2
-                            : ((int64_t)e * p.strideA + (int64_t)(tm * TM + wave * (IA * RPI)) * ldA) * 2;   // bytes
-  const int64_t ubaseB = ((int64_t)e * p.strideB + (int64_t)(tn * TN + wave * (IB * RPI)) * K) * 2;
+  const int catl = (lane & 15) ^ ((lane >> 4) << 2);          // logical 16-byte chunk of the (k, m) row
+  const uint32_t voffAT = a_pan ? (uint32_t)((lane >> 4) * 64 + (int64_t)(catl >> 2) * panel + (catl & 3) * 16)
+                                : (uint32_t)((lane >> 4) * ldA * 2 + catl * 16);
+  const int64_t ubaseA = AT ? (a_pan ? (int64_t)e * p.strideA * 2 + (int64_t)(tm * (TM / 32)) * panel + (int64_t)(wave * IA * 4) * 64
+                                     : ((int64_t)e * p.strideA + (int64_t)tm * TM + (int64_t)(wave * IA * 4) * ldA) * 2)
+                            : (int64_t)e * p.strideA * 2 + (int64_t)(tm * TM + wave * (IA * RPI)) * rpA;   // bytes
+  const int64_t ubaseB = (int64_t)e * p.strideB * 2 + (int64_t)(tn * TN + wave * (IB * RPI)) * rpB;
   // (k, n) B tile: TK rows of TN*2 = 512 bytes, two rows per DMA instruction; lane -> (row
   // lane/32, physical chunk lane%32); the chunk index is XORed with 4*(row&3), so that the 4
   // rows a transposing read touches per 32 lanes fall into 4 different 64-byte bank windows.
@@ -287,9 +303,13 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   constexpr bool BT = (EPI == EPI_BX);
   static_assert(!BT || (TN == 256 && IB % 2 == 0 && IB * NWAVES * 2 == TK), "(k,n) tile layout");
   const int ldn = p.N;
-  const uint32_t voffB0 = (uint32_t)((lane >> 5) * ldn * 2 + (((lane & 31) ^ (((lane >> 5)) << 2)) * 16));
-  const uint32_t voffB1 = (uint32_t)((lane >> 5) * ldn * 2 + (((lane & 31) ^ ((2 + (lane >> 5)) << 2)) * 16));
-  const int64_t ubaseBT = ((int64_t)e * p.strideB + (int64_t)tn * TN + (int64_t)(wave * IB * 2) * ldn) * 2;
+  const int cb0 = (lane & 31) ^ ((lane >> 5) << 2), cb1 = (lane & 31) ^ ((2 + (lane >> 5)) << 2);
+  const uint32_t voffB0 = b_pan ? (uint32_t)((lane >> 5) * 64 + (int64_t)(cb0 >> 2) * panel + (cb0 & 3) * 16)
+                                : (uint32_t)((lane >> 5) * ldn * 2 + cb0 * 16);
+  const uint32_t voffB1 = b_pan ? (uint32_t)((lane >> 5) * 64 + (int64_t)(cb1 >> 2) * panel + (cb1 & 3) * 16)
+                                : (uint32_t)((lane >> 5) * ldn * 2 + cb1 * 16);
+  const int64_t ubaseBT = b_pan ? (int64_t)e * p.strideB * 2 + (int64_t)(tn * (TN / 32)) * panel + (int64_t)(wave * IB * 2) * 64
+                                : ((int64_t)e * p.strideB + (int64_t)tn * TN + (int64_t)(wave * IB * 2) * ldn) * 2;
 
   // Operand pointers of the three terms are fetched from the argument block once, here: a
   // scalar load inside the K loop would have to be waited for with lgkmcnt(0), which also
@@ -301,21 +321,22 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     Abase[t3] = (const char *)p.A[t3] + ubaseA;
     Bbase[t3] = (const char *)p.B[t3] + (BT ? ubaseBT : ubaseB);
   }
-  const int64_t advB = BT ? (int64_t)TK * ldn * 2 : (int64_t)ROWB;
-  const int64_t advA = AT ? (int64_t)TK * ldA * 2 : (int64_t)ROWB;
+  // bytes from one K tile to the next, and from one DMA instruction of a tile to the next
+  const int64_t advB = BT ? (b_pan ? (int64_t)TK * 64 : (int64_t)TK * ldn * 2) : (b_pan ? panel : (int64_t)ROWB);
+  const int64_t advA = AT ? (a_pan ? (int64_t)TK * 64 : (int64_t)TK * ldA * 2) : (a_pan ? panel : (int64_t)ROWB);
+  const int64_t roA = AT ? (a_pan ? (int64_t)4 * 64 : (int64_t)4 * ldA * 2) : (int64_t)RPI * rpA;
+  const int64_t roB = BT ? (b_pan ? (int64_t)2 * 64 : (int64_t)2 * ldn * 2) : (int64_t)RPI * rpB;
   const char *curA = Abase[0], *curB = Bbase[0];
   int is_kt = 0, is_term = 0;
   // DMA instruction i of a stage (0 .. IPS-1: the A tile's IA, then the B tile's IB)
   auto issue_piece = [&](int i, unsigned char *stage) {
     if (i < IA) {
-      const int64_t ro = AT ? (int64_t)(i * 4) * ldA * 2 : (int64_t)(i * RPI) * ldA * 2;
       const uint32_t vo = AT ? voffAT : ((i & 1) ? voff1 : voff0);
-      dma16(curA + ro + vo, lds_addr(stage + (wave * IA + i) * 1024));
+      dma16(curA + i * roA + vo, lds_addr(stage + (wave * IA + i) * 1024));
     } else {
       const int j = i - IA;
-      const int64_t ro = BT ? (int64_t)(j * 2) * ldn * 2 : (int64_t)(j * RPI) * K * 2;
-      const uint32_t vo = BT ? ((j & 1) ? voffB1 : voffB0) : ((j & 1) ? voff1 : voff0);
-      dma16(curB + ro + vo, lds_addr(stage + TM * ROWB + (wave * IB + j) * 1024));
+      const uint32_t vo = BT ? ((j & 1) ? voffB1 : voffB0) : ((j & 1) ? voffN1 : voffN0);
+      dma16(curB + j * roB + vo, lds_addr(stage + TM * ROWB + (wave * IB + j) * 1024));
     }
   };
   auto issue_advance = [&]() {
@@ -467,14 +488,21 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     const int q = wave * 2 + (bi & 1);
     return st(q / kBufPerStage) + (q % kBufPerStage) * kInBuf;
   };
-  const uint32_t vo_in0 = (uint32_t)((lane >> 3) * N * 2 + (((lane & 7) ^ (lane >> 3)) * 16));
-  const uint32_t vo_in1 = (uint32_t)((lane >> 3) * N * 2 + (((lane & 7) ^ (lane >> 3) ^ 1) * 16));
+  // (panel layout: the slab is two 2 KiB blocks, rows 64 bytes apart)
+  const bool x_pan = !PLAINV && p.x_panel != 0;
+  const int ci0 = (lane & 7) ^ (lane >> 3), ci1 = ci0 ^ 1;
+  const uint32_t vo_in0 = x_pan ? (uint32_t)((lane >> 3) * 64 + (int64_t)(ci0 >> 2) * panel + (ci0 & 3) * 16)
+                                : (uint32_t)((lane >> 3) * N * 2 + ci0 * 16);
+  const uint32_t vo_in1 = x_pan ? (uint32_t)((lane >> 3) * 64 + (int64_t)(ci1 >> 2) * panel + (ci1 & 3) * 16)
+                                : (uint32_t)((lane >> 3) * N * 2 + ci1 * 16);
+  const int64_t in_row = x_pan ? 64 : (int64_t)N * 2;       // bytes between consecutive rows of the slab
   auto fetch_in = [&](int bi) {
-    const int64_t ub = (mn + (int64_t)(gi0w + bi * 32) * N + gj0w) * 2;
+    const int64_t ub = x_pan ? mn * 2 + (int64_t)(gj0w / 32) * panel + (int64_t)(gi0w + bi * 32) * 64
+                             : (mn + (int64_t)(gi0w + bi * 32) * N + gj0w) * 2;
     unsigned char *b = inbuf(bi);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int64_t ro = (int64_t)(8 * j) * N * 2;
+      const int64_t ro = (int64_t)(8 * j) * in_row;
       const uint32_t vo = (j & 1) ? vo_in1 : vo_in0;
       dma16_epi((const char *)p.Xh + ub + ro + vo, lds_addr(b + j * 1024));
       dma16_epi((const char *)p.Xl + ub + ro + vo, lds_addr(b + 4096 + j * 1024));
@@ -697,19 +725,25 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           }
         __builtin_amdgcn_s_waitcnt(0xC07F);
         __builtin_amdgcn_wave_barrier();
+        // element offset of chunk c (8 columns) of slab row `row` in the output iterate
+        const bool y_pan = p.y_panel != 0;
+        auto y_off = [&](int row, int c) -> int64_t {
+          return y_pan ? mn + ((int64_t)(gj0w / 32 + (c >> 2)) * M + gi0 + row) * 32 + (c & 3) * 8
+                       : mn + (int64_t)(gi0 + row) * N + gj0w + c * 8;
+        };
 #pragma unroll
         for (int pz = 0; pz < 4; ++pz) {
           const int idx = pz * 64 + lane, row = idx >> 3, c = idx & 7;
           const int off = row * 128 + ((c ^ ((row & 7) ^ ((row >> 3) & 1))) * 16);
           const anc_u32x4 qh = *(const anc_u32x4 *)(b + off);
-          epi_st((anc_u32x4 *)(p.Yh + mn + (int64_t)(gi0 + row) * N + gj0w + c * 8), qh);
+          epi_st((anc_u32x4 *)(p.Yh + y_off(row, c)), qh);
         }
 #pragma unroll
         for (int pz = 0; pz < 4; ++pz) {
           const int idx = pz * 64 + lane, row = idx >> 3, c = idx & 7;
           const int off = row * 128 + ((c ^ ((row & 7) ^ ((row >> 3) & 1))) * 16);
           const anc_u32x4 ql = *(const anc_u32x4 *)(b + 4096 + off);
-          epi_st((anc_u32x4 *)(p.Yl + mn + (int64_t)(gi0 + row) * N + gj0w + c * 8), ql);
+          epi_st((anc_u32x4 *)(p.Yl + y_off(row, c)), ql);
         }
       }
       // the buffer is free again once the staged rows have been read back
@@ -780,19 +814,25 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
       for (int i = 0; i < 8; ++i) anc_pk_pair(ov[bj][2 * i], ov[bj][2 * i + 1], hv[bj][i], lv[bj][i]);
+    // Where the slab (rows gi0.., columns gj0w..) and its mirror image (rows gj0w.., columns gi0..:
+    // 64 rows of one 32-column panel, a contiguous 4 KiB in panel layout) go in an (M, M) matrix.
+    const bool f_pan = p.f_panel != 0;
+    const int64_t o_rows = f_pan ? mm + ((int64_t)(gj0w / 32) * M + gi0) * 32 : mm + (int64_t)gi0 * M + gj0w;
+    const int64_t o_cols = f_pan ? mm + ((int64_t)(gi0 / 32) * M + gj0w) * 32 : mm + (int64_t)gj0w * M + gi0;
+    const int64_t ps = f_pan ? (int64_t)M * 32 : 0, ldT = f_pan ? 32 : M;
     if (EPI == EPI_GRAM) {
-      stage_rows(region, hv, lane, p.Fh + mm + (int64_t)gi0 * M + gj0w, M);
-      if (mirror) stage_cols(region, hv, lane, p.Fh + mm + (int64_t)gj0w * M + gi0, M);
+      stage_rows(region, hv, lane, p.Fh + o_rows, M, ps);
+      if (mirror) stage_cols(region, hv, lane, p.Fh + o_cols, ldT);
       if (p.Fl != nullptr) {
-        stage_rows(region, lv, lane, p.Fl + mm + (int64_t)gi0 * M + gj0w, M);
-        if (mirror) stage_cols(region, lv, lane, p.Fl + mm + (int64_t)gj0w * M + gi0, M);
+        stage_rows(region, lv, lane, p.Fl + o_rows, M, ps);
+        if (mirror) stage_cols(region, lv, lane, p.Fl + o_cols, ldT);
       }
     } else if (EPI == EPI_BMAT) {
-      stage_rows(region, hv, lane, p.Bh + mm + (int64_t)gi0 * M + gj0w, M);
-      if (mirror) stage_cols(region, hv, lane, p.Bh + mm + (int64_t)gj0w * M + gi0, M);
+      stage_rows(region, hv, lane, p.Bh + o_rows, M, ps);
+      if (mirror) stage_cols(region, hv, lane, p.Bh + o_cols, ldT);
       if (p.Bl != nullptr) {
-        stage_rows(region, lv, lane, p.Bl + mm + (int64_t)gi0 * M + gj0w, M);
-        if (mirror) stage_cols(region, lv, lane, p.Bl + mm + (int64_t)gj0w * M + gi0, M);
+        stage_rows(region, lv, lane, p.Bl + o_rows, M, ps);
+        if (mirror) stage_cols(region, lv, lane, p.Bl + o_cols, ldT);
       }
       __builtin_amdgcn_s_waitcnt(0xC07F);
       asm volatile("" ::: "memory");
