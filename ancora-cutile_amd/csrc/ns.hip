@@ -19,8 +19,10 @@
 // Xh alone is the matrix-core operand of the early iterations. Where the shape needs it (see
 // split_plan below) late iterations add the residual products: A gets Xh Xl^T + Xl Xh^T and
 // B X gets Boff Xl as extra accumulation terms of the same tile. The symmetric products are
-// "NT" (both operands K-contiguous rows of X or F); B X reads the iterate (K, N) row-major
-// as it lies in memory and transposes inside LDS reads, so X exists in one layout only. The
+// "NT" (both operands K-contiguous rows of X or F); B X reads the iterate as (k, n) tiles
+// and transposes inside LDS reads, so no transposed copy of X exists. The 256-tile kernels
+// keep every matrix the chain writes for itself in panel layout (32-column panels, see NsGemm);
+// the input pair and everything the 128-tile kernels touch is row-major. The
 // fp32 input is read once (normalisation) and the fp32 result written once (last step).
 //
 // Determinism: one workgroup owns one 128x128 output tile and its whole K loop, terms in

@@ -20,6 +20,9 @@
 // X = a X + B X is the iterate itself, (k, n) row-major: its tile is [k][256 columns], fetched
 // as whole 512-byte rows, and its fragments come from transposing LDS reads
 // (ds_read_b64_tr_b16), so no transposed copy of the iterate exists anywhere.
+// Operands in panel layout (NsGemm::f_panel, x_panel) land in the same LDS positions; only the
+// global addresses differ: an [row][k] tile is one contiguous block (rows 64 bytes apart, the
+// next K tile one panel further), a [k][n] tile one 2 KiB block per 32 columns.
 //
 // Stage ring. Tile k of the K loop lives in stage k % NS, each stage a __shared__ array of its
 // own. The DMA instructions of tile k+NS-1 go out between the MFMAs of tile k's first k-step;
