@@ -100,6 +100,7 @@ _PROTOS = {
     "anc_stream_wait_event": (None, [u64, u64]),
     "anc_event_elapsed_ms": (None, [u64, u64, C.POINTER(f32)]),
     "anc_copy_shape": (None, [u64, u64, i64, C.c_int, C.POINTER(i64), u64]),
+    "anc_mfma_rate": (None, [C.c_int, i64, u64, C.POINTER(C.c_double), u64]),
     "anc_copy_kernel": (None, [u64, u64, i64, u64]),
     "anc_profile_enable": (None, [C.c_int]),
     "anc_profile_read": (None, [C.POINTER(f32), C.POINTER(i64)]),

@@ -393,3 +393,72 @@ extern "C" int anc_copy_shape(uint64_t dst, uint64_t src, int64_t n_bytes, int s
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
+
+// ------------------------------------------------------------------ matrix-core reference rate
+// The matrix instruction of the Newton-Schulz GEMMs (v_mfma_f32_32x32x16_bf16) on register
+// operands only, two wavefronts per SIMD on every CU, eight accumulator blocks per wavefront
+// (the GEMM's register tile). What it sustains depends on the operand VALUES: the board runs
+// under a power limit, and products of varying bf16 values draw more than products of zeros
+// or of one constant. values: 0 zeros, 1 one constant pair, 2 pseudo-random values in
+// (-0.05, 0.05), two fragment sets alternating. The counterpart of anc_copy_shape for the
+// matrix pipe: the rate a GEMM's K loop could not exceed on this board with such operands.
+typedef __bf16 mr_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float mr_f32x16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ uint32_t mr_hash(uint32_t x) {
+  x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+  return x;
+}
+__global__ void __launch_bounds__(512) k_mfma_rate(int values, int64_t iters, float *sink) {
+  mr_f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  mr_bf16x8 a[2][4], b[2][2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+#pragma unroll
+    for (int i = 0; i < 6; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t h = mr_hash(((uint32_t)threadIdx.x * 128u + (uint32_t)(s * 48 + i * 8 + e)) * 2654435761u + blockIdx.x);
+        const float v = values == 0 ? 0.0f : values == 1 ? (i < 4 ? 0.5f : 0.25f)
+                                                         : (float)((int)(h & 0xFFFFu) - 32768) * (0.05f / 32768.0f);
+        if (i < 4) a[s][i][e] = (__bf16)v; else b[s][i - 4][e] = (__bf16)v;
+      }
+  }
+  for (int64_t it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
+  }
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) t += acc[i][j][0];
+  if (t == 12345.0f) sink[threadIdx.x] = t;      // never true for these operands; keeps the loop alive
+}
+
+extern "C" int anc_mfma_rate(int values, int64_t iters, uint64_t sink, double *flops, uint64_t stream) {
+  ANC_REQUIRE(values >= 0 && values <= 2 && iters > 0 && iters <= (1ll << 24) && sink != 0 && (sink & 3) == 0 &&
+                  flops != nullptr,
+              "anc_mfma_rate: values 0..2, iters 1..2^24, sink a device buffer of at least 2 KiB");
+  hipDeviceProp_t pr;
+  int dev = 0;
+  ANC_HIP(hipGetDevice(&dev));
+  ANC_HIP(hipGetDeviceProperties(&pr, dev));
+  const int blocks = pr.multiProcessorCount;      // one 8-wavefront workgroup per CU
+  hipStream_t s = anc_stream(stream);
+  AncProfScope prof(ANC_PROF_MISC, s);
+  hipLaunchKernelGGL(k_mfma_rate, dim3((unsigned)blocks), dim3(512), 0, s, values, iters, (float *)sink);
+  ANC_LAUNCH_CHECK();
+  *flops = (double)blocks * 8.0 * (double)iters * 16.0 * 2.0 * 32.0 * 32.0 * 16.0;
+  return ANC_OK;
+}

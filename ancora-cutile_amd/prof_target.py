@@ -19,6 +19,11 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
                                       (anc_copy_shape): TB/s of each, the reference points for
                                       the elementwise optimizer kernels
 
+    python3 -m ancora_cutile_amd.prof_target mfma [launches]            matrix-pipe reference (anc_mfma_rate):
+                                      TFLOP/s of the register-only matrix-instruction loop on zero,
+                                      constant and random operands, with the shader clock rocm-smi
+                                      reports while each runs
+
 Each target allocates its operands, runs the kernel(s) `calls` times on the null stream and
 synchronises; nothing is checked here (parity lives in tests/).
 """
@@ -51,6 +56,48 @@ def main(argv):
             pr = _lib.profile_read()
             _lib.profile_enable(False)
             print("  ".join(f"{k}={v[0]:.3f}ms/{v[1]}" for k, v in pr.items() if v[1]))
+    elif what == "mfma":
+        import re
+        import subprocess
+        import threading
+        import time
+        launches = int(argv[1]) if len(argv) > 1 else 12
+        sink = DevBuf.empty((1024,), np.float32)
+
+        def sclk():
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
+            except Exception:
+                return None
+            m = re.search(r"sclk clock level:\s*\S+\s*\((\d+)Mhz\)", out)
+            return int(m.group(1)) if m else None
+
+        for name, values in (("zeros", 0), ("constant", 1), ("random", 2), ("zeros", 0), ("random", 2)):
+            samples, stop = [], threading.Event()
+
+            def poll():
+                time.sleep(0.5)
+                while not stop.is_set():
+                    v = sclk()
+                    if v:
+                        samples.append(v)
+
+            th = threading.Thread(target=poll, daemon=True)
+            th.start()
+            fl = ctypes.c_double()
+            rates = []
+            for _ in range(launches):
+                e0, e1 = _lib.Event(), _lib.Event()
+                e0.record(0)
+                _lib.api.anc_mfma_rate(values, 400000, sink.ptr, ctypes.byref(fl), 0)
+                e1.record(0)
+                e1.sync()
+                rates.append(fl.value / (e0.elapsed_ms(e1) * 1e-3) / 1e12)
+            stop.set()
+            th.join(timeout=15)
+            busy = sorted(v for v in samples if v > 300)
+            print(f"{name:9s} first launch {rates[0]:7.1f}  last {rates[-1]:7.1f} TFLOP/s over {launches} launches; "
+                  f"sclk while running: {busy if busy else 'n/a'} MHz", flush=True)
     elif what == "adamw":
         n = int(argv[1]) // 64 * 64
         calls = int(argv[2]) if len(argv) > 2 else 3

@@ -59,6 +59,62 @@ def synth(shapes, seed=0):
     return params, grads
 
 
+def read_sclk_mhz():
+    """Current shader clock in MHz from `rocm-smi --showclocks` (read-only), or None."""
+    import re
+    import subprocess
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
+    except Exception:
+        return None
+    m = re.search(r"sclk clock level:\s*\S+\s*\((\d+)Mhz\)", out)
+    return int(m.group(1)) if m else None
+
+
+def sustained_sclk(run_steps, seconds=1.5):
+    """Median shader clock while `run_steps(n)` keeps the GPU busy with optimizer steps: a sampler
+    thread polls rocm-smi, the main thread keeps launching (launches are asynchronous and the
+    library calls drop the GIL). Outside the timed region. None if rocm-smi gives nothing."""
+    import threading
+    samples, stop = [], threading.Event()
+
+    def poll():
+        time.sleep(0.4)                      # let the clock settle under load
+        while not stop.is_set():
+            v = read_sclk_mhz()
+            if v:
+                samples.append(v)
+
+    th = threading.Thread(target=poll, daemon=True)
+    th.start()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        run_steps(5)
+    stop.set()
+    th.join(timeout=15)
+    samples = sorted(v for v in samples if v > 300)   # drop samples taken while the GPU idled
+    return samples[len(samples) // 2] if samples else None
+
+
+def mfma_reference(_lib, DevBuf):
+    """TFLOP/s of the register-only matrix-instruction loop (anc_mfma_rate) on zero and on random
+    operands: what the matrix pipe sustains on this board without any memory traffic."""
+    import ctypes
+    sink = DevBuf.empty((1024,), np.float32)
+    out = {}
+    for name, values in (("zeros", 0), ("random", 2)):
+        fl = ctypes.c_double()
+        _lib.api.anc_mfma_rate(values, 20000, sink.ptr, ctypes.byref(fl), 0)      # clocks settle
+        e0, e1 = _lib.Event(), _lib.Event()
+        e0.record(0)
+        _lib.api.anc_mfma_rate(values, 400000, sink.ptr, ctypes.byref(fl), 0)
+        e1.record(0)
+        e1.sync()
+        out[name] = round(fl.value / (e0.elapsed_ms(e1) * 1e-3) / 1e12, 1)
+    sink.free()
+    return out
+
+
 def kernel_source_sha16():
     """Hash of the Newton-Schulz kernel sources: ties a recorded counter figure to the code it was
     measured on."""
@@ -437,6 +493,18 @@ def main():
         nh128, extra128 = ns_hard_info(b.ws.buf.ptr, b.E, b.M, b.Nn, 5, "bf16_tile128")
         lower128 += ex128 + extra128
         last_bx += ns_product_flops(b.E, b.M, b.Nn, 4, 2, 5, "bf16")
+    # What the board sustains: the shader clock while the step runs (the nominal 2.4 GHz is not
+    # held under the power limit) and the matrix pipe's register-only rate on zero / random operands
+    opt.muon.engine.serial = bool(args.serial)
+
+    def run_steps(n):
+        for _ in range(n):
+            opt.step(gdev, 0)
+        _lib.stream_sync(0)
+
+    sclk = sustained_sclk(run_steps)
+    mfma_ref = mfma_reference(_lib, DevBuf)
+
     # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
     # last X = a X + B X) also reads and writes the weights
     gemm_kinds = ("ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx", "ns_gemm_bx_update")
@@ -497,6 +565,13 @@ def main():
                                                      "frac": round(pure_achieved / PEAK_BF16_TFLOPS, 4),
                                                      "avg_launch_ms": round(pure_ms / max(1, pure_launches), 4)},
                      "avg_launch_ms": round(gemm_ms / max(1, gemm_launches), 4),
+                     # context, not the fraction asked for: the board holds `sustained_sclk_mhz`, not
+                     # its nominal clock, under the step's load, and its matrix pipe alone (registers
+                     # only) sustains `mfma_register_loop_tflops.random` on operands that vary
+                     "frac_of_peak_at_sustained_clock": (round(achieved / (PEAK_BF16_TFLOPS * sclk * 1e3 / info["clock_khz"]), 4)
+                                                         if sclk and info["clock_khz"] else None),
+                     "frac_of_register_loop_on_random_operands": (round(achieved / mfma_ref["random"], 4)
+                                                                  if mfma_ref.get("random") else None),
                      "executed_tflop_per_step": round(executed / 1e12, 3),
                      "executed_counts": "what the kernels multiply: residual and gated terms, and of the symmetric "
                                         "products the 256x256 tiles on or below the diagonal, each in full "
@@ -522,6 +597,8 @@ def main():
         "event_ms_per_step": round(ev_ms, 3), "wall_ms_per_step": round(wall_ms, 3),
         "streams": "serial" if args.serial else "one: the Newton-Schulz chains of all shape groups advance together (grouped launches)",
         "copy_kernel_gbps": round(copy_gbps, 1),
+        "sustained_sclk_mhz": sclk,
+        "mfma_register_loop_tflops": mfma_ref,
         "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
         "device": {"name": info["name"] or info["arch"].split(":")[0], "arch": info["arch"], "cus": info["cu_count"],
                    "clock_khz": info["clock_khz"]},

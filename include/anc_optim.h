@@ -100,6 +100,14 @@ int anc_copy_kernel(uint64_t dst, uint64_t src, int64_t n_bytes, uint64_t stream
  * each of the two buffers; *bytes_moved receives the bytes read plus written. */
 int anc_copy_shape(uint64_t dst, uint64_t src, int64_t n_bytes, int shape, int64_t *bytes_moved,
                    uint64_t stream);
+/* The matrix pipe's counterpart of anc_copy_shape (no reference counterpart): `iters` rounds of 16
+ * v_mfma_f32_32x32x16_bf16 on register operands per wavefront, eight wavefronts on every CU, no
+ * memory traffic. values: 0 zeros, 1 one constant pair, 2 pseudo-random bf16 values. The board
+ * runs under a power limit and the rate it sustains depends on the operand values, so this is
+ * the ceiling a GEMM K loop has on this board with such operands, next to the nominal
+ * 2.5 PFLOP/s. sink: device buffer of at least 2 KiB (never written); *flops receives the
+ * floating-point operations of the launch; time it with events around the call. */
+int anc_mfma_rate(int values, int64_t iters, uint64_t sink, double *flops, uint64_t stream);
 
 /* ------------------------------------------------------------- profiling ----
  * Per-kernel timing with HIP events on the launch stream, for the benchmarks (the
