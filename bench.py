@@ -115,6 +115,54 @@ def mfma_reference(_lib, DevBuf):
     return out
 
 
+def measure_gemm_traffic(workload):
+    """HBM bytes per k_ns_gemm_big launch, measured now: two child runs of this script under
+    `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE: the profiler does not split counters over
+    passes), each scaled by what the same counter reads for the 1 GiB copy kernel the run contains.
+    Called before this process touches the GPU. Returns (bytes_per_launch, detail dict)."""
+    import shutil
+    import signal
+    import sqlite3
+    import subprocess
+    import tempfile
+    if shutil.which("rocprofv3") is None:
+        raise RuntimeError("rocprofv3 not found")
+    top = tempfile.mkdtemp(prefix="anc_traffic_", dir="/tmp")
+    res = {}
+    for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
+        cmd = ["rocprofv3", "--pmc", ctr, "-d", os.path.join(top, ctr), "-o", ctr, "--",
+               "python3", os.path.abspath(__file__), "--workload", workload, "--serial", "--steps", "3",
+               "--warmup", "1", "--no-cpu", "--no-clock"]
+        log(" ".join(cmd))
+        pr = subprocess.Popen(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, start_new_session=True,
+                              stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        try:
+            rc = pr.wait(timeout=280)
+        except subprocess.TimeoutExpired:
+            os.killpg(pr.pid, signal.SIGKILL)
+            raise RuntimeError(f"rocprofv3 --pmc {ctr} did not finish")
+        if rc != 0:
+            raise RuntimeError(f"rocprofv3 --pmc {ctr} exited with {rc}")
+        dbs = [os.path.join(d, f) for d, _, fs in os.walk(os.path.join(top, ctr)) for f in fs if f.endswith("_results.db")]
+        if not dbs:
+            raise RuntimeError(f"no results database under {top}/{ctr}")
+        rows = sqlite3.connect(dbs[0]).execute(
+            "select kernel_name, count(*), sum(value) from counters_collection where counter_name = ? "
+            "group by kernel_name", (ctr,)).fetchall()
+        copy = [r for r in rows if "k_copy16" in r[0]]
+        gemm = [r for r in rows if "k_ns_gemm_big" in r[0]]
+        if not copy or not gemm:
+            raise RuntimeError(f"{ctr}: copy or GEMM kernel missing from the counter table")
+        unit_kib = (1 << 20) / (sum(r[2] for r in copy) / sum(r[1] for r in copy))   # KiB per count: 1 GiB moved each way
+        n = sum(r[1] for r in gemm)
+        res[ctr] = (sum(r[2] for r in gemm) * unit_kib * 1024.0 / n, n, unit_kib)
+    shutil.rmtree(top, ignore_errors=True)
+    total = int(res["FETCH_SIZE"][0] + res["WRITE_SIZE"][0])
+    return total, {"read_bytes_per_launch": int(res["FETCH_SIZE"][0]), "write_bytes_per_launch": int(res["WRITE_SIZE"][0]),
+                   "launches_counted": res["FETCH_SIZE"][1], "fetch_unit_kib": round(res["FETCH_SIZE"][2], 4),
+                   "write_unit_kib": round(res["WRITE_SIZE"][2], 4)}
+
+
 def kernel_source_sha16():
     """Hash of the Newton-Schulz kernel sources: ties a recorded counter figure to the code it was
     measured on."""
@@ -376,6 +424,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=28, help=argparse.SUPPRESS)   # smaller sets for debugging
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-clock", action="store_true",
+                    help="skip the sustained-clock sampling and the matrix-pipe reference launches")
+    ap.add_argument("--traffic", action="store_true",
+                    help="measure roofline.traffic now: two extra runs of this script under rocprofv3 --pmc "
+                         "(about a minute); without it the figure recorded under profiles/ is reported while "
+                         "the kernel sources are the ones it was taken with")
+    ap.add_argument("--write-traffic", action="store_true",
+                    help="with --traffic: also rewrite profiles/ns_gemm_traffic.json from the measurement")
     ap.add_argument("--tokens", type=int, default=8192, help="tokens per micro-batch of --workload dw")
     ap.add_argument("--dw-acts", default="x", choices=("x", "xT"),
                     help="--workload dw: activations as they lie (T,K), or transposed by the caller")
@@ -397,6 +453,10 @@ def main():
 
     if args.workload in ("ns", "adamw", "dw"):
         return side_workload(args)
+    live_traffic = None
+    if args.traffic:          # child processes first: this one has not touched the GPU yet
+        live_traffic = measure_gemm_traffic(args.workload)
+        log(f"HBM bytes per k_ns_gemm_big launch, measured: {live_traffic[0]} {live_traffic[1]}")
     from ancora_cutile_amd import HybridOptimizer, DevBuf, PE_SCHEDULE, _lib
     from ancora_cutile_amd.hybrid import resident_is_muon
     from ancora_cutile_amd.muon_ns import ns_flops, ns_product_flops, ns_hard_info
@@ -502,8 +562,8 @@ def main():
             opt.step(gdev, 0)
         _lib.stream_sync(0)
 
-    sclk = sustained_sclk(run_steps)
-    mfma_ref = mfma_reference(_lib, DevBuf)
+    sclk = None if args.no_clock else sustained_sclk(run_steps)
+    mfma_ref = {} if args.no_clock else mfma_reference(_lib, DevBuf)
 
     # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
     # last X = a X + B X) also reads and writes the weights
@@ -533,7 +593,18 @@ def main():
     # the kernel sources still have the hash those runs were taken with; otherwise null.
     traffic, traffic_note = None, "not measured in this run"
     tpath = os.path.join(ROOT, "profiles", "ns_gemm_traffic.json")
-    if args.workload == "qwen3" and args.layers == 28 and os.path.exists(tpath):
+    if live_traffic is not None:
+        traffic = live_traffic[0]
+        traffic_note = ("measured in this run: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE child runs of this command, "
+                        f"scaled by the 1 GiB copy kernel {live_traffic[1]}")
+        if args.write_traffic and args.workload == "qwen3" and args.layers == 28:
+            with open(tpath, "w") as f:
+                json.dump({"kernel": "k_ns_gemm_big", "hbm_bytes_per_launch": traffic, **live_traffic[1],
+                           "source": "profiles/hybrid_step_qwen3_0p6b_hbm_traffic.md",
+                           "source_sha16": kernel_source_sha16(),
+                           "command": "python3 bench.py --traffic --write-traffic --no-cpu"}, f, indent=1)
+                f.write("\n")
+    elif args.workload == "qwen3" and args.layers == 28 and os.path.exists(tpath):
         with open(tpath) as f:
             tj = json.load(f)
         if tj.get("source_sha16") == kernel_source_sha16():
