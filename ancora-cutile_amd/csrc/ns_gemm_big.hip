@@ -277,9 +277,9 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // Panel layout (see NsGemm): rows of a tile lie 64 bytes apart, consecutive K tiles one panel
   // (rows_of_the_matrix * 64 bytes) apart; a (k, n) tile is one 2 KiB block per 32 columns.
   const int ldA = p.ldA > 0 ? p.ldA : K;
-  constexpr bool PLAINV0 = (VAR == VAR_PLAIN);
-  const bool a_pan = !PLAINV0 && (EPI == EPI_GRAM ? p.x_panel != 0 : p.f_panel != 0);
-  const bool b_pan = !PLAINV0 && (EPI == EPI_BMAT ? p.f_panel != 0 : p.x_panel != 0);
+  static_assert(TK == 32, "a K tile is one 32-column panel");
+  const bool a_pan = !PLAINV && (EPI == EPI_GRAM ? p.x_panel != 0 : p.f_panel != 0);
+  const bool b_pan = !PLAINV && (EPI == EPI_BMAT ? p.f_panel != 0 : p.x_panel != 0);
   const int64_t panel = (int64_t)p.M * 64;          // bytes per panel (every matrix of the chain has M rows)
   const int rpA = a_pan ? 64 : ldA * 2;             // bytes between consecutive rows of the A operand
   const int rpB = b_pan ? 64 : K * 2;               // the same for an "NT" B operand
