@@ -333,3 +333,48 @@ def test_backward_to_step_hand_off(gpu):
     for n in params:
         assert bits_equal(ma[n], mb[n])
     g_ln.free()
+
+
+def test_accumulated_micro_batches_against_one_batch(gpu):
+    """The reference's accumulation check (tests/training/test_grad_accum.py:60-93) on this path:
+    the gradient of 2T tokens in one call against two calls of T tokens, the second accumulating
+    onto the first. (B) the two gradients agree to the reference's bar (rel < 2e-3; here only the
+    fp32 regrouping of the sum separates them); (C) the accumulated route repeats bit for bit;
+    (D) after one AdamW step on each, at least 98 % of the updated weights are bit-identical."""
+    from ancora_cutile_amd import AdamW, DevBuf
+    from ancora_cutile_amd.grads import gemm_dW
+    T, K, N = 1024, 512, 1024
+    x, dy = _inputs(2 * T, K, N, 77)
+    rng = np.random.default_rng(5)
+    w0 = (0.02 * rng.standard_normal((K, N))).astype(np.float32)
+
+    def one_batch():
+        p = _problem(x, dy, 2 * T, K, N, emit=True)
+        gemm_dW([p])
+        out = p["dW"].to_numpy(), p["g16"].to_numpy()
+        _free(p)
+        return out
+
+    def accumulated():
+        p0 = _problem(x[:T], dy[:T], T, K, N, emit=True)
+        gemm_dW([p0])
+        first = p0["dW"].to_numpy()
+        p1 = _problem(x[T:], dy[T:], T, K, N, emit=True, dW0=first)
+        gemm_dW([p1])
+        out = p1["dW"].to_numpy(), p1["g16"].to_numpy()
+        _free(p0); _free(p1)
+        return out
+
+    (gA, hA), (gB, hB), (gB2, hB2) = one_batch(), accumulated(), accumulated()
+    assert rel_fro(gB, gA) < 2e-3 and rel_fro(gB, gA) < 1e-6          # (B): reference bar, then what it is here
+    assert bits_equal(gB, gB2) and bits_equal(hB, hB2)                 # (C)
+    assert rel_fro(gA, gemm_dw(x, dy)) < 2e-5 and rel_fro(gB, gemm_dw(x, dy)) < 2e-5
+    new = []
+    for h in (hA, hB):
+        opt = AdamW({"w": w0}, lr=1e-3, grad_dtype=np.uint16)
+        g = DevBuf(h)
+        opt.step({"w": g}, 0)
+        new.append(opt.weights()["w"])
+        opt.free(); g.free()
+    same = float((new[0].view(np.uint32) == new[1].view(np.uint32)).mean())
+    assert same >= 0.98, same                                          # (D): the reference's bar
