@@ -115,6 +115,23 @@ def mfma_reference(_lib, DevBuf):
     return out
 
 
+def gemm_bytes_from_counter_db(path, ctr):
+    """(bytes per k_ns_gemm_big launch, launches, KiB per count) from a rocprofv3 results database
+    that holds counter `ctr` for the GEMM launches and for the 1 GiB copy kernel of the same run
+    (which moves 1 GiB each way: its reading fixes the counter's unit)."""
+    import sqlite3
+    rows = sqlite3.connect(path).execute(
+        "select kernel_name, count(*), sum(value) from counters_collection where counter_name = ? "
+        "group by kernel_name", (ctr,)).fetchall()
+    copy = [r for r in rows if "k_copy16" in r[0]]
+    gemm = [r for r in rows if "k_ns_gemm_big" in r[0]]
+    if not copy or not gemm:
+        raise RuntimeError(f"{ctr}: copy or GEMM kernel missing from the counter table")
+    unit_kib = (1 << 20) / (sum(r[2] for r in copy) / sum(r[1] for r in copy))
+    n = sum(r[1] for r in gemm)
+    return sum(r[2] for r in gemm) * unit_kib * 1024.0 / n, n, unit_kib
+
+
 def measure_gemm_traffic(workload):
     """HBM bytes per k_ns_gemm_big launch, measured now: two child runs of this script under
     `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE: the profiler does not split counters over
@@ -122,7 +139,6 @@ def measure_gemm_traffic(workload):
     Called before this process touches the GPU. Returns (bytes_per_launch, detail dict)."""
     import shutil
     import signal
-    import sqlite3
     import subprocess
     import tempfile
     if shutil.which("rocprofv3") is None:
@@ -146,16 +162,7 @@ def measure_gemm_traffic(workload):
         dbs = [os.path.join(d, f) for d, _, fs in os.walk(os.path.join(top, ctr)) for f in fs if f.endswith("_results.db")]
         if not dbs:
             raise RuntimeError(f"no results database under {top}/{ctr}")
-        rows = sqlite3.connect(dbs[0]).execute(
-            "select kernel_name, count(*), sum(value) from counters_collection where counter_name = ? "
-            "group by kernel_name", (ctr,)).fetchall()
-        copy = [r for r in rows if "k_copy16" in r[0]]
-        gemm = [r for r in rows if "k_ns_gemm_big" in r[0]]
-        if not copy or not gemm:
-            raise RuntimeError(f"{ctr}: copy or GEMM kernel missing from the counter table")
-        unit_kib = (1 << 20) / (sum(r[2] for r in copy) / sum(r[1] for r in copy))   # KiB per count: 1 GiB moved each way
-        n = sum(r[1] for r in gemm)
-        res[ctr] = (sum(r[2] for r in gemm) * unit_kib * 1024.0 / n, n, unit_kib)
+        res[ctr] = gemm_bytes_from_counter_db(dbs[0], ctr)
     shutil.rmtree(top, ignore_errors=True)
     total = int(res["FETCH_SIZE"][0] + res["WRITE_SIZE"][0])
     return total, {"read_bytes_per_launch": int(res["FETCH_SIZE"][0]), "write_bytes_per_launch": int(res["WRITE_SIZE"][0]),

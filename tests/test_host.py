@@ -148,3 +148,27 @@ def test_flop_accounting_matches_the_tiles_the_kernels_multiply():
     sym = 10 * 2 * 256 * 256 * M
     assert ex_sq == 4 * (2 * sym + 2.0 * M ** 3) + 1 * (3 * sym + sym + 2 * 2.0 * M ** 3)
     assert ns_flops(1, M, M, 5, "fp32")[0] == ns_flops(1, M, M, 5, "fp32")[1]
+
+
+def test_bench_reads_gemm_traffic_from_a_counter_database(tmp_path):
+    """bench.py --traffic: bytes per GEMM launch = counter sum over the GEMM launches, in the unit the
+    1 GiB copy kernel of the same run fixes. A hand-made database with a known answer."""
+    import sqlite3
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    db = str(tmp_path / "x_results.db")
+    con = sqlite3.connect(db)
+    con.execute("create table counters_collection (kernel_name text, counter_name text, value real)")
+    rows = [("k_copy16(a, b, long)", "FETCH_SIZE", 524288.0), ("k_copy16(a, b, long)", "FETCH_SIZE", 524288.0),
+            ("void k_ns_gemm_big<0, 256>(NsGemmMulti)", "FETCH_SIZE", 1000.0),
+            ("void k_ns_gemm_big<2, 128>(NsGemmMulti)", "FETCH_SIZE", 3000.0),
+            ("void k_ns_gemm_big<2, 128>(NsGemmMulti)", "WRITE_SIZE", 77.0),
+            ("k_adamw_multi", "FETCH_SIZE", 5.0)]
+    con.executemany("insert into counters_collection values (?, ?, ?)", rows)
+    con.commit()
+    con.close()
+    per_launch, n, unit = bench.gemm_bytes_from_counter_db(db, "FETCH_SIZE")
+    assert unit == 2.0 and n == 2 and per_launch == (1000.0 + 3000.0) * 2.0 * 1024.0 / 2
+    with pytest.raises(RuntimeError):
+        bench.gemm_bytes_from_counter_db(db, "WRITE_SIZE")          # no copy kernel row for this counter
