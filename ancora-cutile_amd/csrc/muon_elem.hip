@@ -309,7 +309,7 @@ k_mom_multi(const anc_muon_desc_t *__restrict__ table, int n_weights, float mom,
   if (!load_ctl(ctl, clip)) return;
   const anc_muon_desc_t d = find_weight(table, n_weights, (int64_t)blockIdx.x);
   const int64_t local = (int64_t)blockIdx.x - d.tile0;
-  MomArgs a{(float *)d.buf, (const void *)d.g, (void *)d.u, d.K, d.N};
+  MomArgs a{(float *)d.buf, (const void *)d.g, (void *)d.u, d.K, d.N, nullptr, nullptr};
   if (d.transpose) {
     if (d.g_dtype == ANC_BF16) mom_tile_t<ANC_BF16, UD>(a, local, mom, nesterov, clip);
     else                       mom_tile_t<ANC_F32, UD>(a, local, mom, nesterov, clip);
@@ -427,7 +427,7 @@ extern "C" int anc_muon_momentum(uint64_t buf, uint64_t g, uint64_t u, int64_t K
   ANC_REQUIRE((g_dtype == ANC_F32 || g_dtype == ANC_BF16) && (u_dtype == ANC_F32 || u_dtype == ANC_BF16),
               "anc_muon_momentum: bad dtype");
   ANC_REQUIRE(((buf | g | u) & 15) == 0, "anc_muon_momentum: pointers must be 16-byte aligned");
-  MomArgs a{(float *)buf, (const void *)g, (void *)u, (int)K, (int)N};
+  MomArgs a{(float *)buf, (const void *)g, (void *)u, (int)K, (int)N, nullptr, nullptr};
   const anc_step_ctl_t *c = (const anc_step_ctl_t *)ctl;
   const dim3 grid((unsigned)((K * N) / kBlockElems)), block(kThreads);
   hipStream_t s = anc_stream(stream);

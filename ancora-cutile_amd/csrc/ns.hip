@@ -886,7 +886,7 @@ extern "C" int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N, int s
   { AncProfScope prof(ANC_PROF_NS_PREP, s); hipLaunchKernelGGL(k_ns_prep, dim3(prep_grid), dim3(kThreads), 0, s, X32, pl.recip, mn, total8,
                      pl.Xh[0], pl.Xl[0]); }
   ANC_LAUNCH_CHECK();
-  ChainProb cp{pl, pl.Xh[0], pl.Xl[0], 1, nullptr, X32, E, M, N};
+  ChainProb cp{pl, pl.Xh[0], pl.Xl[0], 1, nullptr, X32, E, M, N, nullptr};
   return run_bf16_chain(&cp, 1, steps, coef, force_small, s);
 }
 
@@ -918,7 +918,7 @@ extern "C" int anc_ns_batched_pair(uint64_t Uh, uint64_t Ul, uint64_t fro_partia
   { AncProfScope prof(ANC_PROF_NS_FRO, s); hipLaunchKernelGGL(k_pair_rescale, dim3((unsigned)E), dim3(kThreads), 0, s,
                      (uint16_t *)Uh, (uint16_t *)Ul, pl.pow2, M * N); }
   ANC_LAUNCH_CHECK();
-  ChainProb cp{pl, (const uint16_t *)Uh, (const uint16_t *)Ul, 0, pl.recip, (float *)X32_out, E, M, N};
+  ChainProb cp{pl, (const uint16_t *)Uh, (const uint16_t *)Ul, 0, pl.recip, (float *)X32_out, E, M, N, nullptr};
   return run_bf16_chain(&cp, 1, steps, coef, force_small, s);
 }
 

@@ -55,9 +55,6 @@ namespace {
 #define LDS3(p) ((__attribute__((address_space(3))) void *)(p))
 #define GLB1(p) ((const __attribute__((address_space(1))) void *)(p))
 
-// vmcnt(0), leave lgkmcnt/expcnt alone (gfx9 encoding: vmcnt [3:0]+[15:14], expcnt [6:4], lgkmcnt [11:8])
-__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
-
 // X = a X + B X reads its symmetric B operand by rows k (see AT below).
 constexpr bool kBxReadsBByRows = true;
 
