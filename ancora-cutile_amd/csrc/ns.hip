@@ -465,8 +465,17 @@ struct SplitPlan {
   static constexpr int kGateIters = 8;
   float gate_tau[kGateIters];
   unsigned gate_bx;
+  // The wide gate: a matrix whose proxy lies in (wide_lo, wide_hi) adds the residual of X to
+  // A = X X^T from iteration wide_gram_from on and the residuals of X, F and Boff to all three
+  // products from iteration wide_all_from on. wide_hi == 0: no such gate.
+  float wide_lo, wide_hi;
+  int wide_gram_from, wide_all_from;
   bool gated(int k) const { return k >= 0 && k < kGateIters && k < x_from && gate_tau[k] > 0.0f; }
+  bool wide() const { return wide_hi > 0.0f; }
+  bool wide_gram(int k) const { return wide() && k >= wide_gram_from && k < x_from; }
+  bool wide_all(int k) const { return wide() && k >= wide_all_from && k < fb_from; }
   bool any_gate(int steps) const {
+    if (wide()) return true;
     for (int k = 0; k < steps; ++k) if (gated(k)) return true;
     return false;
   }
@@ -483,7 +492,16 @@ struct SplitPlan {
 //     matrix with independent entries needs them in the last one only (1.66e-3 against 1.41e-3 at
 //     1024x1024, 5.3e-4 either way with outlier rows), the column-scaled case needs both (1.85e-3
 //     against 2.09e-3). So the first of the two is gated low.
-constexpr float kTauHard = 2.5f, kTauPlain = 1.3f;
+//   kTauWideLo .. kTauWideHi: inputs whose spectrum is spread over decades, or with many moderately
+//     large columns. Measured proxies (1024x1024 / 1024x3072): log-uniform spectrum over one decade
+//     1.4 / 4.0, 1.5 decades 2.4 / 7.4, two 3.6 / 11.3, three 5.8 / 19.4; 10 % of the columns x10 8.4;
+//     against 1 % of the columns x100 100, x1000 102, a rank-32 signal over noise 32 / 95, a
+//     power-law spectrum 146 / 437. In the band the plan above leaves 2.5e-3 .. 4.2e-3 (every operand
+//     rounding of the later iterations counts: the small singular values are still far from 1);
+//     with the residual of X in A = X X^T from iteration 1 and all residuals in all products of the
+//     last three iterations: 1.0e-4 .. 4.8e-4. Above the band the gates above suffice (8e-4 ..
+//     1.4e-3; only outliers x1000 miss the bar, with or without these terms at 1024x1024).
+constexpr float kTauHard = 2.5f, kTauPlain = 1.3f, kTauWideLo = 2.5f, kTauWideHi = 40.0f;
 SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
   SplitPlan sp{};
   sp.x_from = sp.fb_from = steps;
@@ -497,6 +515,10 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
   // The first iterations are insensitive (the singular values are still far below 1, so
   // B X is a small correction to a X); residuals start at a fixed iteration index.
   if (M >= 1024) {
+    if (steps == 5) {                         // the schedule length the wide gate was measured on
+      sp.wide_lo = kTauWideLo; sp.wide_hi = kTauWideHi;
+      sp.wide_gram_from = 1; sp.wide_all_from = 2;
+    }
     if (N < 2 * M) {
       sp.x_from = steps - 2 < 3 ? steps - 2 : 3;
       sp.gate_tau[1] = sp.gate_tau[2] = kTauHard;
@@ -558,7 +580,7 @@ Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int ste
     pl.A32 = c.take<float>(E * M * M);
     pl.Fh = c.take<uint16_t>(E * M * M);
     pl.Bh = c.take<uint16_t>(E * M * M);
-    if (pl.sp.fb_from < steps) {
+    if (pl.sp.fb_from < steps || pl.sp.wide()) {
       pl.Fl = c.take<uint16_t>(E * M * M);
       pl.Bl = c.take<uint16_t>(E * M * M);
     }
@@ -632,11 +654,20 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       g.f_panel = big ? 1 : 0;
       g.x_panel = (big && k > 0) ? 1 : 0;
       g.y_panel = big ? 1 : 0;
+      // the wide gate of this iteration (a band of the proxy; the proxy is N * sum, hence the / N)
+      const bool wide_g = pl.sp.wide_gram(k);      // implies !split
+      const bool wide_a = pl.sp.wide_all(k);       // implies !split_fb
+      auto set_wide = [&](NsGemm &w, int nterms_wide) {
+        if (w.cond == nullptr) { w.cond = pl.cond; w.cond_thresh = 1e300; w.nterms_hard = w.nterms; }
+        w.wide_lo = (double)pl.sp.wide_lo / (double)N;
+        w.wide_hi = (double)pl.sp.wide_hi / (double)N;
+        w.nterms_wide = nterms_wide;
+      };
       // A = X X^T
       ga[q] = g;
       ga[q].A[0] = curH[q]; ga[q].B[0] = curH[q]; ga[q].nterms = 1;
       const bool gated = pl.sp.gated(k);           // implies !split
-      if (split || gated) {
+      if (split || gated || wide_g) {
         ga[q].A[1] = curH[q]; ga[q].B[1] = curL[q];
         ga[q].A[2] = curL[q]; ga[q].B[2] = curH[q];
         if (split) ga[q].nterms = 3;
@@ -646,14 +677,25 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
         ga[q].cond_thresh = (double)pl.sp.gate_tau[k] / (double)N;
         ga[q].nterms_hard = 3;
       }
+      if (wide_g) set_wide(ga[q], 3);
+      if (wide_a) {                                // the residual of F, for the matrices in the band only
+        set_wide(ga[q], split ? 0 : 3);
+        ga[q].Fl = pl.Fl;
+        ga[q].lo_gated = 1;
+      }
       ga[q].K = (int)N; ga[q].strideA = mn; ga[q].strideB = mn; ga[q].tiles_m = tM; ga[q].tiles_n = tM; ga[q].lower = 1;
       // B = b A + c A A
       gb[q] = g;
       gb[q].A[0] = pl.Fh; gb[q].B[0] = pl.Fh; gb[q].nterms = 1;
-      if (split_fb) {
+      if (split_fb || wide_a) {
         gb[q].A[1] = pl.Fh; gb[q].B[1] = pl.Fl;
         gb[q].A[2] = pl.Fl; gb[q].B[2] = pl.Fh;
-        gb[q].nterms = 3;
+        if (split_fb) gb[q].nterms = 3;
+      }
+      if (wide_a) {
+        set_wide(gb[q], 3);
+        gb[q].Bl = pl.Bl;
+        gb[q].lo_gated = 1;
       }
       gb[q].K = (int)M; gb[q].strideA = M * M; gb[q].strideB = M * M; gb[q].tiles_m = tM; gb[q].tiles_n = tM; gb[q].lower = 1;
       // X = a X + B X
@@ -667,6 +709,11 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
         gx[q].nterms_hard = 2;
       }
       if (split_fb) { gx[q].A[gx[q].nterms] = pl.Bl; gx[q].B[gx[q].nterms] = curH[q]; ++gx[q].nterms; }
+      if (wide_a) {                                // [Bh Xh, Bh Xl, Bl Xh]: the lists above are prefixes of it
+        gx[q].A[1] = pl.Bh; gx[q].B[1] = curL[q];
+        gx[q].A[2] = pl.Bl; gx[q].B[2] = curH[q];
+        set_wide(gx[q], 3);
+      }
       gx[q].K = (int)M; gx[q].strideA = M * M; gx[q].strideB = mn; gx[q].tiles_m = tM; gx[q].tiles_n = tN; gx[q].lower = 0;
       gx[q].Xh = curH[q]; gx[q].Xl = curL[q];
       gx[q].Yh = last ? nullptr : pl.Xh[nxt[q]];
@@ -722,8 +769,10 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
 extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode) {
   mode &= ~ANC_NS_TILE128;
   if (check_shape(E, M, N, mode, "anc_ns_workspace_bytes")) return -1;
-  // sized for any step count: with steps >= 3 every optional buffer of the mode is present
-  return make_plan(0, E, M, N, mode, 64).bytes;
+  // sized for any step count: with steps >= 3 every optional buffer of the mode's plan is present;
+  // the 5-step schedule adds the residual buffers of the wide gate
+  const int64_t a = make_plan(0, E, M, N, mode, 64).bytes, b = make_plan(0, E, M, N, mode, 5).bytes;
+  return a > b ? a : b;
 }
 
 // FLOPs of the output tiles a symmetric M x M product really multiplies, per unit of K: the tiles
@@ -809,7 +858,17 @@ extern "C" int anc_ns_hard_info(uint64_t workspace, int64_t E, int64_t M, int64_
     double t = host[(size_t)(e * kCondParts)];
     for (int i = 1; i < kCondParts; ++i) t = t + host[(size_t)(e * kCondParts + i)];
     bool any = false;
+    const bool in_band = pl.sp.wide() && t > (double)pl.sp.wide_lo / (double)N && t < (double)pl.sp.wide_hi / (double)N;
     for (int k = 0; k < steps; ++k) {
+      if (in_band) {                    // the wide gate takes precedence over the others
+        const bool sx = k >= pl.sp.x_from;
+        if (pl.sp.wide_gram(k)) { *extra_flops += gram_extra; any = true; }
+        if (pl.sp.wide_all(k)) {
+          *extra_flops += 2.0 * sym_tile_flops(M, N, force_small) * (double)M + (sx ? 1.0 : 2.0) * bx_extra;
+          any = true;
+        }
+        continue;
+      }
       if (!pl.sp.gated(k) || !(t > (double)pl.sp.gate_tau[k] / (double)N)) continue;
       any = true;
       *extra_flops += gram_extra + (((pl.sp.gate_bx >> k) & 1u) ? bx_extra : 0.0);

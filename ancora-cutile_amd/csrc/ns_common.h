@@ -85,6 +85,13 @@ struct NsGemm {
                              // nterms_hard terms instead of nterms (its list is a prefix of the hard one)
   double cond_thresh;
   int nterms_hard;
+  // Second gate on the same proxy: a matrix whose sum lies strictly between wide_lo and wide_hi
+  // (a spectrum spread over decades, many moderately large columns) multiplies nterms_wide terms;
+  // 0 = no such gate. It takes precedence over the gate above. With lo_gated set, the residual
+  // outputs Fl / Bl are written for such matrices only (else for every matrix when non-null).
+  double wide_lo, wide_hi;
+  int nterms_wide;
+  int lo_gated;
   const float *scale;        // (E) or null. The operands are an unnormalised iterate U and the step
                              // acts on X = scale*U: GRAM multiplies its accumulator by scale^2, BX
                              // multiplies the accumulator and the epilogue's X by scale.
@@ -101,12 +108,23 @@ struct NsGemm {
 // Number of accumulation terms of matrix e: p.nterms, or p.nterms_hard for a matrix that the
 // conditioning proxy marks as hard. The partial sums are added in a fixed order, so every
 // workgroup of every launch takes the same decision for a matrix.
-__device__ __forceinline__ int anc_ns_terms(const NsGemm &p, int e) {
-  if (p.cond == nullptr) return p.nterms;
+__device__ __forceinline__ double anc_ns_proxy(const NsGemm &p, int e) {
   const double *c = p.cond + (int64_t)e * kCondParts;
   double s = c[0];
 #pragma unroll
   for (int i = 1; i < kCondParts; ++i) s = s + c[i];
+  return s;
+}
+// Does matrix e lie in the band of the second gate?
+__device__ __forceinline__ bool anc_ns_wide(const NsGemm &p, int e) {
+  if (p.cond == nullptr || p.wide_hi <= 0.0) return false;
+  const double s = anc_ns_proxy(p, e);
+  return s > p.wide_lo && s < p.wide_hi;
+}
+__device__ __forceinline__ int anc_ns_terms(const NsGemm &p, int e) {
+  if (p.cond == nullptr) return p.nterms;
+  const double s = anc_ns_proxy(p, e);
+  if (p.nterms_wide > 0 && s > p.wide_lo && s < p.wide_hi) return p.nterms_wide;
   return s > p.cond_thresh ? p.nterms_hard : p.nterms;
 }
 

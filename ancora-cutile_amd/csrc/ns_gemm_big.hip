@@ -474,6 +474,10 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   float sc = 1.0f;
   if (EPI != EPI_BMAT && p.scale != nullptr) sc = p.scale[e];
   const float acc_scale = (EPI == EPI_GRAM) ? sc * sc : sc;
+  // residual output (Fl of GRAM, Bl of BMAT): for every matrix, or only for those in the band of
+  // the second conditioning gate (uniform over the workgroup: a function of the matrix)
+  const bool write_lo = (EPI == EPI_GRAM ? p.Fl != nullptr : EPI == EPI_BMAT ? p.Bl != nullptr : false) &&
+                        (p.lo_gated == 0 || anc_ns_wide(p, e));
 
   // X = a X + B X reads the iterate at the output position (the bf16 pair Xh, Xl). A 32x64 slab
   // of each is 32 rows of 128 bytes: 4 DMA instructions (8 rows each, lane -> row lane/8, chunk
@@ -763,7 +767,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       // Wait for this slab's DMA only (see the X = a X + B X branch). Stores of a slab: 4 per
       // staged bf16 block (Bh, its mirror, and the same for Bl); the conditional dB stores of
       // diagonal tiles only add to what may stay outstanding, so leaving them out is safe.
-      const int nst = 4 * ((mirror ? 2 : 1) * (p.Bl != nullptr ? 2 : 1));
+      const int nst = 4 * ((mirror ? 2 : 1) * (write_lo ? 2 : 1));
       if (bi == 0) wait_vm<8>();
       else if (bi == 3) { if (nst == 4) wait_vm<4>(); else if (nst == 8) wait_vm<8>(); else wait_vm<16>(); }
       else { if (nst == 4) wait_vm<12>(); else if (nst == 8) wait_vm<16>(); else wait_vm<24>(); }
@@ -823,14 +827,14 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     if (EPI == EPI_GRAM) {
       stage_rows(region, hv, lane, p.Fh + o_rows, M, ps);
       if (mirror) stage_cols(region, hv, lane, p.Fh + o_cols, ldT);
-      if (p.Fl != nullptr) {
+      if (write_lo) {
         stage_rows(region, lv, lane, p.Fl + o_rows, M, ps);
         if (mirror) stage_cols(region, lv, lane, p.Fl + o_cols, ldT);
       }
     } else if (EPI == EPI_BMAT) {
       stage_rows(region, hv, lane, p.Bh + o_rows, M, ps);
       if (mirror) stage_cols(region, hv, lane, p.Bh + o_cols, ldT);
-      if (p.Bl != nullptr) {
+      if (write_lo) {
         stage_rows(region, lv, lane, p.Bl + o_rows, M, ps);
         if (mirror) stage_cols(region, lv, lane, p.Bl + o_cols, ldT);
       }
