@@ -442,12 +442,19 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *             1.3, both X-products of iteration 3 (5-step chains; every matrix has them in
  *             iteration 4): a matrix with independent entries or outlier rows does without
  *             (1.66e-3 / 5e-4 at 1024x1024), the column-scaled case needs them (1.85e-3);
- *   2M <= N < 3M: no gate (1.6e-3 on the outlier-column case as it is).
+ *   2M <= N < 3M: none of these (1.6e-3 on the outlier-column case as it is);
+ *   M >= 1024, 5-step chains, every N: strictly between 2.5 and 40 (the wide gate: a spectrum spread
+ *             over two or three decades reads 3.6 .. 19, 10 % of the columns x10 reads 8.4; outlier
+ *             columns x100, low-rank signals and power-law spectra read 30 .. 440 and do not need
+ *             it), the residual of X in A = X X^T from iteration 1 and the residuals of X, F and
+ *             Boff in all three products of iterations 2..4 (about 2.3 times the matrix-core work,
+ *             for that matrix alone): 1.9e-4 .. 5e-4 instead of 2.5e-3 .. 4.2e-3. It takes precedence
+ *             over the gates above.
  * The decision depends on the matrix alone (fixed-order sums), never on the batch. Accuracy bar of
  * ANC_NS_BF16 with the Polar-Express schedule: 2e-3 relative Frobenius on inputs with independent
- * entries, with row or column outliers up to x100 on 1 % of the rows or columns, with columns
- * scaled over a factor 30; spectra spread over two decades or more (condition number >= 1e2 with
- * a log-uniform spectrum) reach 2.5e-3 .. 4e-3 and need ANC_NS_BF16_X3. Keller coefficients
+ * entries, with row or column outliers up to x100 on 1 % of the rows or columns, with 10 % of the
+ * columns x10, with columns scaled over a factor 30, with log-uniform spectra up to condition
+ * number 1e3. Not met: outliers x1000 (2.7e-3 .. 4e-3; ANC_NS_BF16_X3). Keller coefficients
  * amplify operand rounding about twice as much (4.5e-3 at 1024x1024).
  *
  * M and N must be multiples of 128 (the reference's tile alignment,
