@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("ANCORA_OPTIM_LIB") or os.path.join(_HERE, "csrc", "li
 
 F32, BF16 = 0, 1                  # ANC_F32 / ANC_BF16
 FORM_DIV, FORM_IBC = 0, 1         # ANC_ADAMW_FORM_*
-NS_BF16, NS_FP32, NS_BF16_FAST, NS_BF16_X3 = 0, 1, 2, 3   # ANC_NS_*
+NS_BF16, NS_FP32, NS_BF16_FAST, NS_BF16_X3, NS_BF16_LATE3 = 0, 1, 2, 3, 4   # ANC_NS_*
 GN_CHUNK = 8192                   # ANC_GN_CHUNK
 MUON_MAX_SCALES = 8               # ANC_MUON_MAX_SCALES
 

@@ -190,6 +190,7 @@ class MuonEngine:
         lr_scales = (ctypes.c_float * MUON_MAX_SCALES)(*[lr * s for s in self.scales])
         seed_base = ((self.seed + 1000003 * self.t) & 0xFFFFFFFF) if self.sr else 0
         coef = muon_ns.coef_array(schedule, self.ns)
+        self._run_mode = muon_ns.effective_mode(self.mode, schedule)
         together = [b for b in self.batches
                     if self.grouped and self.fused_prologue and b.M % 256 == 0 and b.Nn % 256 == 0]
         if not self.concurrent and len(self.batches) > 1:
@@ -215,18 +216,18 @@ class MuonEngine:
                 if i < len(self._streams):
                     self._fork.wait_on(st)
             b.build(b.U, self.scale_index)
-            buf = b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self.mode))
+            buf = b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self._run_mode))
             if self.fused_prologue:
                 self._momentum_pair(b, ctl, st)
                 n_el = b.E * b.M * b.Nn
                 api.anc_ns_batched_pair(b.U.ptr, b.U.ptr + n_el * 2, b.fro.ptr,
                                         b.total_blocks // b.E, b.U.ptr, b.E, b.M, b.Nn, self.ns, coef,
-                                        1e-7, muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(st))
+                                        1e-7, muon_ns.MODES[self._run_mode], buf.ptr, buf.nbytes, int(st))
             else:
                 api.anc_muon_momentum_multi(b.table.ptr, b.E, b.total_blocks, self.mom,
                                             int(self.nesterov), F32, ctl, int(st))
                 api.anc_ns_batched(b.U.ptr, b.E, b.M, b.Nn, self.ns, coef, 1e-7,
-                                   muon_ns.MODES[self.mode], buf.ptr, buf.nbytes, int(st))
+                                   muon_ns.MODES[self._run_mode], buf.ptr, buf.nbytes, int(st))
             api.anc_muon_update_multi(b.table.ptr, b.E, b.total_blocks, lr_scales, F32,
                                       int(self.sr), seed_base, ctl, int(st))
             if forked:
@@ -246,7 +247,7 @@ class MuonEngine:
         probs = (_lib.NsProblem * len(group))()
         for k, b in enumerate(group):
             b.build(b.U, self.scale_index)
-            buf = b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self.mode))
+            buf = b.ws.ensure(muon_ns.ns_workspace_bytes(b.E, b.M, b.Nn, self._run_mode))
             self._momentum_pair(b, ctl, si)
             n_el = b.E * b.M * b.Nn
             probs[k] = _lib.NsProblem(b.U.ptr, b.U.ptr + n_el * 2, b.fro.ptr, b.U.ptr, buf.ptr,
@@ -254,10 +255,10 @@ class MuonEngine:
         if self.fused_update and not any(w.get("p16T") is not None for b in group for w in b.weights):
             tables = (ctypes.c_uint64 * len(group))(*[b.table.ptr for b in group])
             api.anc_muon_ns_update_multi(probs, len(group), tables, self.ns, coef, 1e-7,
-                                         muon_ns.MODES[self.mode], lr_scales, int(self.sr), seed_base, ctl,
+                                         muon_ns.MODES[self._run_mode], lr_scales, int(self.sr), seed_base, ctl,
                                          int(si))
             return
-        api.anc_ns_batched_pair_multi(probs, len(group), self.ns, coef, 1e-7, muon_ns.MODES[self.mode],
+        api.anc_ns_batched_pair_multi(probs, len(group), self.ns, coef, 1e-7, muon_ns.MODES[self._run_mode],
                                       int(si))
         for b in group:
             api.anc_muon_update_multi(b.table.ptr, b.E, b.total_blocks, lr_scales, F32,

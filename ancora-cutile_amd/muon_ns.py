@@ -17,7 +17,7 @@ import ctypes
 import numpy as np
 
 from . import _lib
-from ._lib import api, NS_BF16, NS_FP32, NS_BF16_FAST, NS_BF16_X3
+from ._lib import api, NS_BF16, NS_FP32, NS_BF16_FAST, NS_BF16_X3, NS_BF16_LATE3
 from .devbuf import DevBuf
 
 NTM, NTN, NTK = 128, 128, 64                       # ancora/kernels/muon_ns.py:20
@@ -31,8 +31,13 @@ PE_SCHEDULE = [(4.0848, -6.8946, 2.9270),
                (2.8366, -3.0525, 1.2012)]
 
 MODES = {"bf16": NS_BF16, "bf16_fast": NS_BF16_FAST, "bf16_x3": NS_BF16_X3, "fp32": NS_FP32,
+         "bf16_late3": NS_BF16_LATE3,
+         # the gated plan whatever the schedule ("bf16" turns into "bf16_late3" under Keller's
+         # coefficients, see effective_mode)
+         "bf16_gated": NS_BF16,
          # same arithmetic forced onto the 128x128-tile kernel (ANC_NS_TILE128), for tests
-         "bf16_tile128": NS_BF16 | 0x100, "bf16_fast_tile128": NS_BF16_FAST | 0x100}
+         "bf16_tile128": NS_BF16 | 0x100, "bf16_fast_tile128": NS_BF16_FAST | 0x100,
+         "bf16_late3_tile128": NS_BF16_LATE3 | 0x100}
 
 
 def _coef_at(schedule, k):
@@ -60,6 +65,24 @@ def set_polar_express(on: bool):
 
 def _resolve(schedule):
     return _DEFAULT_SCHEDULE if schedule is _KELLER else schedule
+
+
+def is_keller(schedule):
+    """True for a resolved schedule that applies Keller's triple in every iteration."""
+    return schedule is None or all(tuple(t) == (A_COEF, B_COEF, C_COEF) for t in schedule)
+
+
+def effective_mode(mode, schedule):
+    """The mode a chain call runs in. Keller's quintic does not drive the singular values to 1
+    (they end in 0.7 .. 1.2), so the off-diagonal of A = X X^T never becomes small and the bf16
+    rounding of every operand stays a first-order error up to the last iteration: the gated plan
+    of "bf16", tuned on Polar Express, reaches 3e-3 .. 5e-3 there. Under Keller "bf16" therefore
+    runs as "bf16_late3" (residual terms in every product of the last three iterations, 2.2 times
+    the matrix-core work, well inside 2e-3); "bf16_gated" keeps the gated plan. `schedule` is
+    the resolved one (None = Keller)."""
+    if mode == "bf16" and is_keller(schedule):
+        return "bf16_late3"
+    return mode
 
 
 def coef_array(schedule, steps):
@@ -138,6 +161,7 @@ def ns_batched(X32, E, M, N, si, steps=5, eps=1e-7, schedule=_KELLER, mode="bf16
     schedule = _resolve(schedule)
     if X32.dtype != np.float32 or X32.size < E * M * N:
         raise ValueError(f"ns_batched: X32 must hold {E}x{M}x{N} float32, has {X32.size} {X32.dtype}")
+    mode = effective_mode(mode, schedule)
     ws = _SHARED_WS if workspace is None else workspace
     need = ns_workspace_bytes(E, M, N, mode)
     buf = ws.ensure(need)
@@ -160,6 +184,7 @@ def ns_batched_pair(U, fro_partials, n_partials, E, M, N, si, steps=5, eps=1e-7,
         raise ValueError(f"ns_batched_pair: U must hold {E}x{M}x{N} float32, has {U.size} {U.dtype}")
     if mode == "fp32" or steps < 2:
         raise ValueError("ns_batched_pair: bf16 modes and steps >= 2 only")
+    mode = effective_mode(mode, schedule)
     ws = _SHARED_WS if workspace is None else workspace
     buf = ws.ensure(ns_workspace_bytes(E, M, N, mode))
     coef = coef_array(schedule, steps)
@@ -173,6 +198,7 @@ def _run_bf16(gX, E, M, N, si, steps, eps, schedule, mode, workspace):
         raise ValueError("newton_schulz_resident: gX must hold the packed bf16 (uint16) batch")
     if M % NTM or N % NTN or M > N:
         raise ValueError(f"newton_schulz_resident: (M,N)=({M},{N}) must be 128-aligned with M <= N")
+    mode = effective_mode(mode, schedule)
     ws = _SHARED_WS if workspace is None else workspace
     n = E * M * N
     need = ns_workspace_bytes(E, M, N, mode)

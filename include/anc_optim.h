@@ -428,6 +428,13 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *                     accumulation terms per product in every iteration): about 1e-5 from the
  *                     fp32 chain on every input tried, ill-conditioned ones included, for three
  *                     times the matrix-core work of ANC_NS_BF16_FAST.
+ *   ANC_NS_BF16_LATE3 ANC_NS_BF16 with the residuals of both operands in all three products of the
+ *                     last three iterations, for every matrix and without gates, for M >= 1024
+ *                     (M < 1024 runs that plan under ANC_NS_BF16 already): about 2.2 times the
+ *                     matrix-core work of ANC_NS_BF16_FAST. For coefficients that do not drive the
+ *                     singular values to 1: Keller's quintic (ancora/kernels/muon_ns.py:21) leaves
+ *                     them in 0.7 .. 1.2, offdiag(A) never becomes small and ANC_NS_BF16 reaches
+ *                     2.8e-3 .. 5e-3 only; this mode 3e-5 .. 8e-4.
  *   ANC_NS_FP32       every product in fp32 (validation mode).
  *
  * Conditioning gates (ANC_NS_BF16 only). After the first A = X X^T the chain measures
@@ -455,7 +462,8 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  * entries, with row or column outliers up to x100 on 1 % of the rows or columns, with 10 % of the
  * columns x10, with columns scaled over a factor 30, with log-uniform spectra up to condition
  * number 1e3. Not met: outliers x1000 (2.7e-3 .. 4e-3; ANC_NS_BF16_X3). Keller coefficients
- * amplify operand rounding about twice as much (4.5e-3 at 1024x1024).
+ * amplify operand rounding about twice as much (4.5e-3 at 1024x1024): with them the bar is that of
+ * ANC_NS_BF16_LATE3, which the host layer selects for that schedule.
  *
  * M and N must be multiples of 128 (the reference's tile alignment,
  * ancora/optim/muon.py:98). workspace must hold anc_ns_workspace_bytes(E,M,N,mode)
@@ -464,8 +472,14 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
 #define ANC_NS_FP32 1
 #define ANC_NS_BF16_FAST 2
 #define ANC_NS_BF16_X3 3
+#define ANC_NS_BF16_LATE3 4
 /* Flag OR-ed into a bf16 mode: use the 128x128-tile GEMM kernel even where the 256x256-tile
- * kernel applies. Both produce the same bits; the flag exists so that tests can show it. */
+ * kernel applies. The two produce the same bits wherever no product has residual terms
+ * (ANC_NS_BF16_FAST; ANC_NS_BF16 on wide matrices that take no gate). Residual terms are added
+ * in an order that depends on which elements of a symmetric product are computed and which are
+ * mirrored, hence on the tile size: the results then differ in the last fp32 bits of A and B
+ * (1e-6 .. 4e-4 of the result, largest on gated outlier-column inputs, inside the accuracy bar
+ * either way). The flag exists so that tests can show both. */
 #define ANC_NS_TILE128 0x100
 int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode);
 int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N,

@@ -25,8 +25,8 @@ def _cos(a, b):
 def test_device_muon_reproduces_the_host_class(gpu, K, N, sched):
     """Same W0, same five gradients: the accumulated update W0 - W5 against the numpy class.
     The momentum buffer never depends on the weights, so it is bit-equal after every step and the
-    five update directions are each one chain call: the reference's bars hold with its default
-    (Keller) schedule, the 2e-3 bar with Polar-Express."""
+    five update directions are each one chain call: the reference's bars and the 2e-3 bar hold
+    with its default (Keller) schedule and with Polar-Express."""
     from ancora_cutile_amd import DeviceMuon, DevBuf
     from ancora_cutile_amd.muon import _f32bf_trunc
     schedule = None if sched == "keller" else PE_SCHEDULE
@@ -48,7 +48,7 @@ def test_device_muon_reproduces_the_host_class(gpu, K, N, sched):
     c, r = _cos(du_d, du_h), rel_fro(du_d, du_h)
     print(f"({K},{N}) {sched}: accumulated update cos {c:.6f} rel {r:.3e}")
     assert c > 0.99 and r < 0.06                                    # _probe_device_muon.py:65
-    assert r < (2e-3 if sched == "pe" else 5e-3)
+    assert r < 2e-3
     assert bits_equal(dm.p16.to_numpy(), bf16_rne_bits(Wd))         # refreshed by RNE after a step
     g_dev.free()
     dm.free()
@@ -127,7 +127,7 @@ def test_device_newton_schulz5_matches_the_host_function(gpu):
         want = ns5_ref(G, 5)
         got = newton_schulz5(G)
         assert got.shape == (K, N) and got.dtype == np.float32
-        assert rel_fro(got, want) < 5e-3, (K, N)                     # Keller, default bf16 mode
+        assert rel_fro(got, want) < 2e-3, (K, N)                     # Keller, default bf16 mode
         assert rel_fro(newton_schulz5(G, mode="fp32"), want) < 1e-5, (K, N)
         X = G.T if K > N else G
         pe = host_ns(X, PE_SCHEDULE, 5)

@@ -114,6 +114,12 @@ def test_schedule_toggle_and_constants():
     prev = muon_ns.set_polar_express(True)
     assert prev is None and muon_ns._resolve(muon_ns._KELLER) is muon_ns.PE_SCHEDULE
     assert muon_ns._resolve(None) is None                      # explicit None still means Keller
+    # Keller's coefficients turn "bf16" into the late-three plan; Polar Express keeps the gated one
+    assert muon_ns.effective_mode("bf16", None) == "bf16_late3"
+    assert muon_ns.effective_mode("bf16", [(3.4445, -4.7750, 2.0315)] * 5) == "bf16_late3"
+    assert muon_ns.effective_mode("bf16", muon_ns.PE_SCHEDULE) == "bf16"
+    for m in ("bf16_gated", "bf16_fast", "bf16_x3", "fp32"):
+        assert muon_ns.effective_mode(m, None) == m
     assert muon_ns.set_polar_express(False) is muon_ns.PE_SCHEDULE
     assert muon_ns._coef_at(muon_ns.PE_SCHEDULE, 7) == muon_ns.PE_SCHEDULE[-1]
     assert muon_ns._coef_at(None, 0) == (3.4445, -4.7750, 2.0315)
