@@ -518,7 +518,7 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
     // offdiag(A) never becomes small and every operand rounding stays first-order): 1024x1024
     // Gaussian 3.7e-3 -> 6e-5, 1024x3072 2.8e-3 -> 3e-5, condition number 1e3 2.5e-4 .. 3.2e-4,
     // 1 % of the columns x100 3.6e-4 .. 7.9e-4; residuals in the last two iterations only leave
-    // 2.2e-3 at 1024x1024. M < 1024 already runs this plan.
+    // 2.2e-3 at 1024x1024. M < 1024 runs a heavier plan in either mode (below).
     sp.x_from = sp.fb_from = steps > 3 ? steps - 3 : 0;
     return sp;
   }
@@ -544,8 +544,15 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
       sp.gate_tau[2] = kTauHard;
     }
   } else {
-    sp.x_from = sp.fb_from = steps - 3 < 2 ? steps - 3 : 2;
-    sp.gate_tau[1] = kTauHard;
+    // Small matrices average fewer rounding errors per element and cost next to nothing: all
+    // residuals from iteration 1 on, from iteration 0 below M = 256, no gates. With them from
+    // iteration 2 (relative Frobenius error, Polar Express / Keller): 128x128 condition number 1e3
+    // 4.0e-3 / 2.8e-3, columns scaled 0.1..3 under Keller 2.5e-3, 128x384 and 256x512 condition
+    // number 1e3 5.5e-3 / 4.0e-3 and 2.4e-3 / 1.8e-3, 512x1024 with 1 % of the columns x100
+    // 4.4e-3; from iteration 1: at most 1.0e-3 on all of these from M = 256 on; 128x128 with one
+    // column x100 still 4.8e-3, 1e-5 from iteration 0.
+    const int from = M < 256 ? 0 : 1;
+    sp.x_from = sp.fb_from = steps - 3 < from ? steps - 3 : from;
   }
   if (sp.x_from < 0) sp.x_from = 0;
   if (sp.fb_from < 0) sp.fb_from = 0;

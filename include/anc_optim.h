@@ -430,7 +430,7 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *                     times the matrix-core work of ANC_NS_BF16_FAST.
  *   ANC_NS_BF16_LATE3 ANC_NS_BF16 with the residuals of both operands in all three products of the
  *                     last three iterations, for every matrix and without gates, for M >= 1024
- *                     (M < 1024 runs that plan under ANC_NS_BF16 already): about 2.2 times the
+ *                     (M < 1024 runs a heavier plan in either mode, see below): about 2.2 times the
  *                     matrix-core work of ANC_NS_BF16_FAST. For coefficients that do not drive the
  *                     singular values to 1: Keller's quintic (ancora/kernels/muon_ns.py:21) leaves
  *                     them in 0.7 .. 1.2, offdiag(A) never becomes small and ANC_NS_BF16 reaches
@@ -450,6 +450,10 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *             iteration 4): a matrix with independent entries or outlier rows does without
  *             (1.66e-3 / 5e-4 at 1024x1024), the column-scaled case needs them (1.85e-3);
  *   2M <= N < 3M: none of these (1.6e-3 on the outlier-column case as it is);
+ *   M < 1024: no gates. Small matrices average fewer rounding errors per element and cost next to
+ *             nothing: every product carries the residuals of X, F and Boff from iteration 1 on
+ *             (from iteration 0 below M = 256), for every matrix, in ANC_NS_BF16 and
+ *             ANC_NS_BF16_LATE3 alike (at most 1e-3 on the input classes below, both schedules);
  *   M >= 1024, 5-step chains, every N: strictly between 2.5 and 40 (the wide gate: a spectrum spread
  *             over two or three decades reads 3.6 .. 19, 10 % of the columns x10 reads 8.4; outlier
  *             columns x100, low-rank signals and power-law spectra read 30 .. 440 and do not need

@@ -351,7 +351,8 @@ def test_outlier_columns_take_the_gate_and_meet_the_bar(gpu, M, N):
     X = np.stack([gauss, cols, rows])
     got = run_ns(X)
     n_hard, extra = _hard_count(3, M, N)
-    gated = N < 2 * M or N >= 3 * M               # 2M <= N < 3M meets the bar without the extra terms
+    # 2M <= N < 3M meets the bar without the extra terms; M < 1024 has them for every matrix
+    gated = M >= 1024 and (N < 2 * M or N >= 3 * M)
     assert (n_hard == 1 and extra > 0) if gated else (n_hard == 0 and extra == 0)
     errs = [rel_fro(got[e], host_ns(X[e], PE_SCHEDULE, 5)) for e in range(3)]
     print(f"({M},{N}) gaussian {errs[0]:.3e}  outlier columns {errs[1]:.3e}  outlier rows {errs[2]:.3e}")
@@ -364,6 +365,25 @@ def test_outlier_columns_take_the_gate_and_meet_the_bar(gpu, M, N):
     assert _hard_count(1, M, N, "bf16_fast") == (0, 0.0)
     if gated:
         assert rel_fro(fast[0], host_ns(X[1], PE_SCHEDULE, 5)) > errs[1]
+
+
+@pytest.mark.parametrize("M,N", [(128, 128), (128, 384), (256, 256), (256, 512), (512, 1024), (768, 768)])
+@pytest.mark.parametrize("sched", ["pe", "keller"])
+def test_small_matrices_on_hard_inputs_within_the_bar(gpu, M, N, sched):
+    """M < 1024 carries all residual terms from iteration 1 on (from iteration 0 below M = 256), for
+    every matrix and without gates: condition number 1e3, columns scaled 0.1..3 and 1 % of the
+    columns x100 stay within 6e-4 under both schedules (measured: at most 4.3e-4) (with residuals from iteration 2 only:
+    up to 5.5e-3 at M = 128, 4.4e-3 at 512x1024)."""
+    rng = np.random.default_rng(7 * M + N)
+    schedule = PE_SCHEDULE if sched == "pe" else None
+    X = np.stack([_log_spectrum(rng, M, N, 1e3),
+                  rng.standard_normal((M, N)).astype(np.float32) * rng.uniform(0.1, 3, N).astype(np.float32),
+                  _outlier_cols(rng, M, N)])
+    got = run_ns(X, schedule=schedule)
+    errs = [rel_fro(got[e], host_ns(X[e], schedule, 5)) for e in range(3)]
+    print(f"({M},{N}) {sched}: cond 1e3 {errs[0]:.3e}  columns scaled {errs[1]:.3e}  outlier columns {errs[2]:.3e}")
+    assert max(errs) < 6e-4
+    assert _hard_count(3, M, N) == (0, 0.0)
 
 
 @pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 1536), (1024, 3072)])
