@@ -538,9 +538,11 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
         sp.gate_bx = 1u << 3;
         sp.x_from = 4;
       }
-    } else if (N >= 3 * M) {
-      // iteration 2 alone. In between (2M <= N < 3M) nothing: there the outlier-column case meets
-      // the bar without (1.6e-3 at 1024x2048) and the term would buy 6 %.
+    } else if (N >= 3 * M || N > 2 * M || M > 1024) {
+      // iteration 2 alone. Not at 1024x2048 itself: there the outlier-column case meets the bar
+      // without (1.57e-3 .. 1.61e-3 over seeds) and the term would cost its matrices 6 %; the rest
+      // of 2M <= N < 3M does not (1024x2560 1.8e-3, 1536x3072 2.1e-3, 2048x4096 2.2e-3, 4096x8192
+      // 2.3e-3 without).
       sp.gate_tau[2] = kTauHard;
     }
   } else {

@@ -449,7 +449,8 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *             1.3, both X-products of iteration 3 (5-step chains; every matrix has them in
  *             iteration 4): a matrix with independent entries or outlier rows does without
  *             (1.66e-3 / 5e-4 at 1024x1024), the column-scaled case needs them (1.85e-3);
- *   2M <= N < 3M: none of these (1.6e-3 on the outlier-column case as it is);
+ *   2M <= N < 3M: as N >= 3M (1536x3072, 2048x4096: 1.0e-3 instead of 2.1e-3 .. 2.3e-3), except
+ *             1024x2048 itself: none (1.6e-3 on the outlier-column case as it is);
  *   M < 1024: no gates. Small matrices average fewer rounding errors per element and cost next to
  *             nothing: every product carries the residuals of X, F and Boff from iteration 1 on
  *             (from iteration 0 below M = 256), for every matrix, in ANC_NS_BF16 and
