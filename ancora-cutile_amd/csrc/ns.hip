@@ -491,7 +491,10 @@ struct SplitPlan {
 //   kTauPlain: N < 2M runs the residual of X in both X-products of the last two iterations; a
 //     matrix with independent entries needs them in the last one only (1.66e-3 against 1.41e-3 at
 //     1024x1024, 5.3e-4 either way with outlier rows), the column-scaled case needs both (1.85e-3
-//     against 2.09e-3). So the first of the two is gated low.
+//     against 2.09e-3). So the first of the two is gated low. Between the two thresholds square
+//     matrices were still within 4 % of the bar (columns scaled over 0.03..3, proxy 1.79: 1.93e-3;
+//     log-normal column scales, sigma 0.45, proxy 2.2: 1.79e-3), so iteration 2 carries the same
+//     two terms behind the same gate: 1.48e-3 and 1.25e-3.
 //   kTauWideLo .. kTauWideHi: inputs whose spectrum is spread over decades, or with many moderately
 //     large columns. Measured proxies (1024x1024 / 1024x3072): log-uniform spectrum over one decade
 //     1.4 / 4.0, 1.5 decades 2.4 / 7.4, two 3.6 / 11.3, three 5.8 / 19.4; 10 % of the columns x10 8.4;
@@ -534,8 +537,8 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
       sp.x_from = steps - 2 < 3 ? steps - 2 : 3;
       sp.gate_tau[1] = sp.gate_tau[2] = kTauHard;
       if (steps == 5) {                       // the schedule the low gate was measured on
-        sp.gate_tau[3] = kTauPlain;
-        sp.gate_bx = 1u << 3;
+        sp.gate_tau[2] = sp.gate_tau[3] = kTauPlain;
+        sp.gate_bx = (1u << 2) | (1u << 3);
         sp.x_from = 4;
       }
     } else if (N >= 3 * M || N > 2 * M || M > 1024) {

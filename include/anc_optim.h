@@ -446,9 +446,10 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *   N >= 3M:  above 2.5, A = X X^T of iteration 2 (1 % of the columns x100 at 1024x3072: 1.15e-3
  *             instead of 2.2e-3);
  *   N < 2M:   above 2.5, A = X X^T of iterations 1 and 2 (1024x1024: 8e-4 instead of 3.8e-3); above
- *             1.3, both X-products of iteration 3 (5-step chains; every matrix has them in
+ *             1.3, both X-products of iterations 2 and 3 (5-step chains; every matrix has them in
  *             iteration 4): a matrix with independent entries or outlier rows does without
- *             (1.66e-3 / 5e-4 at 1024x1024), the column-scaled case needs them (1.85e-3);
+ *             (1.67e-3 / 5e-4 at 1024x1024), column-scaled ones need them (columns scaled over
+ *             0.1..3: 1.45e-3; 2.1e-3 with iteration 4 alone, 1.9e-3 with iterations 3 and 4);
  *   2M <= N < 3M: as N >= 3M (1536x3072, 2048x4096: 1.0e-3 instead of 2.1e-3 .. 2.3e-3), except
  *             1024x2048 itself: none (1.6e-3 on the outlier-column case as it is);
  *   M < 1024: no gates. Small matrices average fewer rounding errors per element and cost next to
