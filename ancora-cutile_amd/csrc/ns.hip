@@ -437,6 +437,102 @@ __global__ void __launch_bounds__(kThreads) k_ns_cond(NsCondArgs a) {
   }
 }
 
+// ------------------------------------------------------------------ column statistic, classification
+// The proxy cannot tell a few huge COLUMNS (N/r of them: 1 % of the columns x100 reads 100 whatever
+// N) from a low-rank signal over weak noise (rank 32: N/32), and the two need different plans: the
+// first meets the bar with the cheap gates, the second only with every residual term (rank 32 plus
+// 10 % noise at 1024x2048: 2.9e-3 against 1.4e-4). What separates them is where the mass sits among
+// the columns: colc = N * sum_j c_j^4 / (sum_j c_j^2)^2 over the column norms c_j of the input is
+// N/r for r outlier columns (equal to the proxy) and 1.0 .. 1.5 for anything rotationally spread.
+// The same statistic separates, just below the band, scaled columns (colc = proxy: the low gate
+// suffices) from a spectrum with a gap (colc = 1: near-duplicate rows, 2.4e-3 at 1024x1024 without
+// the wide gate's terms, 4.6e-4 with).
+// k_ns_colstat: one block per 64 columns of a matrix; 8 lanes cover a row piece with 16-byte
+// loads, the 32 row groups walk the M rows (fp64 sums of squares: the pair entries run on
+// unnormalised input) and are added in order through LDS; the block leaves (sum c^2, sum c^4) of
+// its columns (one wavefront's butterfly). A block returns at
+// once unless the matrix's proxy asks for the statistic. k_ns_classify: one lane per matrix adds
+// the partial sums in order and writes the flag every later product reads.
+struct WideRule {
+  double near_lo, lo, hi;    // in units of the proxy N * ||offdiag(A0)||^2; near_lo == lo: no near range
+};
+constexpr double kColcFrac = 0.25, kColcFlat = 1.3;
+__device__ __forceinline__ double cond_proxy(const double *c, int N) {
+  double s = c[0];
+#pragma unroll
+  for (int i = 1; i < kCondParts; ++i) s = s + c[i];
+  return s * (double)N;
+}
+__device__ __host__ __forceinline__ bool wants_colstat(const WideRule &r, double p) {
+  return p >= r.hi || (p > r.near_lo && p <= r.lo);
+}
+struct NsColArgs {
+  int n;
+  int blocks[kMaxGroups];          // colstat: E * parts, classify: E
+  const uint16_t *Xh[kMaxGroups];  // (E, M, N) row-major
+  const double *cond[kMaxGroups];
+  double *part[kMaxGroups];        // (E, parts, 2)
+  int32_t *flag[kMaxGroups];       // (E)
+  int M[kMaxGroups], N[kMaxGroups], parts[kMaxGroups];
+  WideRule rule[kMaxGroups];
+};
+constexpr int kColBlock = 64;       // columns per block of k_ns_colstat
+constexpr int kColRowGroups = kThreads / (kColBlock / 8);
+__global__ void __launch_bounds__(kThreads) k_ns_colstat(NsColArgs a) {
+  __shared__ double colsum[kColRowGroups][kColBlock];
+  int b = (int)blockIdx.x, q = 0;
+  while (q + 1 < a.n && b >= a.blocks[q]) { b -= a.blocks[q]; ++q; }
+  const int e = b / a.parts[q], part = b % a.parts[q];
+  const int M = a.M[q], N = a.N[q];
+  if (!wants_colstat(a.rule[q], cond_proxy(a.cond[q] + (int64_t)e * kCondParts, N))) return;
+  // lane (rg, cg): columns part*64 + 8*cg .. +7 (one 16-byte load per row), rows rg, rg + 32, ...
+  const int cg = (int)threadIdx.x & 7, rg = (int)threadIdx.x >> 3;
+  const uint16_t *src = a.Xh[q] + (int64_t)e * M * N + part * kColBlock + 8 * cg;
+  double c[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+#pragma unroll 8
+  for (int i = rg; i < M; i += kColRowGroups) {
+    const anc_u32x4 w = *(const anc_u32x4 *)(src + (int64_t)i * N);
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const double x0 = (double)__uint_as_float(u[k] << 16), x1 = (double)__uint_as_float(u[k] & 0xFFFF0000u);
+      c[2 * k] = c[2 * k] + x0 * x0;
+      c[2 * k + 1] = c[2 * k + 1] + x1 * x1;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) colsum[rg][8 * cg + k] = c[k];
+  __syncthreads();
+  if (threadIdx.x < kColBlock) {            // one wavefront: the row groups in order, then the butterfly
+    double c2 = colsum[0][threadIdx.x];
+#pragma unroll
+    for (int r = 1; r < kColRowGroups; ++r) c2 = c2 + colsum[r][threadIdx.x];
+    const double s2 = anc_wave_sum_f64(c2), s4 = anc_wave_sum_f64(c2 * c2);
+    if (threadIdx.x == 0) {
+      double *out = a.part[q] + ((int64_t)e * a.parts[q] + part) * 2;
+      out[0] = s2;
+      out[1] = s4;
+    }
+  }
+}
+__global__ void __launch_bounds__(kThreads) k_ns_classify(NsColArgs a) {
+  int t = (int)(blockIdx.x * kThreads + threadIdx.x), q = 0;
+  while (q + 1 < a.n && t >= a.blocks[q]) { t -= a.blocks[q]; ++q; }
+  if (t >= a.blocks[q]) return;
+  const int e = t, N = a.N[q];
+  const WideRule r = a.rule[q];
+  const double p = cond_proxy(a.cond[q] + (int64_t)e * kCondParts, N);
+  bool wide = p > r.lo && p < r.hi;
+  if (!wide && wants_colstat(r, p)) {
+    const double *c = a.part[q] + (int64_t)e * a.parts[q] * 2;
+    double s2 = c[0], s4 = c[1];
+    for (int i = 1; i < a.parts[q]; ++i) { s2 = s2 + c[2 * i]; s4 = s4 + c[2 * i + 1]; }
+    const double colc = s2 > 0.0 ? (double)N * s4 / (s2 * s2) : 1.0;
+    wide = p >= r.hi ? colc < kColcFrac * p : colc < kColcFlat;
+  }
+  a.flag[q][e] = wide ? 1 : 0;
+}
+
 // ------------------------------------------------------------------------- workspace
 struct Carve {
   uint64_t base;
@@ -465,10 +561,11 @@ struct SplitPlan {
   static constexpr int kGateIters = 8;
   float gate_tau[kGateIters];
   unsigned gate_bx;
-  // The wide gate: a matrix whose proxy lies in (wide_lo, wide_hi) adds the residual of X to
-  // A = X X^T from iteration wide_gram_from on and the residuals of X, F and Boff to all three
-  // products from iteration wide_all_from on. wide_hi == 0: no such gate.
-  float wide_lo, wide_hi;
+  // The wide gate: a matrix whose proxy lies in (wide_lo, wide_hi), or outside it with a column
+  // statistic that says so (k_ns_classify), adds the residual of X to A = X X^T from iteration
+  // wide_gram_from on and the residuals of X, F and Boff to all three products from iteration
+  // wide_all_from on. wide_hi == 0: no such gate.
+  float wide_lo, wide_hi, wide_near;   // wide_near: start of the near range below the band (== wide_lo: none)
   int wide_gram_from, wide_all_from;
   bool gated(int k) const { return k >= 0 && k < kGateIters && k < x_from && gate_tau[k] > 0.0f; }
   bool wide() const { return wide_hi > 0.0f; }
@@ -504,7 +601,16 @@ struct SplitPlan {
 //     with the residual of X in A = X X^T from iteration 1 and all residuals in all products of the
 //     last three iterations: 1.0e-4 .. 4.8e-4. Above the band the gates above suffice (8e-4 ..
 //     1.4e-3; only outliers x1000 miss the bar, with or without these terms at 1024x1024).
-constexpr float kTauHard = 2.5f, kTauPlain = 1.3f, kTauWideLo = 2.5f, kTauWideHi = 40.0f;
+//   Outside the band the column statistic decides (k_ns_colstat): above it, a matrix whose column
+//     concentration is below a quarter of its proxy is not an outlier-column matrix but a low-rank
+//     signal over weak noise or a steep spectrum (rank 32 + 10 % noise at 1024x2048 / 1024x3072,
+//     proxy 65 / 97: 2.9e-3 with the gates above, 1.4e-4 with the wide gate's terms; + 1 % noise
+//     5.0e-3 -> 2.5e-4); just below it (kTauWideNear .. kTauWideLo, N < 2M only), a matrix with
+//     flat column norms has a gap in its spectrum (near-duplicate rows, proxy 2.0: 2.4e-3 -> 4.6e-4)
+//     while scaled columns (concentration = proxy) stay with the low gate.
+//   The wide gate's terms start at iteration 1: from iteration 2 the low-rank cases above stay at
+//     1.5e-3 .. 2.7e-3.
+constexpr float kTauHard = 2.5f, kTauPlain = 1.3f, kTauWideLo = 2.5f, kTauWideHi = 40.0f, kTauWideNear = 1.9f;
 SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
   SplitPlan sp{};
   sp.x_from = sp.fb_from = steps;
@@ -531,7 +637,8 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
   if (M >= 1024) {
     if (steps == 5) {                         // the schedule length the wide gate was measured on
       sp.wide_lo = kTauWideLo; sp.wide_hi = kTauWideHi;
-      sp.wide_gram_from = 1; sp.wide_all_from = 2;
+      sp.wide_near = N < 2 * M ? kTauWideNear : kTauWideLo;
+      sp.wide_gram_from = 1; sp.wide_all_from = 1;
     }
     if (N < 2 * M) {
       sp.x_from = steps - 2 < 3 ? steps - 2 : 3;
@@ -573,6 +680,9 @@ struct Plan {
   float *recip;
   float *pow2;           // (E) power-of-two pre-scale of tiny inputs, pair entries
   double *cond;          // (E, kCondParts) conditioning proxy, bf16 modes
+  double *colpart;       // (E, col_parts, 2) column statistic, plans with a wide gate
+  int32_t *wide_flag;    // (E) the wide gate's decision
+  int col_parts;
   // bf16 modes
   uint16_t *Xh[2], *Xl[2];
   float *A32, *dA, *dB;
@@ -610,6 +720,11 @@ Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int ste
     pl.dA = c.take<float>(E * M);
     pl.dB = c.take<float>(E * M);
     pl.cond = c.take<double>(E * kCondParts);
+    if (pl.sp.wide()) {
+      pl.col_parts = (int)(N / kColBlock);
+      pl.colpart = c.take<double>(E * pl.col_parts * 2);
+      pl.wide_flag = c.take<int32_t>(E);
+    }
   }
   pl.bytes = c.off;
   return pl;
@@ -682,9 +797,7 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       const bool wide_g = pl.sp.wide_gram(k);      // implies !split
       const bool wide_a = pl.sp.wide_all(k);       // implies !split_fb
       auto set_wide = [&](NsGemm &w, int nterms_wide) {
-        if (w.cond == nullptr) { w.cond = pl.cond; w.cond_thresh = 1e300; w.nterms_hard = w.nterms; }
-        w.wide_lo = (double)pl.sp.wide_lo / (double)N;
-        w.wide_hi = (double)pl.sp.wide_hi / (double)N;
+        w.wide_flag = pl.wide_flag;
         w.nterms_wide = nterms_wide;
       };
       // A = X X^T
@@ -767,6 +880,28 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       AncProfScope prof(ANC_PROF_NS_FRO, s);
       hipLaunchKernelGGL(k_ns_cond, dim3((unsigned)blocks), dim3(kThreads), 0, s, ca);
       ANC_LAUNCH_CHECK();
+      // the wide gate's decision per matrix, from the proxy and, where it asks, the column norms
+      NsColArgs cs{}, cf{};
+      int cs_blocks = 0, cf_lanes = 0;
+      for (int q = 0; q < n; ++q) {
+        const Plan &pl = cp[q].pl;
+        if (!pl.sp.wide()) continue;
+        const int i = cs.n;
+        cs.Xh[i] = cp[q].inH; cs.cond[i] = pl.cond; cs.part[i] = pl.colpart; cs.flag[i] = pl.wide_flag;
+        cs.M[i] = (int)cp[q].M; cs.N[i] = (int)cp[q].N; cs.parts[i] = pl.col_parts;
+        cs.rule[i] = WideRule{(double)pl.sp.wide_near, (double)pl.sp.wide_lo, (double)pl.sp.wide_hi};
+        cs.blocks[i] = (int)(cp[q].E * pl.col_parts);
+        cs_blocks += cs.blocks[i];
+        ++cs.n;
+      }
+      if (cs.n > 0) {
+        cf = cs;
+        for (int i = 0; i < cf.n; ++i) { cf.blocks[i] = cs.blocks[i] / cs.parts[i]; cf_lanes += cf.blocks[i]; }
+        hipLaunchKernelGGL(k_ns_colstat, dim3((unsigned)cs_blocks), dim3(kThreads), 0, s, cs);
+        ANC_LAUNCH_CHECK();
+        hipLaunchKernelGGL(k_ns_classify, dim3((unsigned)((cf_lanes + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, cf);
+        ANC_LAUNCH_CHECK();
+      }
     }
     {
       AncProfScope prof(ANC_PROF_NS_BMAT, s);
@@ -876,13 +1011,16 @@ extern "C" int anc_ns_hard_info(uint64_t workspace, int64_t E, int64_t M, int64_
   std::vector<double> host((size_t)(E * kCondParts));
   ANC_HIP(hipStreamSynchronize(anc_stream(stream)));
   ANC_HIP(hipMemcpy(host.data(), pl.cond, host.size() * sizeof(double), hipMemcpyDeviceToHost));
+  std::vector<int32_t> flags((size_t)E, 0);
+  if (pl.sp.wide())
+    ANC_HIP(hipMemcpy(flags.data(), pl.wide_flag, flags.size() * sizeof(int32_t), hipMemcpyDeviceToHost));
   const double gram_extra = 2.0 * sym_tile_flops(M, N, force_small) * (double)N;     // two more terms
   const double bx_extra = 2.0 * (double)M * (double)M * (double)N;                   // one more term
   for (int64_t e = 0; e < E; ++e) {
     double t = host[(size_t)(e * kCondParts)];
     for (int i = 1; i < kCondParts; ++i) t = t + host[(size_t)(e * kCondParts + i)];
     bool any = false;
-    const bool in_band = pl.sp.wide() && t > (double)pl.sp.wide_lo / (double)N && t < (double)pl.sp.wide_hi / (double)N;
+    const bool in_band = flags[(size_t)e] != 0;
     for (int k = 0; k < steps; ++k) {
       if (in_band) {                    // the wide gate takes precedence over the others
         const bool sx = k >= pl.sp.x_from;

@@ -85,11 +85,12 @@ struct NsGemm {
                              // nterms_hard terms instead of nterms (its list is a prefix of the hard one)
   double cond_thresh;
   int nterms_hard;
-  // Second gate on the same proxy: a matrix whose sum lies strictly between wide_lo and wide_hi
-  // (a spectrum spread over decades, many moderately large columns) multiplies nterms_wide terms;
-  // 0 = no such gate. It takes precedence over the gate above. With lo_gated set, the residual
-  // outputs Fl / Bl are written for such matrices only (else for every matrix when non-null).
-  double wide_lo, wide_hi;
+  // Second gate: a matrix that k_ns_classify flagged (a spectrum spread over decades, many
+  // moderately large columns, a low-rank signal over weak noise) multiplies nterms_wide terms;
+  // wide_flag null or nterms_wide 0 = no such gate. It takes precedence over the gate above. With
+  // lo_gated set, the residual outputs Fl / Bl are written for such matrices only (else for every
+  // matrix when non-null).
+  const int32_t *wide_flag;  // (E)
   int nterms_wide;
   int lo_gated;
   const float *scale;        // (E) or null. The operands are an unnormalised iterate U and the step
@@ -115,17 +116,14 @@ __device__ __forceinline__ double anc_ns_proxy(const NsGemm &p, int e) {
   for (int i = 1; i < kCondParts; ++i) s = s + c[i];
   return s;
 }
-// Does matrix e lie in the band of the second gate?
+// Did the classification flag matrix e for the second gate?
 __device__ __forceinline__ bool anc_ns_wide(const NsGemm &p, int e) {
-  if (p.cond == nullptr || p.wide_hi <= 0.0) return false;
-  const double s = anc_ns_proxy(p, e);
-  return s > p.wide_lo && s < p.wide_hi;
+  return p.wide_flag != nullptr && p.wide_flag[e] != 0;
 }
 __device__ __forceinline__ int anc_ns_terms(const NsGemm &p, int e) {
+  if (p.nterms_wide > 0 && anc_ns_wide(p, e)) return p.nterms_wide;
   if (p.cond == nullptr) return p.nterms;
-  const double s = anc_ns_proxy(p, e);
-  if (p.nterms_wide > 0 && s > p.wide_lo && s < p.wide_hi) return p.nterms_wide;
-  return s > p.cond_thresh ? p.nterms_hard : p.nterms;
+  return anc_ns_proxy(p, e) > p.cond_thresh ? p.nterms_hard : p.nterms;
 }
 
 // Up to 8 independent problems of the same kind (the same product of different shape groups)

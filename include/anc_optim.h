@@ -456,20 +456,32 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *             nothing: every product carries the residuals of X, F and Boff from iteration 1 on
  *             (from iteration 0 below M = 256), for every matrix, in ANC_NS_BF16 and
  *             ANC_NS_BF16_LATE3 alike (at most 1e-3 on the input classes below, both schedules);
- *   M >= 1024, 5-step chains, every N: strictly between 2.5 and 40 (the wide gate: a spectrum spread
- *             over two or three decades reads 3.6 .. 19, 10 % of the columns x10 reads 8.4; outlier
- *             columns x100, low-rank signals and power-law spectra read 30 .. 440 and do not need
- *             it), the residual of X in A = X X^T from iteration 1 and the residuals of X, F and
- *             Boff in all three products of iterations 2..4 (about 2.3 times the matrix-core work,
- *             for that matrix alone): 1.9e-4 .. 5e-4 instead of 2.5e-3 .. 4.2e-3. It takes precedence
- *             over the gates above.
+ *   M >= 1024, 5-step chains, every N: the wide gate. A matrix takes it if its proxy lies strictly
+ *             between 2.5 and 40 (a spectrum spread over two or three decades reads 3.6 .. 19, 10 %
+ *             of the columns x10 reads 8.4, a rank-128 signal over weak noise 17), or if it lies
+ *             outside and the matrix's column norms say what the proxy cannot: with
+ *             colc = N * sum_j c_j^4 / (sum_j c_j^2)^2 over the column norms c_j of the input,
+ *             proxy >= 40 and colc < proxy / 4 (a low-rank signal over weak noise, a steep
+ *             spectrum: colc about 1, where outlier columns read colc = proxy and keep the cheap
+ *             gates above), or N < 2M, 1.9 < proxy <= 2.5 and colc < 1.3 (a gap in the spectrum,
+ *             e.g. near-duplicate rows; scaled columns read colc = proxy and keep the low gate).
+ *             Such a matrix adds the residuals of X, F and Boff to all three products of iterations
+ *             1..4 (about 2.6 times the matrix-core work, for that matrix alone): condition number
+ *             1e2 .. 1e4 2e-5 .. 8e-5 instead of 2.5e-3 .. 4.2e-3, rank 32 over 10 % / 1 % noise
+ *             2.2e-4 / 3.9e-4 instead of 2.9e-3 / 5.0e-3, near-duplicate rows 6e-5 instead of
+ *             2.4e-3. It takes precedence over the gates above.
  * The decision depends on the matrix alone (fixed-order sums), never on the batch. Accuracy bar of
  * ANC_NS_BF16 with the Polar-Express schedule: 2e-3 relative Frobenius on inputs with independent
  * entries, with row or column outliers up to x100 on 1 % of the rows or columns, with 10 % of the
  * columns x10, with columns scaled over a factor 30, with log-uniform spectra up to condition
- * number 1e3. Not met: outliers x1000 (2.7e-3 .. 4e-3; ANC_NS_BF16_X3). Keller coefficients
- * amplify operand rounding about twice as much (4.5e-3 at 1024x1024): with them the bar is that of
- * ANC_NS_BF16_LATE3, which the host layer selects for that schedule.
+ * number 1e4, with power-law spectra, with low-rank signals over noise down to 1 %, with
+ * near-duplicate rows, with sparse (90 % zeros) and heavy-tailed (Student t, 1.5 degrees of freedom
+ * and up) entries, on shapes up to 4096x8192. Not met: outliers x1000 (2.7e-3 .. 4e-3;
+ * ANC_NS_BF16_X3). Keller coefficients amplify operand rounding about twice as much (4.5e-3 at
+ * 1024x1024): with them the bar is that of ANC_NS_BF16_LATE3, which the host layer selects for
+ * that schedule; it holds on the same classes except a single element of 1000 standard deviations
+ * (3e-5 .. 3e-3 depending on the shape: an isolated singular value that hangs on one rounded
+ * operand element and that Keller's polynomial, unlike the Polar-Express one, does not contract).
  *
  * M and N must be multiples of 128 (the reference's tile alignment,
  * ancora/optim/muon.py:98). workspace must hold anc_ns_workspace_bytes(E,M,N,mode)

@@ -415,6 +415,48 @@ def test_wide_spectrum_inputs_take_the_wide_gate_and_meet_the_bar(gpu, M, N, con
     assert n_gated == 1 and extra > 0
 
 
+@pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 2048), (1024, 3072), (2048, 4096)])
+def test_low_rank_signal_over_weak_noise_is_told_from_outlier_columns(gpu, M, N):
+    """A rank-32 signal over 10 % or 1 % noise and 1 % of the columns x100 read about the same
+    conditioning proxy (N/32 against 100) but need different plans: the column statistic tells
+    them apart. The low-rank matrices take every residual term from iteration 1 on (2.9e-3 and
+    5.0e-3 with the outlier-column gates alone), the outlier-column matrix keeps its cheap gate, and
+    each keeps the bits it has in a batch of its own."""
+    rng = np.random.default_rng(M + 3 * N)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    lr = (rng.standard_normal((M, 32)) @ rng.standard_normal((32, N))).astype(np.float32)
+    X = np.stack([lr + np.float32(0.1) * g, _outlier_cols(rng, M, N), lr + np.float32(0.01) * g, g])
+    got = run_ns(X)
+    n_gated, extra = _hard_count(4, M, N)
+    errs = [rel_fro(got[e], host_ns(X[e], PE_SCHEDULE, 5)) for e in range(4)]
+    print(f"({M},{N}) rank 32 + 10 % noise {errs[0]:.3e}  outlier columns {errs[1]:.3e}  "
+          f"rank 32 + 1 % noise {errs[2]:.3e}  gaussian {errs[3]:.3e}")
+    assert errs[0] < 4e-4 and errs[2] < 6e-4 and errs[1] < TOL_BF16 and errs[3] < TOL_BF16
+    assert n_gated == (2 if (M, N) == (1024, 2048) else 3)      # 1024x2048 has no outlier-column gate
+    per = []
+    for e in range(4):
+        alone = run_ns(X[e:e + 1])
+        per.append(_hard_count(1, M, N)[1])
+        assert bits_equal(alone[0], got[e]), e
+    assert per[0] == per[2] > 2 * per[1] and per[3] == 0 and abs(sum(per) - extra) <= 1e-6 * extra
+
+
+@pytest.mark.parametrize("M,N", [(1024, 1024), (1536, 1536), (1024, 1536)])
+def test_near_duplicate_rows_take_the_wide_gate(gpu, M, N):
+    """Half of the rows repeat the other half up to 1 % noise: a spectrum with a gap, proxy 1 + N/M
+    (just below the band for N < 2M) and flat column norms. 2.2e-3 .. 2.4e-3 with the low gate
+    alone; a matrix with scaled columns and the same proxy stays with the low gate."""
+    rng = np.random.default_rng(M + N)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    d = g.copy()
+    d[M // 2:] = d[:M - M // 2] + np.float32(0.01) * g[M // 2:]
+    sc = g * np.exp(0.45 * rng.standard_normal(N)).astype(np.float32)
+    got = run_ns(np.stack([d, sc]))
+    e_dup, e_sc = rel_fro(got[0], host_ns(d, PE_SCHEDULE, 5)), rel_fro(got[1], host_ns(sc, PE_SCHEDULE, 5))
+    print(f"({M},{N}) near-duplicate rows {e_dup:.3e}  log-normal columns {e_sc:.3e}")
+    assert e_dup < 2e-4 and 4e-4 < e_sc < 1.6e-3
+
+
 @pytest.mark.parametrize("M,N", [(1024, 1024), (2048, 2048), (1024, 1536)])
 def test_column_scaled_square_matrices_between_the_gates(gpu, M, N):
     """Proxy between the low gate (1.3) and the wide gate's band (2.5): columns scaled over 0.03..3
