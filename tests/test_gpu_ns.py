@@ -439,6 +439,10 @@ def test_low_rank_signal_over_weak_noise_is_told_from_outlier_columns(gpu, M, N)
         per.append(_hard_count(1, M, N)[1])
         assert bits_equal(alone[0], got[e]), e
     assert per[0] == per[2] > 2 * per[1] and per[3] == 0 and abs(sum(per) - extra) <= 1e-6 * extra
+    if M == 1024:      # the 128x128-tile kernel reads the same flags
+        small = run_ns(X[:2], mode="bf16_tile128")
+        assert rel_fro(small[0], got[0]) < 1e-4 and rel_fro(small[1], got[1]) < 5e-4
+        assert _hard_count(2, M, N, "bf16_tile128")[0] == n_gated - 1
 
 
 @pytest.mark.parametrize("M,N", [(1024, 1024), (1536, 1536), (1024, 1536)])
