@@ -628,14 +628,18 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
     // Gaussian 3.7e-3 -> 6e-5, 1024x3072 2.8e-3 -> 3e-5, condition number 1e3 2.5e-4 .. 3.2e-4,
     // 1 % of the columns x100 3.6e-4 .. 7.9e-4; residuals in the last two iterations only leave
     // 2.2e-3 at 1024x1024. M < 1024 runs a heavier plan in either mode (below).
-    sp.x_from = sp.fb_from = steps > 3 ? steps - 3 : 0;
+    // From iteration 2 on whatever the chain's length (Keller's iterates do not settle, so a longer
+    // chain keeps adding first-order roundings: with the last three iterations only, 6 steps gave
+    // 3.1e-3 and 8 steps 8.9e-3 at 1024x1024), and the last three of a shorter one.
+    sp.x_from = sp.fb_from = steps >= 5 ? 2 : (steps > 3 ? steps - 3 : 0);
     return sp;
   }
   if (mode != ANC_NS_BF16 && mode != ANC_NS_BF16_LATE3) return sp;
   // The first iterations are insensitive (the singular values are still far below 1, so
   // B X is a small correction to a X); residuals start at a fixed iteration index.
   if (M >= 1024) {
-    if (steps == 5) {                         // the schedule length the wide gate was measured on
+    if (steps >= 2) {                         // terms from iteration 1 to the end, whatever the length
+                                              // (cond 1e3 without: 6 steps 4.4e-3 .. 7e-3, 8 steps 6e-3 .. 1.8e-2)
       sp.wide_lo = kTauWideLo; sp.wide_hi = kTauWideHi;
       sp.wide_near = N < 2 * M ? kTauWideNear : kTauWideLo;
       sp.wide_gram_from = 1; sp.wide_all_from = 1;
@@ -654,6 +658,9 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
       // of 2M <= N < 3M does not (1024x2560 1.8e-3, 1536x3072 2.1e-3, 2048x4096 2.2e-3, 4096x8192
       // 2.3e-3 without).
       sp.gate_tau[2] = kTauHard;
+      // a chain shorter than the 5 steps this was measured on ends before iteration 2's term has
+      // paid off (3 steps at 1024x3072: 2.3e-3, 2 steps 2.7e-3): iteration 1 as well
+      if (steps < 5) sp.gate_tau[1] = kTauHard;
     }
   } else {
     // Small matrices average fewer rounding errors per element and cost next to nothing: all

@@ -428,8 +428,9 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *                     accumulation terms per product in every iteration): about 1e-5 from the
  *                     fp32 chain on every input tried, ill-conditioned ones included, for three
  *                     times the matrix-core work of ANC_NS_BF16_FAST.
- *   ANC_NS_BF16_LATE3 ANC_NS_BF16 with the residuals of both operands in all three products of the
- *                     last three iterations, for every matrix and without gates, for M >= 1024
+ *   ANC_NS_BF16_LATE3 ANC_NS_BF16 with the residuals of both operands in all three products from
+ *                     iteration 2 on (the last three of a 5-step chain; the last three of a
+ *                     shorter one), for every matrix and without gates, for M >= 1024
  *                     (M < 1024 runs a heavier plan in either mode, see below): about 2.2 times the
  *                     matrix-core work of ANC_NS_BF16_FAST. For coefficients that do not drive the
  *                     singular values to 1: Keller's quintic (ancora/kernels/muon_ns.py:21) leaves
@@ -444,7 +445,7 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  * matrix add the residual of X (three accumulation terms in A = X X^T, two in X = a X + B X)
  * according to it:
  *   N >= 3M:  above 2.5, A = X X^T of iteration 2 (1 % of the columns x100 at 1024x3072: 1.15e-3
- *             instead of 2.2e-3);
+ *             instead of 2.2e-3), and of iteration 1 in chains shorter than 5 steps;
  *   N < 2M:   above 2.5, A = X X^T of iterations 1 and 2 (1024x1024: 8e-4 instead of 3.8e-3); above
  *             1.3, both X-products of iterations 2 and 3 (5-step chains; every matrix has them in
  *             iteration 4): a matrix with independent entries or outlier rows does without
@@ -456,7 +457,7 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *             nothing: every product carries the residuals of X, F and Boff from iteration 1 on
  *             (from iteration 0 below M = 256), for every matrix, in ANC_NS_BF16 and
  *             ANC_NS_BF16_LATE3 alike (at most 1e-3 on the input classes below, both schedules);
- *   M >= 1024, 5-step chains, every N: the wide gate. A matrix takes it if its proxy lies strictly
+ *   M >= 1024, every N, chains of any length: the wide gate. A matrix takes it if its proxy lies strictly
  *             between 2.5 and 40 (a spectrum spread over two or three decades reads 3.6 .. 19, 10 %
  *             of the columns x10 reads 8.4, a rank-128 signal over weak noise 17), or if it lies
  *             outside and the matrix's column norms say what the proxy cannot: with
@@ -465,8 +466,8 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *             spectrum: colc about 1, where outlier columns read colc = proxy and keep the cheap
  *             gates above), or N < 2M, 1.9 < proxy <= 2.5 and colc < 1.3 (a gap in the spectrum,
  *             e.g. near-duplicate rows; scaled columns read colc = proxy and keep the low gate).
- *             Such a matrix adds the residuals of X, F and Boff to all three products of iterations
- *             1..4 (about 2.6 times the matrix-core work, for that matrix alone): condition number
+ *             Such a matrix adds the residuals of X, F and Boff to all three products from iteration
+ *             1 on (about 2.6 times the matrix-core work, for that matrix alone): condition number
  *             1e2 .. 1e4 2e-5 .. 8e-5 instead of 2.5e-3 .. 4.2e-3, rank 32 over 10 % / 1 % noise
  *             2.2e-4 / 3.9e-4 instead of 2.9e-3 / 5.0e-3, near-duplicate rows 6e-5 instead of
  *             2.4e-3. It takes precedence over the gates above.

@@ -415,6 +415,24 @@ def test_wide_spectrum_inputs_take_the_wide_gate_and_meet_the_bar(gpu, M, N, con
     assert n_gated == 1 and extra > 0
 
 
+@pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 3072)])
+@pytest.mark.parametrize("sched", ["pe", "keller"])
+def test_other_chain_lengths_within_the_bar(gpu, M, N, sched):
+    """3, 4, 6 and 8 iterations (the schedule's last triple repeats beyond its length). The wide
+    gate's terms run from iteration 1 to the end of any chain and Keller's plan from iteration 2
+    to the end: with both tied to the 5-step chain, 8 steps reached 1.8e-2 on a spectrum over three
+    decades (Polar Express) and 8.9e-3 on independent entries (Keller)."""
+    rng = np.random.default_rng(M + N)
+    schedule = PE_SCHEDULE if sched == "pe" else None
+    X = np.stack([rng.standard_normal((M, N)).astype(np.float32), _outlier_cols(rng, M, N),
+                  _log_spectrum(rng, M, N, 1e3)])
+    for steps in (3, 4, 6, 8):
+        got = run_ns(X, steps=steps, schedule=schedule)
+        errs = [rel_fro(got[e], host_ns(X[e], schedule, steps)) for e in range(3)]
+        print(f"({M},{N}) {sched} {steps} steps: gaussian {errs[0]:.3e}  outlier columns {errs[1]:.3e}  cond 1e3 {errs[2]:.3e}")
+        assert max(errs) < TOL_BF16, steps
+
+
 @pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 2048), (1024, 3072), (2048, 4096)])
 def test_low_rank_signal_over_weak_noise_is_told_from_outlier_columns(gpu, M, N):
     """A rank-32 signal over 10 % or 1 % noise and 1 % of the columns x100 read about the same
