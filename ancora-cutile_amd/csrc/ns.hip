@@ -447,8 +447,8 @@ __global__ void __launch_bounds__(kThreads) k_ns_cond(NsCondArgs a) {
 // The same statistic separates, just below the band, scaled columns (colc = proxy: the low gate
 // suffices) from a spectrum with a gap (colc = 1: near-duplicate rows, 2.4e-3 at 1024x1024 without
 // the wide gate's terms, 4.6e-4 with).
-// k_ns_colstat: one block per 64 columns of a matrix; 8 lanes cover a row piece with 16-byte
-// loads, the 32 row groups walk the M rows (fp64 sums of squares: the pair entries run on
+// k_ns_colstat: one block per 64 columns of a matrix; 8 lanes cover a 128-byte row piece with
+// 16-byte loads, the 32 row groups walk the M rows (fp64 sums of squares: the pair entries run on
 // unnormalised input) and are added in order through LDS; the block leaves (sum c^2, sum c^4) of
 // its columns (one wavefront's butterfly). A block returns at
 // once unless the matrix's proxy asks for the statistic. k_ns_classify: one lane per matrix adds
@@ -476,45 +476,56 @@ struct NsColArgs {
   int M[kMaxGroups], N[kMaxGroups], parts[kMaxGroups];
   WideRule rule[kMaxGroups];
 };
-constexpr int kColBlock = 64;       // columns per block of k_ns_colstat
-constexpr int kColRowGroups = kThreads / (kColBlock / 8);
+constexpr int kColBlock = 64;       // columns per block of k_ns_colstat (measured: 64 -> 92 us, 256 -> 104 us
+                                    // per Qwen3-0.6B step: more blocks beat longer row pieces)
+constexpr int kColLanes = kColBlock / 8, kColRowGroups = kThreads / kColLanes;
 __global__ void __launch_bounds__(kThreads) k_ns_colstat(NsColArgs a) {
   __shared__ double colsum[kColRowGroups][kColBlock];
+  __shared__ double wave_sum[2][kColBlock / 64];
   int b = (int)blockIdx.x, q = 0;
   while (q + 1 < a.n && b >= a.blocks[q]) { b -= a.blocks[q]; ++q; }
   const int e = b / a.parts[q], part = b % a.parts[q];
   const int M = a.M[q], N = a.N[q];
   if (!wants_colstat(a.rule[q], cond_proxy(a.cond[q] + (int64_t)e * kCondParts, N))) return;
   // lane (rg, cg): columns part*64 + 8*cg .. +7 (one 16-byte load per row), rows rg, rg + 32, ...
-  const int cg = (int)threadIdx.x & 7, rg = (int)threadIdx.x >> 3;
-  const uint16_t *src = a.Xh[q] + (int64_t)e * M * N + part * kColBlock + 8 * cg;
+  const int cg = (int)threadIdx.x % kColLanes, rg = (int)threadIdx.x / kColLanes;
+  const int j = part * kColBlock + 8 * cg;
   double c[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+  if (j < N) {
+    const uint16_t *src = a.Xh[q] + (int64_t)e * M * N + j;
 #pragma unroll 8
-  for (int i = rg; i < M; i += kColRowGroups) {
-    const anc_u32x4 w = *(const anc_u32x4 *)(src + (int64_t)i * N);
-    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+    for (int i = rg; i < M; i += kColRowGroups) {
+      const anc_u32x4 w = *(const anc_u32x4 *)(src + (int64_t)i * N);
+      const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const double x0 = (double)__uint_as_float(u[k] << 16), x1 = (double)__uint_as_float(u[k] & 0xFFFF0000u);
-      c[2 * k] = c[2 * k] + x0 * x0;
-      c[2 * k + 1] = c[2 * k + 1] + x1 * x1;
+      for (int k = 0; k < 4; ++k) {
+        const double x0 = (double)__uint_as_float(u[k] << 16), x1 = (double)__uint_as_float(u[k] & 0xFFFF0000u);
+        c[2 * k] = c[2 * k] + x0 * x0;
+        c[2 * k + 1] = c[2 * k + 1] + x1 * x1;
+      }
     }
   }
 #pragma unroll
   for (int k = 0; k < 8; ++k) colsum[rg][8 * cg + k] = c[k];
   __syncthreads();
-  if (threadIdx.x < kColBlock) {            // one wavefront: the row groups in order, then the butterfly
+  if (threadIdx.x < kColBlock) {               // one lane per column: the row groups in order
     double c2 = colsum[0][threadIdx.x];
 #pragma unroll
     for (int r = 1; r < kColRowGroups; ++r) c2 = c2 + colsum[r][threadIdx.x];
     const double s2 = anc_wave_sum_f64(c2), s4 = anc_wave_sum_f64(c2 * c2);
-    if (threadIdx.x == 0) {
-      double *out = a.part[q] + ((int64_t)e * a.parts[q] + part) * 2;
-      out[0] = s2;
-      out[1] = s4;
-    }
+    if ((threadIdx.x & 63) == 0) { wave_sum[0][threadIdx.x >> 6] = s2; wave_sum[1][threadIdx.x >> 6] = s4; }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double t2 = wave_sum[0][0], t4 = wave_sum[1][0];
+#pragma unroll
+    for (int w = 1; w < kColBlock / 64; ++w) { t2 = t2 + wave_sum[0][w]; t4 = t4 + wave_sum[1][w]; }
+    double *out = a.part[q] + ((int64_t)e * a.parts[q] + part) * 2;
+    out[0] = t2;
+    out[1] = t4;
   }
 }
+static_assert(kColBlock % 64 == 0 && kColBlock <= kThreads, "k_ns_colstat: whole wavefronts of one lane per column in the final sum");
 __global__ void __launch_bounds__(kThreads) k_ns_classify(NsColArgs a) {
   int t = (int)(blockIdx.x * kThreads + threadIdx.x), q = 0;
   while (q + 1 < a.n && t >= a.blocks[q]) { t -= a.blocks[q]; ++q; }
@@ -728,7 +739,7 @@ Plan make_plan(uint64_t base, int64_t E, int64_t M, int64_t N, int mode, int ste
     pl.dB = c.take<float>(E * M);
     pl.cond = c.take<double>(E * kCondParts);
     if (pl.sp.wide()) {
-      pl.col_parts = (int)(N / kColBlock);
+      pl.col_parts = (int)((N + kColBlock - 1) / kColBlock);
       pl.colpart = c.take<double>(E * pl.col_parts * 2);
       pl.wide_flag = c.take<int32_t>(E);
     }

@@ -21,8 +21,8 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
 
     python3 -m ancora_cutile_amd.prof_target mfma [launches]            matrix-pipe reference (anc_mfma_rate):
                                       TFLOP/s of the register-only matrix-instruction loop on zero,
-                                      constant and random operands, with the shader clock rocm-smi
-                                      reports while each runs
+                                      constant and random operands, with the shader clock and package
+                                      power sysfs reports while each runs
 
 Each target allocates its operands, runs the kernel(s) `calls` times on the null stream and
 synchronises; nothing is checked here (parity lives in tests/).
@@ -57,30 +57,25 @@ def main(argv):
             _lib.profile_enable(False)
             print("  ".join(f"{k}={v[0]:.3f}ms/{v[1]}" for k, v in pr.items() if v[1]))
     elif what == "mfma":
-        import re
-        import subprocess
         import threading
         import time
         launches = int(argv[1]) if len(argv) > 1 else 12
         sink = DevBuf.empty((1024,), np.float32)
 
-        def sclk():
-            try:
-                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
-            except Exception:
-                return None
-            m = re.search(r"sclk clock level:\s*\S+\s*\((\d+)Mhz\)", out)
-            return int(m.group(1)) if m else None
+        from .sysfs import sclk_mhz as sclk, power_w
 
         for name, values in (("zeros", 0), ("constant", 1), ("random", 2), ("zeros", 0), ("random", 2)):
-            samples, stop = [], threading.Event()
+            samples, watts, stop = [], [], threading.Event()
 
             def poll():
                 time.sleep(0.5)
                 while not stop.is_set():
-                    v = sclk()
+                    v, w = sclk(), power_w()
                     if v:
                         samples.append(v)
+                    if w:
+                        watts.append(w)
+                    time.sleep(0.02)
 
             th = threading.Thread(target=poll, daemon=True)
             th.start()
@@ -96,8 +91,10 @@ def main(argv):
             stop.set()
             th.join(timeout=15)
             busy = sorted(v for v in samples if v > 300)
+            med = lambda xs: xs[len(xs) // 2] if xs else None
             print(f"{name:9s} first launch {rates[0]:7.1f}  last {rates[-1]:7.1f} TFLOP/s over {launches} launches; "
-                  f"sclk while running: {busy if busy else 'n/a'} MHz", flush=True)
+                  f"sclk while running: median {med(busy)} MHz (min {busy[0] if busy else None}, max {busy[-1] if busy else None}, "
+                  f"{len(busy)} samples); package power median {med(sorted(watts))} W", flush=True)
     elif what == "adamw":
         n = int(argv[1]) // 64 * 64
         calls = int(argv[2]) if len(argv) > 2 else 3

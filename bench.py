@@ -60,30 +60,29 @@ def synth(shapes, seed=0):
 
 
 def read_sclk_mhz():
-    """Current shader clock in MHz from `rocm-smi --showclocks` (read-only), or None."""
-    import re
-    import subprocess
-    try:
-        out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
-    except Exception:
-        return None
-    m = re.search(r"sclk clock level:\s*\S+\s*\((\d+)Mhz\)", out)
-    return int(m.group(1)) if m else None
+    """Current shader clock in MHz from sysfs (read-only, no child process), or None."""
+    from ancora_cutile_amd.sysfs import sclk_mhz
+    return sclk_mhz()
 
 
 def sustained_sclk(run_steps, seconds=1.5):
-    """Median shader clock while `run_steps(n)` keeps the GPU busy with optimizer steps: a sampler
-    thread polls rocm-smi, the main thread keeps launching (launches are asynchronous and the
-    library calls drop the GIL). Outside the timed region. None if rocm-smi gives nothing."""
+    """(median shader clock in MHz, median package power in W) while `run_steps(n)` keeps the GPU
+    busy with optimizer steps: a sampler thread polls the board's sysfs entries, the main thread
+    keeps launching (launches are asynchronous and the library calls drop the GIL). Outside the
+    timed region. None where sysfs gives nothing."""
     import threading
-    samples, stop = [], threading.Event()
+    from ancora_cutile_amd.sysfs import power_w
+    clocks, watts, stop = [], [], threading.Event()
 
     def poll():
         time.sleep(0.4)                      # let the clock settle under load
         while not stop.is_set():
-            v = read_sclk_mhz()
+            v, w = read_sclk_mhz(), power_w()
             if v:
-                samples.append(v)
+                clocks.append(v)
+            if w:
+                watts.append(w)
+            time.sleep(0.01)
 
     th = threading.Thread(target=poll, daemon=True)
     th.start()
@@ -92,8 +91,10 @@ def sustained_sclk(run_steps, seconds=1.5):
         run_steps(5)
     stop.set()
     th.join(timeout=15)
-    samples = sorted(v for v in samples if v > 300)   # drop samples taken while the GPU idled
-    return samples[len(samples) // 2] if samples else None
+    clocks = sorted(v for v in clocks if v > 300)   # drop samples taken while the GPU idled
+    watts = sorted(watts)
+    return (clocks[len(clocks) // 2] if clocks else None,
+            round(watts[len(watts) // 2], 1) if watts else None)
 
 
 def mfma_reference(_lib, DevBuf):
@@ -569,7 +570,7 @@ def main():
             opt.step(gdev, 0)
         _lib.stream_sync(0)
 
-    sclk = None if args.no_clock else sustained_sclk(run_steps)
+    sclk, watts = (None, None) if args.no_clock else sustained_sclk(run_steps)
     mfma_ref = {} if args.no_clock else mfma_reference(_lib, DevBuf)
 
     # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
@@ -676,6 +677,7 @@ def main():
         "streams": "serial" if args.serial else "one: the Newton-Schulz chains of all shape groups advance together (grouped launches)",
         "copy_kernel_gbps": round(copy_gbps, 1),
         "sustained_sclk_mhz": sclk,
+        "sustained_power_w": watts,
         "mfma_register_loop_tflops": mfma_ref,
         "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
         "device": {"name": info["name"] or info["arch"].split(":")[0], "arch": info["arch"], "cus": info["cu_count"],
