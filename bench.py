@@ -97,6 +97,83 @@ def sustained_sclk(run_steps, seconds=1.5):
             round(watts[len(watts) // 2], 1) if watts else None)
 
 
+def _median_power(fn, seconds, settle=0.5):
+    """(median package power in W, ms per call) while `fn()` is called back to back for `seconds`."""
+    import threading
+    from ancora_cutile_amd import _lib
+    from ancora_cutile_amd.sysfs import power_w
+    watts, stop = [], threading.Event()
+
+    def poll():
+        time.sleep(settle)
+        while not stop.is_set():
+            w = power_w()
+            if w:
+                watts.append(w)
+            time.sleep(0.01)
+
+    th = threading.Thread(target=poll, daemon=True)
+    th.start()
+    e0, e1 = _lib.Event(), _lib.Event()
+    n, t0 = 0, time.perf_counter()
+    e0.record(0)
+    while time.perf_counter() - t0 < seconds:
+        fn()
+        n += 1
+        if n % 4 == 0:
+            _lib.stream_sync(0)
+    e1.record(0)
+    e1.sync()
+    stop.set()
+    th.join(timeout=5)
+    watts.sort()
+    return (watts[len(watts) // 2] if watts else None), e0.elapsed_ms(e1) / max(1, n)
+
+
+def power_reference(_lib, DevBuf):
+    """Energy prices of the board's two resources, from package power (sysfs) while one of them runs
+    alone: pJ per HBM byte from the 1 GiB copy kernel on random data, pJ per matrix-core FLOP from
+    the register-only loop on random operands, each above the idle power. None without sysfs."""
+    import ctypes
+    _lib.stream_sync(0)
+    idle, _ = _median_power(lambda: time.sleep(0.02), 0.8, settle=0.3)
+    if idle is None:
+        return None
+    n = 1 << 28
+    src, dst = DevBuf.empty((n,), np.float32), DevBuf.empty((n,), np.float32)
+    seed = DevBuf(np.random.default_rng(11).standard_normal(1 << 24).astype(np.float32))
+    for i in range(n >> 24):
+        _lib.api.anc_copy_kernel(src.ptr + (i << 26), seed.ptr, 1 << 26, 0)
+    copy_w, copy_ms = _median_power(lambda: _lib.api.anc_copy_kernel(dst.ptr, src.ptr, 1 << 30, 0), 1.5)
+    for b in (src, dst, seed):
+        b.free()
+    sink, fl = DevBuf.empty((1024,), np.float32), ctypes.c_double()
+    mfma_w, mfma_ms = _median_power(lambda: _lib.api.anc_mfma_rate(2, 100000, sink.ptr, ctypes.byref(fl), 0), 1.5)
+    sink.free()
+    copy_bps, mfma_fps = 2.0 * (1 << 30) / (copy_ms * 1e-3), fl.value / (mfma_ms * 1e-3)
+    return {"idle_w": idle, "copy_w": copy_w, "copy_tbps": round(copy_bps / 1e12, 2),
+            "pj_per_hbm_byte": round((copy_w - idle) / copy_bps * 1e12, 1),
+            "mfma_random_w": mfma_w, "mfma_random_tflops": round(mfma_fps / 1e12, 1),
+            "pj_per_flop": round((mfma_w - idle) / mfma_fps * 1e12, 3)}
+
+
+def power_model(ref, step_w, traffic, launches, executed, gemm_ms):
+    """The GEMM launches of a step priced in energy: HBM bytes at the copy kernel's pJ per byte plus
+    executed FLOPs at the register loop's pJ per FLOP, and the time that energy takes at the power
+    the step draws above idle. `frac` = that time / the measured time: how much of the launches'
+    time the two resources' energy alone accounts for under the package limit."""
+    if not ref or not step_w or not traffic or not gemm_ms:
+        return None
+    joule = traffic * launches * ref["pj_per_hbm_byte"] * 1e-12 + executed * ref["pj_per_flop"] * 1e-12
+    ms_min = joule / (step_w - ref["idle_w"]) * 1e3
+    return {**ref, "step_w": step_w, "gemm_joule_per_step": round(joule, 2),
+            "gemm_ms_at_step_power": round(ms_min, 3), "gemm_ms_measured": round(gemm_ms, 3),
+            "frac": round(ms_min / gemm_ms, 4),
+            "note": "energy balance, context only: roofline.traffic x launches at the copy kernel's energy per byte "
+                    "+ executed FLOPs at the register loop's energy per FLOP (random operands), divided by the "
+                    "power the step draws above idle (idle_w is read right after load, clocks still up)"}
+
+
 def mfma_reference(_lib, DevBuf):
     """TFLOP/s of the register-only matrix-instruction loop (anc_mfma_rate) on zero and on random
     operands: what the matrix pipe sustains on this board without any memory traffic."""
@@ -572,6 +649,7 @@ def main():
 
     sclk, watts = (None, None) if args.no_clock else sustained_sclk(run_steps)
     mfma_ref = {} if args.no_clock else mfma_reference(_lib, DevBuf)
+    power_ref = None if args.no_clock else power_reference(_lib, DevBuf)
 
     # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
     # last X = a X + B X) also reads and writes the weights
@@ -679,6 +757,7 @@ def main():
         "sustained_sclk_mhz": sclk,
         "sustained_power_w": watts,
         "mfma_register_loop_tflops": mfma_ref,
+        "power_model": power_model(power_ref, watts, traffic, gemm_launches, executed, gemm_ms),
         "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
         "device": {"name": info["name"] or info["arch"].split(":")[0], "arch": info["arch"], "cus": info["cu_count"],
                    "clock_khz": info["clock_khz"]},
