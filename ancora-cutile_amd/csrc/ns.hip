@@ -609,8 +609,8 @@ struct SplitPlan {
 //     against 1 % of the columns x100 100, x1000 102, a rank-32 signal over noise 32 / 95, a
 //     power-law spectrum 146 / 437. In the band the plan above leaves 2.5e-3 .. 4.2e-3 (every operand
 //     rounding of the later iterations counts: the small singular values are still far from 1);
-//     with the residual of X in A = X X^T from iteration 1 and all residuals in all products of the
-//     last three iterations: 1.0e-4 .. 4.8e-4. Above the band the gates above suffice (8e-4 ..
+//     with all residuals in all products from iteration 2 on 1.0e-4 .. 4.8e-4, from iteration 1 on
+//     (what runs) 2e-5 .. 8e-5. Above the band the gates above suffice for outlier columns (8e-4 ..
 //     1.4e-3; only outliers x1000 miss the bar, with or without these terms at 1024x1024).
 //   Outside the band the column statistic decides (k_ns_colstat): above it, a matrix whose column
 //     concentration is below a quarter of its proxy is not an outlier-column matrix but a low-rank
@@ -632,8 +632,8 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
     return sp;
   }
   if (mode == ANC_NS_BF16_LATE3 && M >= 1024) {
-    // residuals of X, F and Boff in all three products of the last three iterations, for every
-    // matrix, no gates: what the wide gate gives the matrices it selects. For coefficients that do
+    // residuals of X, F and Boff in all three products from iteration 2 on (the last three of a
+    // 5-step chain), for every matrix, no gates. For coefficients that do
     // not drive the singular values to 1 (Keller's quintic leaves them in 0.7 .. 1.2, so
     // offdiag(A) never becomes small and every operand rounding stays first-order): 1024x1024
     // Gaussian 3.7e-3 -> 6e-5, 1024x3072 2.8e-3 -> 3e-5, condition number 1e3 2.5e-4 .. 3.2e-4,
@@ -663,7 +663,7 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
         sp.gate_bx = (1u << 2) | (1u << 3);
         sp.x_from = 4;
       }
-    } else if (N >= 3 * M || N > 2 * M || M > 1024) {
+    } else if (N > 2 * M || M > 1024) {
       // iteration 2 alone. Not at 1024x2048 itself: there the outlier-column case meets the bar
       // without (1.57e-3 .. 1.61e-3 over seeds) and the term would cost its matrices 6 %; the rest
       // of 2M <= N < 3M does not (1024x2560 1.8e-3, 1536x3072 2.1e-3, 2048x4096 2.2e-3, 4096x8192
@@ -946,8 +946,8 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
 extern "C" int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode) {
   mode &= ~ANC_NS_TILE128;
   if (check_shape(E, M, N, mode, "anc_ns_workspace_bytes")) return -1;
-  // sized for any step count: with steps >= 3 every optional buffer of the mode's plan is present;
-  // the 5-step schedule adds the residual buffers of the wide gate
+  // sized for any step count: with steps >= 3 every optional buffer of the mode's plan is present
+  // (the longer of a long and a 5-step chain's plans, should the two ever differ)
   const int64_t a = make_plan(0, E, M, N, mode, 64).bytes, b = make_plan(0, E, M, N, mode, 5).bytes;
   return a > b ? a : b;
 }
