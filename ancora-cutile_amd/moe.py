@@ -9,8 +9,6 @@ flat tensor goes through AdamW. The router stays on AdamW (wd = 0, :603-604). Th
 copies the backward reads (`_transpose_e`, :370-377, 593-597) are refreshed by the Muon update
 kernel in the same pass; the AdamW variant runs the transpose kernel after the step.
 """
-import ctypes
-
 import numpy as np
 
 from . import _lib

@@ -312,7 +312,7 @@ def cpu_baseline(shapes, lr_adam=3e-4):
 
 def side_workload(args):
     """Configs 3 and 5 as stand-alone timings (same JSON shape, their own metric names)."""
-    from ancora_cutile_amd import DevBuf, StepGuard, AdamW, PE_SCHEDULE, _lib
+    from ancora_cutile_amd import DevBuf, StepGuard, PE_SCHEDULE, _lib
     from ancora_cutile_amd.muon_ns import ns_batched, ns_flops
     _lib.init(0)
     info = _lib.device_info()

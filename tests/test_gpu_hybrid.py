@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 from oracle.adamw_ref import AdamWRef
-from oracle.muon_ref import MuonRef, PE_SCHEDULE, default_is_muon as ref_is_muon
+from oracle.muon_ref import MuonRef, PE_SCHEDULE
 from oracle.bf16_ref import bf16_rne_bits, bits_to_f32
 from util import max_ulp, rel_fro, bits_equal, bf16_grad
 

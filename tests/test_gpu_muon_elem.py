@@ -5,7 +5,7 @@ import pytest
 
 from oracle.bf16_ref import bf16_rne_bits, bf16_sr_bits, bits_to_f32
 from oracle.muon_ref import muon_momentum, muon_update, shape_scale
-from util import max_ulp, bits_equal, bf16_grad
+from util import bits_equal, bf16_grad
 
 pytestmark = pytest.mark.gpu
 

@@ -2,7 +2,6 @@
 GPU: format constants, an independent integer-bit formulation of the rounding checked over every
 bf16 input and every reachable block scale, special cases, and the error bound of the format."""
 import numpy as np
-import pytest
 
 from oracle.quant_ref import e4m3_table, e4m3_rne, quant_mxfp8_w, dequant_mxfp8_w, B
 from oracle.bf16_ref import bf16_rne_bits, bits_to_f32
