@@ -442,8 +442,9 @@ __global__ void __launch_bounds__(kThreads) k_ns_cond(NsCondArgs a) {
 // N) from a low-rank signal over weak noise (rank 32: N/32), and the two need different plans: the
 // first meets the bar with the cheap gates, the second only with every residual term (rank 32 plus
 // 10 % noise at 1024x2048: 2.9e-3 against 1.4e-4). What separates them is where the mass sits among
-// the columns: colc = N * sum_j c_j^4 / (sum_j c_j^2)^2 over the column norms c_j of the input is
-// N/r for r outlier columns (equal to the proxy) and 1.0 .. 1.5 for anything rotationally spread.
+// the columns: colc = N * sum_j c_j^4 / (sum_j c_j^2)^2 over the column norms c_j of the input
+// (taken over every fourth row) is N/r for r outlier columns (equal to the proxy) and 1.0 .. 1.5
+// for anything rotationally spread.
 // The same statistic separates, just below the band, scaled columns (colc = proxy: the low gate
 // suffices) from a spectrum with a gap (colc = 1: near-duplicate rows, 2.4e-3 at 1024x1024 without
 // the wide gate's terms, 4.6e-4 with).
@@ -479,6 +480,9 @@ struct NsColArgs {
 constexpr int kColBlock = 64;       // columns per block of k_ns_colstat (measured: 64 -> 92 us, 256 -> 104 us
                                     // per Qwen3-0.6B step: more blocks beat longer row pieces)
 constexpr int kColLanes = kColBlock / 8, kColRowGroups = kThreads / kColLanes;
+constexpr int kColRowStep = 4;      // every fourth row: the thresholds are coarse (a quarter of the proxy; 1.3
+                                    // against 1.0 and 1.9+), a quarter of the rows places a matrix as well as all
+                                    // of them (flat columns read 1 + 8/M more) and costs a quarter of the bytes
 __global__ void __launch_bounds__(kThreads) k_ns_colstat(NsColArgs a) {
   __shared__ double colsum[kColRowGroups][kColBlock];
   __shared__ double wave_sum[2][kColBlock / 64];
@@ -487,14 +491,14 @@ __global__ void __launch_bounds__(kThreads) k_ns_colstat(NsColArgs a) {
   const int e = b / a.parts[q], part = b % a.parts[q];
   const int M = a.M[q], N = a.N[q];
   if (!wants_colstat(a.rule[q], cond_proxy(a.cond[q] + (int64_t)e * kCondParts, N))) return;
-  // lane (rg, cg): columns part*64 + 8*cg .. +7 (one 16-byte load per row), rows rg, rg + 32, ...
+  // lane (rg, cg): columns part*64 + 8*cg .. +7 (one 16-byte load per row), rows 4 rg, 4 (rg + 32), ...
   const int cg = (int)threadIdx.x % kColLanes, rg = (int)threadIdx.x / kColLanes;
   const int j = part * kColBlock + 8 * cg;
   double c[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
   if (j < N) {
     const uint16_t *src = a.Xh[q] + (int64_t)e * M * N + j;
 #pragma unroll 8
-    for (int i = rg; i < M; i += kColRowGroups) {
+    for (int i = kColRowStep * rg; i < M; i += kColRowStep * kColRowGroups) {
       const anc_u32x4 w = *(const anc_u32x4 *)(src + (int64_t)i * N);
       const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll

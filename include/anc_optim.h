@@ -461,7 +461,8 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *             between 2.5 and 40 (a spectrum spread over two or three decades reads 3.6 .. 19, 10 %
  *             of the columns x10 reads 8.4, a rank-128 signal over weak noise 17), or if it lies
  *             outside and the matrix's column norms say what the proxy cannot: with
- *             colc = N * sum_j c_j^4 / (sum_j c_j^2)^2 over the column norms c_j of the input,
+ *             colc = N * sum_j c_j^4 / (sum_j c_j^2)^2 over the column norms c_j of the input
+ *             (every fourth row of it),
  *             proxy >= 40 and colc < proxy / 4 (a low-rank signal over weak noise, a steep
  *             spectrum: colc about 1, where outlier columns read colc = proxy and keep the cheap
  *             gates above), or N < 2M, 1.9 < proxy <= 2.5 and colc < 1.3 (a gap in the spectrum,
