@@ -647,6 +647,14 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
     // chain keeps adding first-order roundings: with the last three iterations only, 6 steps gave
     // 3.1e-3 and 8 steps 8.9e-3 at 1024x1024), and the last three of a shorter one.
     sp.x_from = sp.fb_from = steps >= 5 ? 2 : (steps > 3 ? steps - 3 : 0);
+    // and the matrices the wide gate flags (below) start one iteration earlier, as they do under
+    // Polar Express: a rank-32 signal over 1 % noise is 2.1e-3 at 1024x1024 with the terms from
+    // iteration 2 and 3e-4 from iteration 1
+    if (sp.x_from > 1) {
+      sp.wide_lo = kTauWideLo; sp.wide_hi = kTauWideHi;
+      sp.wide_near = N < 2 * M ? kTauWideNear : kTauWideLo;
+      sp.wide_gram_from = 1; sp.wide_all_from = 1;
+    }
     return sp;
   }
   if (mode != ANC_NS_BF16 && mode != ANC_NS_BF16_LATE3) return sp;

@@ -430,7 +430,8 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *                     times the matrix-core work of ANC_NS_BF16_FAST.
  *   ANC_NS_BF16_LATE3 ANC_NS_BF16 with the residuals of both operands in all three products from
  *                     iteration 2 on (the last three of a 5-step chain; the last three of a
- *                     shorter one), for every matrix and without gates, for M >= 1024
+ *                     shorter one) for every matrix, and from iteration 1 on for the matrices
+ *                     the wide gate flags (below); none of the other gates. For M >= 1024
  *                     (M < 1024 runs a heavier plan in either mode, see below): about 2.2 times the
  *                     matrix-core work of ANC_NS_BF16_FAST. For coefficients that do not drive the
  *                     singular values to 1: Keller's quintic (ancora/kernels/muon_ns.py:21) leaves
