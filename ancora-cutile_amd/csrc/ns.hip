@@ -457,7 +457,12 @@ __global__ void __launch_bounds__(kThreads) k_ns_cond(NsCondArgs a) {
 struct WideRule {
   double near_lo, lo, hi;    // in units of the proxy N * ||offdiag(A0)||^2; near_lo == lo: no near range
 };
-constexpr double kColcFrac = 0.25, kColcFlat = 1.3;
+// kBulkShare: outlier columns keep the cheap gates while the other columns still hold a few
+// thousandths of the mass (1 % of the columns x100: 1e-2 of it, 8e-4 .. 1.6e-3 with those gates);
+// beyond that the bulk's directions drown in the rounding of the outliers (x300: share 1e-3, 1.4e-3
+// .. 1.9e-3; x1000: 1e-4, 3.6e-3 .. 4.0e-3; x3000: 5.2e-3 .. 5.8e-3) and only every residual
+// term from iteration 1 on recovers them (8e-5 .. 2.9e-4).
+constexpr double kColcFrac = 0.25, kColcFlat = 1.3, kBulkShare = 3e-3;
 __device__ __forceinline__ double cond_proxy(const double *c, int N) {
   double s = c[0];
 #pragma unroll
@@ -540,10 +545,16 @@ __global__ void __launch_bounds__(kThreads) k_ns_classify(NsColArgs a) {
   bool wide = p > r.lo && p < r.hi;
   if (!wide && wants_colstat(r, p)) {
     const double *c = a.part[q] + (int64_t)e * a.parts[q] * 2;
-    double s2 = c[0], s4 = c[1];
-    for (int i = 1; i < a.parts[q]; ++i) { s2 = s2 + c[2 * i]; s4 = s4 + c[2 * i + 1]; }
+    double s2 = c[0], s4 = c[1], lightest = c[0];
+    for (int i = 1; i < a.parts[q]; ++i) {
+      s2 = s2 + c[2 * i];
+      s4 = s4 + c[2 * i + 1];
+      lightest = c[2 * i] < lightest ? c[2 * i] : lightest;
+    }
     const double colc = s2 > 0.0 ? (double)N * s4 / (s2 * s2) : 1.0;
-    wide = p >= r.hi ? colc < kColcFrac * p : colc < kColcFlat;
+    // outlier columns: the share of the mass outside them, from the lightest block of columns
+    const double bulk = s2 > 0.0 ? (double)a.parts[q] * lightest / s2 : 1.0;
+    wide = p >= r.hi ? (colc < kColcFrac * p || bulk < kBulkShare) : colc < kColcFlat;
   }
   a.flag[q][e] = wide ? 1 : 0;
 }

@@ -466,21 +466,24 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *             (every fourth row of it),
  *             proxy >= 40 and colc < proxy / 4 (a low-rank signal over weak noise, a steep
  *             spectrum: colc about 1, where outlier columns read colc = proxy and keep the cheap
- *             gates above), or N < 2M, 1.9 < proxy <= 2.5 and colc < 1.3 (a gap in the spectrum,
+ *             gates above), or proxy >= 40 and less than 3e-3 of the mass outside the outlier
+ *             columns (estimated from the lightest block of 64 columns: 1 % of the columns x100
+ *             leaves 1e-2 there and keeps the cheap gates, x300 and beyond 1e-3 and less), or N < 2M, 1.9 < proxy <= 2.5 and colc < 1.3 (a gap in the spectrum,
  *             e.g. near-duplicate rows; scaled columns read colc = proxy and keep the low gate).
  *             Such a matrix adds the residuals of X, F and Boff to all three products from iteration
  *             1 on (about 2.6 times the matrix-core work, for that matrix alone): condition number
  *             1e2 .. 1e4 2e-5 .. 8e-5 instead of 2.5e-3 .. 4.2e-3, rank 32 over 10 % / 1 % noise
  *             2.2e-4 / 3.9e-4 instead of 2.9e-3 / 5.0e-3, near-duplicate rows 6e-5 instead of
- *             2.4e-3. It takes precedence over the gates above.
+ *             2.4e-3, 1 % of the columns x1000 1e-4 .. 2e-4 instead of 3.6e-3 .. 4.0e-3. It takes
+ *             precedence over the gates above.
  * The decision depends on the matrix alone (fixed-order sums), never on the batch. Accuracy bar of
  * ANC_NS_BF16 with the Polar-Express schedule: 2e-3 relative Frobenius on inputs with independent
  * entries, with row or column outliers up to x100 on 1 % of the rows or columns, with 10 % of the
  * columns x10, with columns scaled over a factor 30, with log-uniform spectra up to condition
  * number 1e4, with power-law spectra, with low-rank signals over noise down to 1 %, with
  * near-duplicate rows, with sparse (90 % zeros) and heavy-tailed (Student t, 1.5 degrees of freedom
- * and up) entries, on shapes up to 4096x8192. Not met: outliers x1000 (2.7e-3 .. 4e-3;
- * ANC_NS_BF16_X3). Keller coefficients amplify operand rounding about twice as much (4.5e-3 at
+ * and up) entries, with 1 % of the rows or columns x30 .. x3000, on shapes up to 4096x8192 (the
+ * worst of them: 1.7e-3, independent entries at N = M). Keller coefficients amplify operand rounding about twice as much (4.5e-3 at
  * 1024x1024): with them the bar is that of ANC_NS_BF16_LATE3, which the host layer selects for
  * that schedule; it holds on the same classes except a single element of 1000 standard deviations
  * (3e-5 .. 3e-3 depending on the shape: an isolated singular value that hangs on one rounded

@@ -465,6 +465,28 @@ def test_low_rank_signal_over_weak_noise_is_told_from_outlier_columns(gpu, M, N)
         assert _hard_count(2, M, N, "bf16_tile128")[0] == n_gated - 1
 
 
+@pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 2048), (1024, 3072)])
+def test_extreme_outlier_columns_take_the_wide_gate(gpu, M, N):
+    """1 % of the columns x300, x1000, x3000: the other columns hold 1e-3 .. 1e-5 of the mass and
+    their directions drown in the rounding of the outliers (3.6e-3 .. 5.8e-3 at x1000 and x3000 with
+    the outlier-column gates). The proxy and the column concentration read the same as at x100;
+    the share of the mass in the lightest block of columns tells them apart. x100 keeps its
+    cheap gate."""
+    from ancora_cutile_amd import muon_ns
+    rng = np.random.default_rng(M + N)
+    g = rng.standard_normal((M, N)).astype(np.float32)
+    cols = rng.choice(N, N // 100, replace=False)
+    base = muon_ns.ns_flops(1, M, N, 5, "bf16")[0]
+    for scale, bound in ((100.0, TOL_BF16), (300.0, 4e-4), (1000.0, 4e-4), (3000.0, 6e-4)):
+        X = g.copy()
+        X[:, cols] *= np.float32(scale)
+        err = rel_fro(run_ns(X[None])[0], host_ns(X, PE_SCHEDULE, 5))
+        extra = _hard_count(1, M, N)[1] / base
+        print(f"({M},{N}) 1 % of the columns x{scale:g}: {err:.3e}, extra matrix-core work {100 * extra:.0f} %")
+        assert err < bound, scale
+        assert (extra < 0.6) if scale == 100.0 else (extra > 1.0), scale
+
+
 @pytest.mark.parametrize("M,N", [(1024, 1024), (1536, 1536), (1024, 1536)])
 def test_near_duplicate_rows_take_the_wide_gate(gpu, M, N):
     """Half of the rows repeat the other half up to 1 % noise: a spectrum with a gap, proxy 1 + N/M
