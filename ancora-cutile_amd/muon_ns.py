@@ -77,8 +77,8 @@ def effective_mode(mode, schedule):
     (they end in 0.7 .. 1.2), so the off-diagonal of A = X X^T never becomes small and the bf16
     rounding of every operand stays a first-order error up to the last iteration: the gated plan
     of "bf16", tuned on Polar Express, reaches 3e-3 .. 5e-3 there. Under Keller "bf16" therefore
-    runs as "bf16_late3" (residual terms in every product from iteration 2 on, 2.2 times
-    the matrix-core work, well inside 2e-3); "bf16_gated" keeps the gated plan. `schedule` is
+    runs as "bf16_late3" (the residual of X from iteration 2 on, those of F and Boff from
+    iteration 3 on: 2.05 times the matrix-core work, 9e-4 at worst); "bf16_gated" keeps the gated plan. `schedule` is
     the resolved one (None = Keller)."""
     if mode == "bf16" and is_keller(schedule):
         return "bf16_late3"

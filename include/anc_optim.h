@@ -428,15 +428,16 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *                     accumulation terms per product in every iteration): about 1e-5 from the
  *                     fp32 chain on every input tried, ill-conditioned ones included, for three
  *                     times the matrix-core work of ANC_NS_BF16_FAST.
- *   ANC_NS_BF16_LATE3 ANC_NS_BF16 with the residuals of both operands in all three products from
- *                     iteration 2 on (the last three of a 5-step chain; the last three of a
- *                     shorter one) for every matrix, and from iteration 1 on for the matrices
- *                     the wide gate flags (below); none of the other gates. For M >= 1024
- *                     (M < 1024 runs a heavier plan in either mode, see below): about 2.2 times the
+ *   ANC_NS_BF16_LATE3 ANC_NS_BF16 with the residual of X in its two products from iteration 2 on and
+ *                     the residuals of F and Boff from iteration 3 on (chains of 5 steps and
+ *                     more; all of them in the last three iterations of a shorter one) for every
+ *                     matrix, and every residual from iteration 1 on for the matrices the wide
+ *                     gate flags (below); none of the other gates. For M >= 1024
+ *                     (M < 1024 runs a heavier plan in either mode, see below): about 2.05 times the
  *                     matrix-core work of ANC_NS_BF16_FAST. For coefficients that do not drive the
  *                     singular values to 1: Keller's quintic (ancora/kernels/muon_ns.py:21) leaves
  *                     them in 0.7 .. 1.2, offdiag(A) never becomes small and ANC_NS_BF16 reaches
- *                     2.8e-3 .. 5e-3 only; this mode 3e-5 .. 8e-4.
+ *                     2.8e-3 .. 5e-3 only; this mode 2e-5 .. 9e-4.
  *   ANC_NS_FP32       every product in fp32 (validation mode).
  *
  * Conditioning gates (ANC_NS_BF16 only). After the first A = X X^T the chain measures

@@ -53,7 +53,7 @@ def test_bf16_mode_within_2e3(gpu, M, N, sched):
         from ancora_cutile_amd import muon_ns
         assert muon_ns.effective_mode("bf16", None) == "bf16_late3"
         if M >= 1024:
-            assert max(errs) < 2e-4
+            assert max(errs) < 1e-3
             # the gated plan, tuned on Polar Express, stays outside the bar there
             gated = run_ns(X[:1], schedule=None, mode="bf16_gated")
             assert 2e-3 < rel_fro(gated[0], host_ns(X[0], None, 5)) < 5.5e-3
