@@ -647,16 +647,16 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
     return sp;
   }
   if (mode == ANC_NS_BF16_LATE3 && M >= 1024) {
-    // residuals of X, F and Boff in all three products from iteration 2 on (the last three of a
-    // 5-step chain), for every matrix, no gates. For coefficients that do
-    // not drive the singular values to 1 (Keller's quintic leaves them in 0.7 .. 1.2, so
-    // offdiag(A) never becomes small and every operand rounding stays first-order): 1024x1024
-    // Gaussian 3.7e-3 -> 6e-5, 1024x3072 2.8e-3 -> 3e-5, condition number 1e3 2.5e-4 .. 3.2e-4,
-    // 1 % of the columns x100 3.6e-4 .. 7.9e-4; residuals in the last two iterations only leave
-    // 2.2e-3 at 1024x1024. M < 1024 runs a heavier plan in either mode (below).
-    // From iteration 2 on whatever the chain's length (Keller's iterates do not settle, so a longer
-    // chain keeps adding first-order roundings: with the last three iterations only, 6 steps gave
-    // 3.1e-3 and 8 steps 8.9e-3 at 1024x1024), and the last three of a shorter one.
+    // For coefficients that do not drive the singular values to 1 (Keller's quintic leaves them in
+    // 0.7 .. 1.2, so offdiag(A) never becomes small and every operand rounding stays first-order:
+    // the gated plan below gives 3.7e-3 at 1024x1024 and 2.8e-3 at 1024x3072 there). Every matrix,
+    // no gates of its own: the residual of X from iteration 2 on, those of F and Boff from
+    // iteration 3 on. All three from iteration 2: 6e-5 / 3e-5 for 2.2 times the plain chain; all
+    // three in the last two iterations only: 2.2e-3 at 1024x1024. M < 1024 runs a heavier plan
+    // in either mode (below).
+    // From a fixed iteration on whatever the chain's length (Keller's iterates do not settle, so a
+    // longer chain keeps adding first-order roundings: with the last three iterations only, 6 steps
+    // gave 3.1e-3 and 8 steps 8.9e-3 at 1024x1024), and the last three of a shorter one.
     sp.x_from = sp.fb_from = steps >= 5 ? 2 : (steps > 3 ? steps - 3 : 0);
     // The residuals of F and Boff can start one iteration after that of X: 8e-4 at 1024x1024
     // (independent entries, scaled columns, outlier columns alike) and 4e-4 .. 7.5e-4 at 1024x3072
