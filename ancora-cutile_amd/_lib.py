@@ -18,6 +18,8 @@ FORM_DIV, FORM_IBC = 0, 1         # ANC_ADAMW_FORM_*
 NS_BF16, NS_FP32, NS_BF16_FAST, NS_BF16_X3, NS_BF16_LATE3 = 0, 1, 2, 3, 4   # ANC_NS_*
 GN_CHUNK = 8192                   # ANC_GN_CHUNK
 MUON_MAX_SCALES = 8               # ANC_MUON_MAX_SCALES
+SR_ON, SR_STEP_SEED, SR_SEED_STRIDE = 1, 2, 1000003   # ANC_SR_*
+ABI_VERSION = 3                   # the anc_abi_version() these prototypes were written for
 
 u64, i64, i32, u32, f32 = C.c_uint64, C.c_int64, C.c_int32, C.c_uint32, C.c_float
 
@@ -35,13 +37,18 @@ class DeviceInfo(C.Structure):
 
 class StepCtl(C.Structure):
     _fields_ = [("sumsq", C.c_double), ("norm", f32), ("clip_scale", f32), ("skip", u32),
-                ("reserved", u32 * 3)]
+                ("t", u32), ("reserved", u32 * 2)]
 
 
 class AdamWHyper(C.Structure):
     _fields_ = [("beta1", f32), ("beta2", f32), ("omb1", f32), ("omb2", f32), ("eps", f32),
                 ("lr", f32), ("bc1", f32), ("bc2", f32), ("form", i32), ("sr", i32),
-                ("seed_base", u32), ("reserved", u32)]
+                ("seed_base", u32), ("step_cap", i32), ("step_table", u64)]
+
+
+class AdamWStepEntry(C.Structure):
+    """anc_adamw_step_t: the scalars of one counted step."""
+    _fields_ = [("bc1", f32), ("bc2", f32), ("lr", f32), ("seed_base", u32)]
 
 
 class AdamWDesc(C.Structure):
@@ -99,15 +106,13 @@ _PROTOS = {
     "anc_event_sync": (None, [u64]),
     "anc_stream_wait_event": (None, [u64, u64]),
     "anc_event_elapsed_ms": (None, [u64, u64, C.POINTER(f32)]),
-    "anc_copy_shape": (None, [u64, u64, i64, C.c_int, C.POINTER(i64), u64]),
-    "anc_mfma_rate": (None, [C.c_int, i64, u64, C.POINTER(C.c_double), u64]),
     "anc_copy_kernel": (None, [u64, u64, i64, u64]),
     "anc_profile_enable": (None, [C.c_int]),
     "anc_profile_read": (None, [C.POINTER(f32), C.POINTER(i64)]),
     "anc_gradnorm_num_partials": (i64, [i64]),
     "anc_gradnorm_partials": (None, [u64, i64, C.c_int, u64, i64, u64]),
     "anc_gradnorm_partials_multi": (None, [u64, i32, i64, u64, u64]),
-    "anc_gradnorm_finalize": (None, [u64, i64, f32, f32, u64, u64]),
+    "anc_gradnorm_finalize": (None, [u64, i64, f32, f32, i32, u64, u64]),
     "anc_gradnorm_static_max_elements": (i64, []),
     "anc_gradnorm_static": (None, [u64, i64, C.c_int, f32, f32, u64, u64]),
     "anc_adamw": (None, [u64, u64, u64, u64, u64, i64, C.c_int, C.POINTER(AdamWHyper), f32, u32,
@@ -187,6 +192,10 @@ def load(path=None):
         fn.argtypes = argtypes
         fn.restype = C.c_int if restype is None else restype
         setattr(api, name, _checked(fn, name) if restype is None else fn)
+    got = lib.anc_abi_version()
+    if got != ABI_VERSION:
+        raise AncoraError(f"{p} has ABI version {got}, this binding was written for {ABI_VERSION}: "
+                          "rebuild the library (python -m ancora_cutile_amd.build)")
     _lib = lib
     return lib
 

@@ -22,7 +22,8 @@ import ctypes
 import numpy as np
 
 from . import _lib
-from ._lib import api, AdamWHyper, AdamWDesc, F32, BF16, FORM_DIV, FORM_IBC
+from ._lib import (api, AdamWHyper, AdamWDesc, AdamWStepEntry, F32, BF16, FORM_DIV, FORM_IBC, SR_ON,
+                   SR_STEP_SEED)
 from .bf16 import bf16_bits as _bf16_bits, bits_f32 as _bits_f32  # noqa: F401  (re-exported)
 from .devbuf import DevBuf, upload_table
 
@@ -110,6 +111,39 @@ class AdamW:
         self._table = None
         self._table_key = None
         self.last_skipped = False
+        self._steps = None           # device table of per-step bias corrections (steps counted on the device)
+        self._steps_cap = 0
+        self._steps_saturated = False
+        self._steps_old = []
+
+    # -- steps counted on the device: bias corrections by step, filled ahead
+    def _bias_corrections(self, t):
+        if self.form == "div":
+            return 1 - self.b1 ** t, 1 - self.b2 ** t
+        return 1.0 / (1.0 - self.b1 ** t), 1.0 / (1.0 - self.b2 ** t)
+
+    def _ensure_step_table(self, t_upper):
+        """Device table of anc_adamw_step_t whose entry t holds the bias corrections of step t, the
+        same Python-double values rounded to fp32 once that `_hyper` passes per step. It ends where
+        both corrections have reached 1.0f (the kernel uses the last entry for every later step);
+        while they have not, it is extended ahead of `t_upper`, the largest step the next launch
+        can be."""
+        if self._steps is not None and (self._steps_saturated or t_upper < self._steps_cap):
+            return
+        cap = max(1024, 2 * self._steps_cap, 2 * int(t_upper))
+        tab = (AdamWStepEntry * (cap + 1))()
+        one = np.float32(1.0)
+        n, saturated = cap, False
+        for t in range(1, cap + 1):
+            bc1, bc2 = self._bias_corrections(t)
+            tab[t].bc1, tab[t].bc2 = bc1, bc2
+            if np.float32(bc1) == one and np.float32(bc2) == one:
+                n, saturated = t, True
+                break
+        if self._steps is not None:
+            self._steps_old.append(self._steps)      # a launch in flight may still read it
+        self._steps = DevBuf(np.frombuffer(tab, dtype=np.uint32, count=4 * (n + 1)).copy())
+        self._steps_cap, self._steps_saturated = n, saturated
 
     # -- descriptor table: one row per tensor, rebuilt only when a gradient pointer changes
     def _build_table(self, gbufs):
@@ -138,11 +172,20 @@ class AdamW:
         ibc2 = 1.0 / (1.0 - self.b2 ** self.t)
         return hyper_ibc(self.lr, self.b1, self.b2, self.eps, ibc1, ibc2, self.sr, sb)
 
-    def launch(self, grads, stream_int, guard=None):
+    def launch(self, grads, stream_int, guard=None, device_steps=False, t_upper=None):
         """Asynchronous part of the step: upload host gradients (DevBuf gradients are used in
         place) and launch the fused kernel once over all tensors. `t` is advanced first, as in
-        ancora/optim/adamw.py:89-91; a caller that later finds the step skipped calls `unstep()`."""
-        self.t += 1
+        ancora/optim/adamw.py:89-91; a caller that later finds the step skipped calls `unstep()`.
+        With `device_steps` the step count lives in the guard's control block (advanced by
+        `guard.compute(..., count_step=True)` unless the step is skipped): the kernel takes the
+        bias corrections of that step from a table and forms the rounding seed from the count, `t`
+        here is left alone and nothing needs undoing; `t_upper` bounds the count from above."""
+        if device_steps:
+            if guard is None:
+                raise ValueError("AdamW.launch: device_steps needs the guard whose block counts the steps")
+            self._ensure_step_table(self.t + 1 if t_upper is None else t_upper)
+        else:
+            self.t += 1
         gbufs = []
         for name, s in self.st.items():
             g = grads[name]
@@ -158,7 +201,15 @@ class AdamW:
                 s["g"].upload(g.reshape(s["R"], C), stream_int)
                 gbufs.append(s["g"])
         self._build_table(gbufs)
-        h = self._hyper()
+        if device_steps:
+            if self.form == "div":
+                h = hyper_div(self.lr, self.b1, self.b2, self.eps, 1, False, self.seed)
+            else:
+                h = hyper_ibc(self.lr, self.b1, self.b2, self.eps, 1.0, 1.0, False, self.seed)
+            h.sr = (SR_ON | SR_STEP_SEED) if self.sr else 0
+            h.step_table, h.step_cap = self._steps.ptr, self._steps_cap
+        else:
+            h = self._hyper()
         api.anc_adamw_multi(self._table.ptr, len(self.st), self._total_blocks, ctypes.byref(h),
                             0 if guard is None else guard.ptr, int(stream_int))
 
@@ -212,3 +263,6 @@ class AdamW:
         if self._table is not None:
             self._table.free()
             self._table = None
+        for b in self._steps_old + ([self._steps] if self._steps is not None else []):
+            b.free()
+        self._steps, self._steps_old = None, []

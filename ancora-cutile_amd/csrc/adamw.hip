@@ -129,11 +129,30 @@ __device__ __forceinline__ bool load_ctl(const anc_step_ctl_t *ctl, float &clip)
   return true;
 }
 
+struct RowStep { float bc1, bc2, lr; uint32_t seed_base; };   // anc_adamw_step_t; entry s: counted step s (1-based)
+
+// Steps counted on the device: the bias corrections of step ctl->t from the table the host filled
+// ahead (the same fp32 values it would pass per step), the rounding seed from the count itself.
+__device__ __forceinline__ void step_scalars(anc_adamw_hyper_t &h, const anc_step_ctl_t *ctl) {
+  if (ctl == nullptr) return;
+  const uint32_t t = ctl->t;
+  if (h.step_table != 0) {
+    const uint32_t i = t < 1u ? 1u : (t > (uint32_t)h.step_cap ? (uint32_t)h.step_cap : t);
+    const RowStep rs = ((const RowStep *)h.step_table)[i];
+    h.bc1 = rs.bc1;
+    h.bc2 = rs.bc2;
+  }
+  if (h.sr & ANC_SR_STEP_SEED) h.seed_base += ANC_SR_SEED_STRIDE * t;
+}
+
 template <int GD, int FORM, int SR>
 __global__ void __launch_bounds__(kThreads)
 k_adamw(Tensor t, anc_adamw_hyper_t h, const anc_step_ctl_t *__restrict__ ctl) {
   float clip;
   if (!load_ctl(ctl, clip)) return;
+  const uint32_t seed0 = h.seed_base;
+  step_scalars(h, ctl);
+  t.seed += h.seed_base - seed0;
   adamw_block<GD, FORM, SR>(t, (int64_t)blockIdx.x, h, clip);
 }
 
@@ -143,6 +162,7 @@ k_adamw_multi(const anc_adamw_desc_t *__restrict__ table, int n_tensors, anc_ada
               const anc_step_ctl_t *__restrict__ ctl) {
   float clip;
   if (!load_ctl(ctl, clip)) return;
+  step_scalars(h, ctl);
   const int64_t blk = (int64_t)blockIdx.x;
   // Last tensor whose first block is <= blk (the table is sorted by blk0).
   int lo = 0, hi = n_tensors - 1;
@@ -200,8 +220,6 @@ k_cast_bf16(const float *__restrict__ p32, uint16_t *__restrict__ p16, int64_t n
 // bit-identical to what the dense kernel would hold. A row is brought up to date (a) before the
 // forward pass gathers it (anc_adamw_rows with grads = 0: replay through step t_now) and (b) by
 // the step itself (replay through t_now - 1, then step t_now with its gradient row).
-struct RowStep { float bc1, bc2, lr; uint32_t seed_base; };   // entry s: counted step s (1-based)
-
 template <int FORM, int SR>
 __global__ void __launch_bounds__(kThreads)
 k_adamw_rows(const int32_t *__restrict__ rows, const float *__restrict__ grads, float *__restrict__ m,
@@ -258,7 +276,10 @@ int check_hyper(const anc_adamw_hyper_t *h, const char *who) {
   ANC_REQUIRE(h != nullptr, "%s: null hyper-parameter block", who);
   ANC_REQUIRE(h->form == ANC_ADAMW_FORM_DIV || h->form == ANC_ADAMW_FORM_IBC,
               "%s: unknown form %d", who, h->form);
-  ANC_REQUIRE(h->sr == 0 || h->sr == 1, "%s: sr must be 0 or 1", who);
+  ANC_REQUIRE(h->sr == 0 || h->sr == ANC_SR_ON || h->sr == (ANC_SR_ON | ANC_SR_STEP_SEED),
+              "%s: sr must be 0, ANC_SR_ON or ANC_SR_ON | ANC_SR_STEP_SEED", who);
+  ANC_REQUIRE(h->step_table == 0 || ((h->step_table & 15) == 0 && h->step_cap >= 1),
+              "%s: step_table must be 16-byte aligned with step_cap >= 1", who);
   return ANC_OK;
 }
 
@@ -282,6 +303,8 @@ extern "C" int anc_adamw(uint64_t g, uint64_t m, uint64_t v, uint64_t p32, uint6
                          int64_t n, int g_dtype, const anc_adamw_hyper_t *h, float wd,
                          uint32_t seed, uint64_t ctl, uint64_t stream) {
   if (int rc = check_hyper(h, "anc_adamw")) return rc;
+  ANC_REQUIRE(ctl != 0 || (h->step_table == 0 && !(h->sr & ANC_SR_STEP_SEED)),
+              "anc_adamw: steps counted on the device need the control block");
   ANC_REQUIRE(g && m && v && p32 && p16, "anc_adamw: null device pointer");
   ANC_REQUIRE(n > 0 && n % 64 == 0, "anc_adamw: n=%lld must be a positive multiple of 64",
               (long long)n);
@@ -312,6 +335,8 @@ extern "C" int anc_adamw(uint64_t g, uint64_t m, uint64_t v, uint64_t p32, uint6
 extern "C" int anc_adamw_multi(uint64_t desc_table, int32_t n_tensors, int64_t total_blocks,
                                const anc_adamw_hyper_t *h, uint64_t ctl, uint64_t stream) {
   if (int rc = check_hyper(h, "anc_adamw_multi")) return rc;
+  ANC_REQUIRE(ctl != 0 || (h->step_table == 0 && !(h->sr & ANC_SR_STEP_SEED)),
+              "anc_adamw_multi: steps counted on the device need the control block");
   ANC_REQUIRE(desc_table != 0 && n_tensors > 0, "anc_adamw_multi: empty descriptor table");
   ANC_REQUIRE(total_blocks > 0 && total_blocks < (1ll << 31),
               "anc_adamw_multi: total_blocks=%lld out of range", (long long)total_blocks);

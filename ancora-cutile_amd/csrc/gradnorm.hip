@@ -49,7 +49,7 @@ constexpr int kFinThreads = 1024;
 
 __global__ void __launch_bounds__(kFinThreads)
 k_gn_finalize(const double *__restrict__ partials, int64_t n_partials, float max_norm, float eps,
-              anc_step_ctl_t *__restrict__ ctl) {
+              int count_step, anc_step_ctl_t *__restrict__ ctl) {
   __shared__ double wave_sum[kFinThreads / 64];
   double acc = 0.0;
   for (int64_t i = threadIdx.x; i < n_partials; i += kFinThreads) acc = acc + partials[i];
@@ -71,7 +71,8 @@ k_gn_finalize(const double *__restrict__ partials, int64_t n_partials, float max
     ctl->norm = norm;
     ctl->clip_scale = clip;
     ctl->skip = finite ? 0u : 1u;
-    ctl->reserved[0] = ctl->reserved[1] = ctl->reserved[2] = 0u;
+    if (count_step && finite) ctl->t = ctl->t + 1u;      // a skipped step is not counted
+    ctl->reserved[0] = ctl->reserved[1] = 0u;
   }
 }
 
@@ -118,13 +119,13 @@ extern "C" int anc_gradnorm_partials_multi(uint64_t desc_table, int32_t n_tensor
 }
 
 extern "C" int anc_gradnorm_finalize(uint64_t partials, int64_t n_partials, float max_norm,
-                                     float eps, uint64_t ctl, uint64_t stream) {
+                                     float eps, int32_t count_step, uint64_t ctl, uint64_t stream) {
   ANC_REQUIRE(partials != 0 && ctl != 0 && n_partials > 0,
               "anc_gradnorm_finalize: bad arguments (n_partials=%lld)", (long long)n_partials);
   ANC_REQUIRE((ctl & 7) == 0, "anc_gradnorm_finalize: ctl must be 8-byte aligned");
   AncProfScope prof(ANC_PROF_GN_FINALIZE, anc_stream(stream));
   hipLaunchKernelGGL(k_gn_finalize, dim3(1), dim3(kFinThreads), 0, anc_stream(stream),
-                     (const double *)partials, n_partials, max_norm, eps, (anc_step_ctl_t *)ctl);
+                     (const double *)partials, n_partials, max_norm, eps, (int)count_step, (anc_step_ctl_t *)ctl);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
 }
@@ -183,7 +184,7 @@ extern "C" int anc_gradnorm_static(uint64_t g, int64_t n, int g_dtype, float max
   else
     hipLaunchKernelGGL(k_gn_partials<ANC_F32>, dim3((unsigned)chunks), dim3(kThreads), 0, s, (const void *)g, n, ptr);
   ANC_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_gn_finalize, dim3(1), dim3(kFinThreads), 0, s, (const double *)ptr, chunks, max_norm, eps,
+  hipLaunchKernelGGL(k_gn_finalize, dim3(1), dim3(kFinThreads), 0, s, (const double *)ptr, chunks, max_norm, eps, 0,
                      (anc_step_ctl_t *)ctl);
   ANC_LAUNCH_CHECK();
   return ANC_OK;

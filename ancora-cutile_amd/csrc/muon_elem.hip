@@ -350,9 +350,10 @@ struct LrScales { float v[ANC_MUON_MAX_SCALES]; };
 template <int OD, int SR>
 __global__ void __launch_bounds__(kThreads)
 k_upd_multi(const anc_muon_desc_t *__restrict__ table, int n_weights, LrScales scales,
-            uint32_t seed_base, const anc_step_ctl_t *__restrict__ ctl) {
+            uint32_t seed_base, int step_seed, const anc_step_ctl_t *__restrict__ ctl) {
   float clip;
   if (!load_ctl(ctl, clip)) return;
+  if (step_seed) seed_base += ANC_SR_SEED_STRIDE * ctl->t;      // steps counted on the device
   const anc_muon_desc_t d = find_weight(table, n_weights, (int64_t)blockIdx.x);
   const int64_t local = (int64_t)blockIdx.x - d.tile0;
   UpdArgs a{(float *)d.p32, (uint16_t *)d.p16, (const void *)d.u, d.K, d.N,
@@ -452,6 +453,7 @@ extern "C" int anc_muon_update(uint64_t p32, uint64_t p16, uint64_t O, int64_t K
   ANC_REQUIRE(p32 && O, "anc_muon_update: null device pointer");
   ANC_REQUIRE(o_dtype == ANC_F32 || o_dtype == ANC_BF16, "anc_muon_update: bad dtype");
   ANC_REQUIRE(((p32 | O) & 15) == 0 && (p16 & 7) == 0, "anc_muon_update: misaligned pointers");
+  ANC_REQUIRE(sr == 0 || sr == ANC_SR_ON, "anc_muon_update: sr must be 0 or ANC_SR_ON");
   UpdArgs a{(float *)p32, (uint16_t *)p16, (const void *)O, (int)K, (int)N, lr_scale, seed};
   const anc_step_ctl_t *c = (const anc_step_ctl_t *)ctl;
   const dim3 grid((unsigned)((K * N) / kBlockElems)), block(kThreads);
@@ -521,12 +523,14 @@ extern "C" int anc_muon_update_multi(uint64_t desc_table, int32_t n_weights, int
   const dim3 grid((unsigned)total_tiles), block(kThreads);
   hipStream_t s = anc_stream(stream);
   AncProfScope prof(ANC_PROF_MUON_UPD, s);
+  const int step_seed = (sr & ANC_SR_STEP_SEED) ? 1 : 0;
+  ANC_REQUIRE(!step_seed || ctl != 0, "anc_muon_update_multi: ANC_SR_STEP_SEED needs the control block");
   const int sel = (o_dtype == ANC_BF16 ? 2 : 0) | (sr ? 1 : 0);
   switch (sel) {
-    case 0: hipLaunchKernelGGL((k_upd_multi<ANC_F32, 0>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, c); break;
-    case 1: hipLaunchKernelGGL((k_upd_multi<ANC_F32, 1>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, c); break;
-    case 2: hipLaunchKernelGGL((k_upd_multi<ANC_BF16, 0>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, c); break;
-    default: hipLaunchKernelGGL((k_upd_multi<ANC_BF16, 1>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, c); break;
+    case 0: hipLaunchKernelGGL((k_upd_multi<ANC_F32, 0>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, step_seed, c); break;
+    case 1: hipLaunchKernelGGL((k_upd_multi<ANC_F32, 1>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, step_seed, c); break;
+    case 2: hipLaunchKernelGGL((k_upd_multi<ANC_BF16, 0>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, step_seed, c); break;
+    default: hipLaunchKernelGGL((k_upd_multi<ANC_BF16, 1>), grid, block, 0, s, tab, (int)n_weights, sc, seed_base, step_seed, c); break;
   }
   ANC_LAUNCH_CHECK();
   return ANC_OK;

@@ -152,6 +152,7 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
   float sc = 1.0f;
   if (EPI != EPI_BMAT && p.scale != nullptr) sc = p.scale[e];
   const float acc_scale = (EPI == EPI_GRAM) ? sc * sc : sc;
+  const bool has_a32 = EPI != EPI_BX && anc_ns_has_a32(p, e);
 #pragma unroll
   for (int bi = 0; bi < 2; ++bi) {
 #pragma unroll
@@ -164,10 +165,10 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
         if (EPI == EPI_GRAM) {
           const bool diag = gi == gj;
           const uint16_t fh = diag ? (uint16_t)0 : (uint16_t)hw_bf16(v);
-          p.A32[mm + (int64_t)gi * M + gj] = v;
+          if (has_a32) p.A32[mm + (int64_t)gi * M + gj] = v;
           p.Fh[mm + (int64_t)gi * M + gj] = fh;
           if (tm != tn) {
-            p.A32[mm + (int64_t)gj * M + gi] = v;
+            if (has_a32) p.A32[mm + (int64_t)gj * M + gi] = v;
             p.Fh[mm + (int64_t)gj * M + gi] = fh;
           }
           if (p.Fl != nullptr) {
@@ -178,7 +179,8 @@ __global__ void __launch_bounds__(kGemmThreads, 2) k_ns_gemm(NsGemm p) {
           }
           if (diag) p.dA[mv + gi] = v;
         } else if (EPI == EPI_BMAT) {
-          const float a = p.A32[mm + (int64_t)gi * M + gj];
+          const float a = has_a32 ? p.A32[mm + (int64_t)gi * M + gj]
+                                  : anc_bf16_bits_to_f32(p.Fh[mm + (int64_t)gi * M + gj]);
           const float di = p.dA[mv + gi], dj = p.dA[mv + gj];
           uint16_t bh, bl = 0;
           if (gi != gj) {
@@ -593,6 +595,13 @@ struct SplitPlan {
   // wide_all_from on. wide_hi == 0: no such gate.
   float wide_lo, wide_hi, wide_near;   // wide_near: start of the near range below the band (== wide_lo: none)
   int wide_gram_from, wide_all_from;
+  // No fp32 copy of A except for the matrices the wide gate flags: B = b A + c A A takes the
+  // off-diagonal entries of A from the bf16 Fh it multiplies anyway. Costs 3 .. 8 % of accuracy where
+  // N >= 2M (independent entries 1.36e-3 -> 1.41e-3 at 1024x2048 and 1.16e-3 -> 1.20e-3 at 1024x3072,
+  // 1 % of the columns x100 1.58e-3 -> 1.66e-3 and 1.15e-3 -> 1.24e-3) and saves 6 of the 13 bytes
+  // per element of A an iteration moves; N < 2M keeps the copy (the column-scaled probe input at
+  // 1024x1024 would go from 1.85e-3 to 2.10e-3).
+  bool drop_a32;
   bool gated(int k) const { return k >= 0 && k < kGateIters && k < x_from && gate_tau[k] > 0.0f; }
   bool wide() const { return wide_hi > 0.0f; }
   bool wide_gram(int k) const { return wide() && k >= wide_gram_from && k < x_from; }
@@ -677,6 +686,7 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
   // The first iterations are insensitive (the singular values are still far below 1, so
   // B X is a small correction to a X); residuals start at a fixed iteration index.
   if (M >= 1024) {
+    sp.drop_a32 = mode == ANC_NS_BF16 && N >= 2 * M;
     if (steps >= 2) {                         // terms from iteration 1 to the end, whatever the length
                                               // (cond 1e3 without: 6 steps 4.4e-3 .. 7e-3, 8 steps 6e-3 .. 1.8e-2)
       sp.wide_lo = kTauWideLo; sp.wide_hi = kTauWideHi;
@@ -830,6 +840,11 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
       NsGemm g{};
       g.M = (int)M; g.N = (int)N;
       g.A32 = pl.A32; g.Fh = pl.Fh; g.dA = pl.dA; g.Bh = pl.Bh; g.dB = pl.dB;
+      if (pl.sp.drop_a32) {
+        // the first iteration runs before the classification: nobody is flagged yet
+        g.a32_gated = 1;
+        g.a32_flag = (k > 0 && pl.sp.wide()) ? pl.wide_flag : nullptr;
+      }
       g.Fl = split_fb ? pl.Fl : nullptr;
       g.Bl = split_fb ? pl.Bl : nullptr;
       g.ca = coef[3 * k]; g.cb = coef[3 * k + 1]; g.cc = coef[3 * k + 2];
@@ -1255,7 +1270,10 @@ extern "C" int anc_muon_ns_update_multi(const anc_ns_problem_t *probs, int32_t n
   ANC_REQUIRE(desc_tables != nullptr && lr_scales != nullptr, "anc_muon_ns_update_multi: null descriptor tables or lr_scales");
   NsUpdate u{};
   for (int k = 0; k < ANC_MUON_MAX_SCALES; ++k) u.lr[k] = lr_scales[k];
-  u.sr = sr ? 1 : 0;
+  ANC_REQUIRE(sr == 0 || sr == ANC_SR_ON || sr == (ANC_SR_ON | ANC_SR_STEP_SEED),
+              "anc_muon_ns_update_multi: sr must be 0, ANC_SR_ON or ANC_SR_ON | ANC_SR_STEP_SEED");
+  ANC_REQUIRE(!(sr & ANC_SR_STEP_SEED) || ctl != 0, "anc_muon_ns_update_multi: ANC_SR_STEP_SEED needs the control block");
+  u.sr = sr;
   u.seed_base = seed_base;
   u.ctl = (const anc_step_ctl_t *)ctl;
   return pair_multi_impl("anc_muon_ns_update_multi", probs, n_probs, desc_tables, &u, steps, coef, eps, mode, stream);

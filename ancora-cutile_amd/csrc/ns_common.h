@@ -69,6 +69,12 @@ struct NsGemm {
   int M, N;                  // matrix dims of the chain (A, B are MxM; X is MxN)
   float ca, cb, cc;
   float *A32;                // (E,M,M) fp32 A            GRAM out, BMAT in
+  // With a32_gated set the fp32 copy of A exists only for the matrices that a32_flag marks (a null
+  // a32_flag marks none): GRAM writes A32 for those alone and BMAT takes the off-diagonal entries
+  // of A from Fh (bf16) for every other matrix. Fh is then read at the output position, which for
+  // the 256-tile kernel means panel layout.
+  int a32_gated;
+  const int32_t *a32_flag;   // (E)
   uint16_t *Fh;              // (E,M,M) bf16 off-diag A   GRAM out
   uint16_t *Fl, *Bl;         // bf16 residuals of F and Boff; null unless this step splits them
   float *dA;                 // (E,M)   diag A            GRAM out, BMAT in
@@ -119,6 +125,11 @@ __device__ __forceinline__ double anc_ns_proxy(const NsGemm &p, int e) {
 // Did the classification flag matrix e for the second gate?
 __device__ __forceinline__ bool anc_ns_wide(const NsGemm &p, int e) {
   return p.wide_flag != nullptr && p.wide_flag[e] != 0;
+}
+// Does matrix e keep the fp32 copy of A (GRAM writes it, BMAT reads it)?
+__device__ __forceinline__ bool anc_ns_has_a32(const NsGemm &p, int e) {
+  if (p.A32 == nullptr) return false;
+  return p.a32_gated == 0 || (p.a32_flag != nullptr && p.a32_flag[e] != 0);
 }
 __device__ __forceinline__ int anc_ns_terms(const NsGemm &p, int e) {
   if (p.nterms_wide > 0 && anc_ns_wide(p, e)) return p.nterms_wide;

@@ -524,6 +524,19 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     for (int j = 0; j < 8; ++j)
       dma16_epi((const char *)p.A32 + ub + (int64_t)(4 * j) * M * 4 + ((j & 1) ? vo_a1 : vo_a0), lds_addr(b + j * 1024));
   };
+  // Without an fp32 copy of A (see NsGemm::a32_gated) B takes the off-diagonal entries of A from
+  // Fh: in panel layout a 32x64 slab is 32 rows of two panels, 2 KiB contiguous each, 4 DMA
+  // instructions (16 rows of one panel each); in the buffer [panel][row][32 columns].
+  const bool has_a32 = EPI != EPI_BX && anc_ns_has_a32(p, e);
+  auto fetch_fh = [&](int bi) {
+    unsigned char *b = inbuf(bi);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t el = mm + ((int64_t)(gj0w / 32 + (j >> 1)) * M + gi0w + bi * 32 + (j & 1) * 16) * 32;
+      dma16_epi((const char *)(p.Fh + el) + lane * 16, lds_addr(b + j * 1024));
+    }
+  };
+  auto fetch_a = [&](int bi) { if (has_a32) fetch_a32(bi); else fetch_fh(bi); };
   int in_lane[2] = {0, 0};
   unsigned char *aux_w = aux + (EPI != EPI_GRAM ? wave * 1024 : 0);
   if (EPI == EPI_BMAT) {
@@ -533,8 +546,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     // dA of the wavefront's rows (lanes 0..31) and columns (lanes 32..47, repeated by 48..63)
     const float *dsrc = (lane < 32) ? p.dA + mv + gi0w + lane * 4 : p.dA + mv + gj0w + (lane & 15) * 4;
     dma16(dsrc, lds_addr(aux_w));
-    fetch_a32(0);
-    fetch_a32(1);
+    fetch_a(0);
+    fetch_a(1);
   }
   unsigned char *dvec_lds = aux_w;
   if (EPI == EPI_BX && !PLAINV) {
@@ -576,7 +589,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       wN = d.N;
       wtr = d.transpose != 0;
       wlr = pm.lr[d.scale_idx & (ANC_MUON_MAX_SCALES - 1)];
-      wseed = pm.seed_base + d.seed;
+      wseed = pm.seed_base + d.seed + ((pm.sr & ANC_SR_STEP_SEED) ? ANC_SR_SEED_STRIDE * pm.ctl->t : 0u);
     }
     // element offset in W of the 4 values lane-piece pz handles
     auto w_off = [&](int gi0, int pz) -> int64_t {
@@ -703,7 +716,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
             for (int k4 = 0; k4 < 4; ++k4) {
               pp[k4] = pp[k4] - wlr * o[k4];
               const uint64_t i = (uint64_t)(we + k4);
-              hb[k4] = pm.sr ? anc_bf16_sr_bits(pp[k4], (uint32_t)(i >> 6), (uint32_t)(i & 63u), wseed)
+              hb[k4] = (pm.sr & ANC_SR_ON) ? anc_bf16_sr_bits(pp[k4], (uint32_t)(i >> 6), (uint32_t)(i & 63u), wseed)
                              : anc_bf16_rne_bits(pp[k4]);
             }
             const anc_f32x4 po = {pp[0], pp[1], pp[2], pp[3]};
@@ -767,16 +780,31 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       // Wait for this slab's DMA only (see the X = a X + B X branch). Stores of a slab: 4 per
       // staged bf16 block (Bh, its mirror, and the same for Bl); the conditional dB stores of
       // diagonal tiles only add to what may stay outstanding, so leaving them out is safe.
+      // A slab's fetch is 8 DMA instructions (A32) or 4 (Fh).
       const int nst = 4 * ((mirror ? 2 : 1) * (write_lo ? 2 : 1));
-      if (bi == 0) wait_vm<8>();
-      else if (bi == 3) { if (nst == 4) wait_vm<4>(); else if (nst == 8) wait_vm<8>(); else wait_vm<16>(); }
-      else { if (nst == 4) wait_vm<12>(); else if (nst == 8) wait_vm<16>(); else wait_vm<24>(); }
+      const int young = bi == 0 ? (has_a32 ? 8 : 4) : bi == 3 ? nst : nst + (has_a32 ? 8 : 4);
+      if (young >= 24) wait_vm<24>();
+      else if (young >= 20) wait_vm<20>();
+      else if (young >= 16) wait_vm<16>();
+      else if (young >= 12) wait_vm<12>();
+      else if (young >= 8) wait_vm<8>();
+      else wait_vm<4>();
       const unsigned char *b = inbuf(bi);
+      if (has_a32) {
 #pragma unroll
-      for (int bj = 0; bj < 2; ++bj)
+        for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          in[bj][r] = *(const float *)(b + in_lane[bj] + (8 * (r >> 2) + (r & 3)) * 256);
+          for (int r = 0; r < 16; ++r)
+            in[bj][r] = *(const float *)(b + in_lane[bj] + (8 * (r >> 2) + (r & 3)) * 256);
+      } else {
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            in[bj][r] = anc_bf16_bits_to_f32(*(const uint16_t *)(b + bj * 2048 + row * 64 + (lane & 31) * 2));
+          }
+      }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const anc_f32x4 d4 = *(const anc_f32x4 *)(aux_w + (bi * 32 + 8 * q + 4 * (lane >> 5)) * 4);
@@ -796,7 +824,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
         const float v = (EPI == EPI_BMAT) ? acc[bi][bj][r] : acc[bi][bj][r] * acc_scale;
         if (EPI == EPI_GRAM) {
           const bool diag = gi == gj;
-          p.A32[mm + (int64_t)gi * M + gj] = v;
+          if (has_a32) p.A32[mm + (int64_t)gi * M + gj] = v;
           ov[bj][r] = diag ? 0.0f : v;
           if (diag) p.dA[mv + gi] = v;
         } else if (EPI == EPI_BMAT) {
@@ -840,7 +868,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       }
       __builtin_amdgcn_s_waitcnt(0xC07F);
       asm volatile("" ::: "memory");
-      if (bi + 2 < 4) fetch_a32(bi + 2);
+      if (bi + 2 < 4) fetch_a(bi + 2);
     }
   }
 }
@@ -851,6 +879,7 @@ int launch_sym(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
   pm.n = n;
   int64_t grid = 0;
   for (int k = 0; k < n; ++k) {
+    ANC_REQUIRE(!ps[k].a32_gated || ps[k].f_panel, "anc_ns_gemm_big: A taken from Fh needs the panel layout");
     pm.g[k] = ps[k];
     pm.g[k].tiles_m = pm.g[k].tiles_n = ps[k].M / 256;
     const int64_t t = Es[k] * ((int64_t)pm.g[k].tiles_m * (pm.g[k].tiles_m + 1) / 2);

@@ -61,10 +61,19 @@ class StepGuard:
     def partials_ptr(self, i):
         return self._partials.ptr + 8 * self._part0[i]
 
-    def compute(self, grads, stream=0, produced=()):
+    def set_t(self, t, stream=0):
+        """Set the device step count (a fresh optimizer starts at 0; a resumed one at its saved
+        count). The rest of the block is rewritten by the next `compute`."""
+        raw = np.zeros(8, np.uint32)
+        raw[5] = np.uint32(int(t))
+        self.ctl.upload(raw, stream)
+
+    def compute(self, grads, stream=0, produced=(), count_step=False):
         """grads: list of DevBuf (float32 or uint16/bf16), in a fixed order. `produced`: indices
         of gradients whose partial sums are already in place (written by their producer since the
-        last call). The result is the same bits either way. Asynchronous."""
+        last call). The result is the same bits either way. `count_step`: advance the block's step
+        count `t` unless the step is skipped (for update kernels that take their per-step scalars
+        from it). Asynchronous."""
         self.plan(grads)
         produced = tuple(sorted(set(int(i) for i in produced)))
         if produced not in self._tables:
@@ -79,13 +88,14 @@ class StepGuard:
         if table is not None:
             api.anc_gradnorm_partials_multi(table.ptr, n_tensors, n_chunks, self._partials.ptr, int(stream))
         api.anc_gradnorm_finalize(self._partials.ptr, self._n_partials, self.max_norm, self.eps,
-                                  self.ctl.ptr, int(stream))
+                                  int(bool(count_step)), self.ctl.ptr, int(stream))
 
     def read(self, stream=0):
         """Synchronise and return the control block as a dict."""
         raw = self.ctl.to_numpy(stream)
         c = StepCtl.from_buffer_copy(raw.tobytes())
-        return {"sumsq": c.sumsq, "norm": c.norm, "clip_scale": c.clip_scale, "skip": bool(c.skip)}
+        return {"sumsq": c.sumsq, "norm": c.norm, "clip_scale": c.clip_scale, "skip": bool(c.skip),
+                "t": int(c.t)}
 
     def _free_tables(self):
         for b in [self._partials] + [t[0] for t in self._tables.values()]:

@@ -55,24 +55,58 @@ class HybridOptimizer:
             muon_kw.update(device=True, si=si)   # here the GPU path is the only path
         adamw_kw = adamw_kw or dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.01)
         if no_decay is None:
-            no_decay = lambda n, p: (p.ndim == 1)          # noqa: E731  don't decay 1-D gains/biases
+            # don't decay 1-D gains/biases (hybrid.py:35-36), nor a router that the predicate leaves
+            # to AdamW: the resident models run it with wd = 0 (ancora/kernels/moe.py:603-604)
+            no_decay = lambda n, p: (p.ndim == 1 or "router" in n.lower())          # noqa: E731
 
-        # A matrix the predicate sends to Muon but whose dims are not multiples of 128 (the (H, E)
-        # router of a MoE model under `default_is_muon`) cannot enter the batched chain; the
-        # reference runs its Newton-Schulz on the host for those (`_ns_ok`,
-        # ancora/optim/muon.py:37-41), here it goes to AdamW, as in the resident models
-        # (ancora/kernels/moe.py:603-604).
+        # A 2-D matrix the predicate sends to Muon stays on Muon whatever its dims (lr, momentum,
+        # no decay: what the reference trains it with): one whose dims are not multiples of 128, the
+        # (H, E) router of a MoE model under `default_is_muon`, runs zero-padded through the same
+        # chain (see `Muon`) where the reference falls back to host Newton-Schulz (`_ns_ok`,
+        # ancora/optim/muon.py:37-41, 307).
         def _aligned(p):
             return p.shape[-2] % NTM == 0 and p.shape[-1] % NTM == 0
-        self.muon_names = [n for n, p in params.items() if is_muon(n, p) and _aligned(p)]
-        self.misaligned_to_adamw = [n for n, p in params.items() if is_muon(n, p) and not _aligned(p)]
+        self.muon_names = [n for n, p in params.items() if is_muon(n, p) and (_aligned(p) or p.ndim == 2)]
+        self.muon_padded = [n for n in self.muon_names if not _aligned(params[n])]
         self.adamw_names = [n for n in params if n not in self.muon_names]
         self.muon = Muon({n: params[n] for n in self.muon_names}, grad_dtype=grad_dtype, **muon_kw)
         self.adamw = AdamW({n: params[n] for n in self.adamw_names},
                            no_decay=tuple(n for n in self.adamw_names if no_decay(n, params[n])),
                            grad_dtype=grad_dtype, **adamw_kw)
         self.guard = StepGuard(max_grad_norm) if (max_grad_norm is not None or guard) else None
-        self.last_skipped = False
+        self._last_skipped = False
+        self._last_ctl = None
+        self._pending = None         # stream of an unsynchronised guarded step whose block was not read yet
+        self._t_upper = 0            # guarded steps issued: the device's step count cannot exceed it
+
+    # The guarded step counts its steps on the device (the guard's control block), so that a skipped
+    # step needs no undo and `step(..., sync=False)` returns without a host synchronisation. The
+    # host mirrors (`last_ctl`, `last_skipped`, the optimizers' `t`) are refreshed when the block
+    # is read: right away in a synchronous step, on first use after an asynchronous one.
+    def _refresh(self):
+        if self._pending is None:
+            return
+        si, self._pending = self._pending, None
+        self._last_ctl = self.guard.read(si)              # synchronises stream si
+        self._last_skipped = self._last_ctl["skip"]
+        self.adamw.t = self._last_ctl["t"]
+        if self.muon.engine is not None:
+            self.muon.engine.t = self._last_ctl["t"]
+
+    @property
+    def last_ctl(self):
+        self._refresh()
+        return self._last_ctl
+
+    @property
+    def last_skipped(self):
+        self._refresh()
+        return self._last_skipped
+
+    def step_count(self):
+        """Steps that passed the guard so far (reads the device block if a step is pending)."""
+        self._refresh()
+        return self.adamw.t
 
     def _grad_bufs(self, grads):
         """Gradient DevBufs in the fixed order of the global norm: Muon names, then AdamW names."""
@@ -93,9 +127,12 @@ class HybridOptimizer:
         self.guard.plan(bufs)
         return self.guard.partials_ptr((self.muon_names + self.adamw_names).index(name))
 
-    def step(self, grads, stream_int, produced=()):
+    def step(self, grads, stream_int, produced=(), sync=True):
         """`produced`: names of resident gradients whose grad-norm partial sums their producer has
-        already written (see `gn_partials_ptr`); same result bits with or without."""
+        already written (see `gn_partials_ptr`); same result bits with or without. `sync=False`
+        (guarded steps with resident gradients): return as soon as the step is queued on
+        `stream_int`, as the reference's resident step does (ancora/model/resident_train.py:338-339);
+        `last_ctl` / `last_skipped` then read the device block when first asked."""
         if self.guard is None:
             self.muon.step({n: grads[n] for n in self.muon_names}, stream_int)
             self.adamw.step({n: grads[n] for n in self.adamw_names}, stream_int)
@@ -106,9 +143,12 @@ class HybridOptimizer:
                 g = grads[n]
                 if not isinstance(g, DevBuf):
                     s = opt.st[n]
-                    g = np.asarray(g)
-                    if g.dtype != s["g"].dtype and s["g"].dtype == np.float32:
-                        g = g.astype(np.float32)
+                    if opt is self.muon:
+                        g = self.muon.host_grad(n, g)
+                    else:
+                        g = np.asarray(g)
+                        if g.dtype != s["g"].dtype and s["g"].dtype == np.float32:
+                            g = g.astype(np.float32)
                     s["g"].upload(g.reshape(s["g"].shape), stream_int)
         resident = {}
         for opt, names in ((self.muon, self.muon_names), (self.adamw, self.adamw_names)):
@@ -116,21 +156,24 @@ class HybridOptimizer:
                 g = grads[n]
                 resident[n] = g if isinstance(g, DevBuf) else opt.st[n]["g"]
         order = self.muon_names + self.adamw_names
-        self.guard.compute(self._grad_bufs(grads), stream_int, produced=[order.index(n) for n in produced])
+        if self._pending is not None and self._pending != stream_int:
+            self._refresh()                # the block is reused: an unread step on another stream first
+        self._t_upper += 1
+        self.guard.compute(self._grad_bufs(grads), stream_int, produced=[order.index(n) for n in produced],
+                           count_step=True)
         # Muon's per-shape chains fork onto their own streams; AdamW runs beside them
         self.muon.launch({n: resident[n] for n in self.muon_names}, stream_int, self.guard,
-                         defer_join=True)
-        self.adamw.launch({n: resident[n] for n in self.adamw_names}, stream_int, self.guard)
+                         defer_join=True, device_steps=True)
+        self.adamw.launch({n: resident[n] for n in self.adamw_names}, stream_int, self.guard,
+                          device_steps=True, t_upper=self._t_upper)
         self.muon.join(stream_int)
-        _lib.stream_sync(stream_int)
-        self.last_ctl = self.guard.read(stream_int)
-        self.last_skipped = self.last_ctl["skip"]
-        if self.last_skipped:
-            self.muon.unstep()
-            self.adamw.unstep()
+        self._pending = stream_int
+        if sync:
+            self._refresh()
 
     def state_dict(self):
         """Optimizer state of both groups as one flat {key: ndarray} mapping."""
+        self._refresh()
         out = {f"muon/{k}": v for k, v in self.muon.state_dict().items()}
         out.update({f"adamw/{k}": v for k, v in self.adamw.state_dict().items()})
         return out
@@ -138,6 +181,10 @@ class HybridOptimizer:
     def load_state_dict(self, sd, stream_int=0):
         self.muon.load_state_dict({k[5:]: v for k, v in sd.items() if k.startswith("muon/")}, stream_int)
         self.adamw.load_state_dict({k[6:]: v for k, v in sd.items() if k.startswith("adamw/")}, stream_int)
+        self._pending = None
+        if self.guard is not None:
+            self.guard.set_t(self.adamw.t, stream_int)
+            self._t_upper = self.adamw.t
         _lib.stream_sync(stream_int)
 
     def save(self, path):

@@ -20,7 +20,7 @@ import ctypes
 import numpy as np
 
 from . import _lib
-from ._lib import api, MuonDesc, F32, BF16, MUON_MAX_SCALES
+from ._lib import api, MuonDesc, F32, BF16, MUON_MAX_SCALES, SR_ON, SR_STEP_SEED
 from .bf16 import bf16_bits, bits_f32, bf16_round as _bf        # noqa: F401
 from .devbuf import DevBuf, upload_table
 from . import muon_ns
@@ -127,7 +127,8 @@ class MuonEngine:
             _check_aligned(K, N)
             w["tr"] = K > N
             w["M"], w["Nn"] = (N, K) if w["tr"] else (K, N)
-            w["scale"] = max(1.0, K / N) ** 0.5                  # ancora/optim/muon.py:232
+            if "scale" not in w:                                  # (a zero-padded weight brings its own)
+                w["scale"] = max(1.0, K / N) ** 0.5              # ancora/optim/muon.py:232
             w.setdefault("seed", idx)
             if w["scale"] not in scales:
                 scales.append(w["scale"])
@@ -181,14 +182,23 @@ class MuonEngine:
             return sum(b.U.nbytes + b.ws.nbytes() for b in self.batches)
         return (self.U.nbytes if self.U is not None else 0) + self.ws.nbytes()
 
-    def step(self, si, lr=0.02, schedule=_KELLER, guard=None, defer_join=False):
+    def step(self, si, lr=0.02, schedule=_KELLER, guard=None, defer_join=False, device_steps=False):
         """One Muon step over every weight. Asynchronous on stream `si`: the work is ordered
-        after everything already queued on `si`, and (unless defer_join) `si` waits for it."""
-        self.t += 1
+        after everything already queued on `si`, and (unless defer_join) `si` waits for it.
+        `device_steps`: the step count lives in the guard's control block (see `AdamW.launch`); the
+        kernels form the rounding seed from it and `t` here is left alone."""
         schedule = muon_ns._resolve(schedule)
         ctl = 0 if guard is None else guard.ptr
         lr_scales = (ctypes.c_float * MUON_MAX_SCALES)(*[lr * s for s in self.scales])
-        seed_base = ((self.seed + 1000003 * self.t) & 0xFFFFFFFF) if self.sr else 0
+        if device_steps:
+            if guard is None:
+                raise ValueError("MuonEngine.step: device_steps needs the guard whose block counts the steps")
+            self._sr_arg = (SR_ON | SR_STEP_SEED) if self.sr else 0
+            seed_base = self.seed & 0xFFFFFFFF
+        else:
+            self.t += 1
+            self._sr_arg = int(self.sr)
+            seed_base = ((self.seed + 1000003 * self.t) & 0xFFFFFFFF) if self.sr else 0
         coef = muon_ns.coef_array(schedule, self.ns)
         self._run_mode = muon_ns.effective_mode(self.mode, schedule)
         together = [b for b in self.batches
@@ -229,7 +239,7 @@ class MuonEngine:
                 api.anc_ns_batched(b.U.ptr, b.E, b.M, b.Nn, self.ns, coef, 1e-7,
                                    muon_ns.MODES[self._run_mode], buf.ptr, buf.nbytes, int(st))
             api.anc_muon_update_multi(b.table.ptr, b.E, b.total_blocks, lr_scales, F32,
-                                      int(self.sr), seed_base, ctl, int(st))
+                                      self._sr_arg, seed_base, ctl, int(st))
             if forked:
                 self._join[i].record(st)
         self._forked = forked
@@ -255,14 +265,14 @@ class MuonEngine:
         if self.fused_update and not any(w.get("p16T") is not None for b in group for w in b.weights):
             tables = (ctypes.c_uint64 * len(group))(*[b.table.ptr for b in group])
             api.anc_muon_ns_update_multi(probs, len(group), tables, self.ns, coef, 1e-7,
-                                         muon_ns.MODES[self._run_mode], lr_scales, int(self.sr), seed_base, ctl,
+                                         muon_ns.MODES[self._run_mode], lr_scales, self._sr_arg, seed_base, ctl,
                                          int(si))
             return
         api.anc_ns_batched_pair_multi(probs, len(group), self.ns, coef, 1e-7, muon_ns.MODES[self._run_mode],
                                       int(si))
         for b in group:
             api.anc_muon_update_multi(b.table.ptr, b.E, b.total_blocks, lr_scales, F32,
-                                      int(self.sr), seed_base, ctl, int(si))
+                                      self._sr_arg, seed_base, ctl, int(si))
 
     def join(self, si):
         """Make stream `si` wait for the per-batch streams of the last step."""
@@ -407,12 +417,25 @@ class BatchedProjMuon:
         self.engine.free()
 
 
+def _ceil_tile(n):
+    return (int(n) + NTM - 1) // NTM * NTM
+
+
 class Muon:
     """fp32-master Muon for 2-D matrix params (ancora/optim/muon.py:287-318). params:
     {name: (R,C) fp32 ndarray}; a 3-D [E,R,C] entry is E independent slices. The reference's host
     class runs Newton-Schulz on the CPU unless `device=True`; this one always runs on the GPU, so
     `device` and `si` are accepted and only `si` is used (as the default stream). `schedule`
-    defaults to the process-wide setting of `set_polar_express` (Keller unless switched)."""
+    defaults to the process-wide setting of `set_polar_express` (Keller unless switched).
+
+    A 2-D matrix whose dims are not multiples of 128 (the (H, E) router of a MoE model under the
+    default routing predicate) cannot enter the tiled chain as it is; the reference runs its
+    Newton-Schulz on the host for those (`_ns_ok`, ancora/optim/muon.py:37-41, 307). Here its
+    state lives zero-padded to the next multiples of 128: the padding rows and columns of the
+    iterate stay exactly zero through the chain (A = X X^T has zero rows there, B X as well), the
+    Frobenius norm does not see them, so the result is the Newton-Schulz of the matrix itself,
+    padded; the shape factor sqrt(max(1, rows/cols)) is that of the original dims. Such a matrix
+    takes host gradients (or a DevBuf already padded); accessors return the original shape."""
 
     def __init__(self, params, lr=0.02, momentum=0.95, nesterov=True, ns_steps=5, device=False,
                  si=None, schedule=_KELLER, mode="bf16", chunk=None, sr=False, seed=0,
@@ -425,19 +448,25 @@ class Muon:
         gdt = np.dtype(grad_dtype)
         for n, p in params.items():
             assert p.ndim in (2, 3), f"Muon is for 2D matrices, {n} is {p.shape}"
-            K, N = p.shape[-2], p.shape[-1]
-            _check_aligned(K, N, f"Muon weight '{n}'")
+            K0, N0 = p.shape[-2], p.shape[-1]
+            K, N = _ceil_tile(K0), _ceil_tile(N0)
+            pad = (K0, N0) if (K, N) != (K0, N0) else None
+            if pad is not None and p.ndim != 2:
+                _check_aligned(K0, N0, f"stacked Muon weight '{n}'")
             E = 1 if p.ndim == 2 else p.shape[0]
-            s = dict(shape=p.shape, E=E, K=K, N=N,
-                     p32=DevBuf(np.ascontiguousarray(p, dtype=np.float32).reshape(E * K, N)),
+            s = dict(shape=p.shape, E=E, K=K, N=N, pad=pad)
+            s.update(p32=DevBuf(self._padded(s, np.ascontiguousarray(p, dtype=np.float32)).reshape(E * K, N)),
                      p16=DevBuf.zeros((E * K, N), np.uint16),
                      buf=DevBuf.zeros((E * K, N), np.float32),
                      g=DevBuf.zeros((E * K, N), gdt))
             self.st[n] = s
             for e in range(E):
-                recs.append(dict(buf=s["buf"].at_pos(e * K), p32=s["p32"].at_pos(e * K),
-                                 p16=s["p16"].at_pos(e * K), G=s["g"].at_pos(e * K), K=K, N=N,
-                                 name=n, e=e))
+                r = dict(buf=s["buf"].at_pos(e * K), p32=s["p32"].at_pos(e * K),
+                         p16=s["p16"].at_pos(e * K), G=s["g"].at_pos(e * K), K=K, N=N,
+                         name=n, e=e)
+                if pad is not None:
+                    r["scale"] = max(1.0, K0 / N0) ** 0.5      # ancora/optim/muon.py:308, original dims
+                recs.append(r)
         self._recs = recs
         self._recs_of = {}
         for r in recs:
@@ -447,11 +476,44 @@ class Muon:
             if recs else None
         self.last_skipped = False
 
-    def launch(self, grads, stream_int=None, guard=None, defer_join=False):
+    @staticmethod
+    def _padded(s, a):
+        """Host array `a` of the parameter's own shape, zero-padded to the stored (K, N)."""
+        if s["pad"] is None:
+            return a
+        out = np.zeros((s["K"], s["N"]), a.dtype)
+        out[:s["pad"][0], :s["pad"][1]] = a.reshape(s["pad"])
+        return out
+
+    @staticmethod
+    def _unpadded(s, a):
+        a = a.reshape(s["E"] * s["K"], s["N"])
+        if s["pad"] is not None:
+            a = np.ascontiguousarray(a[:s["pad"][0], :s["pad"][1]])
+        return a.reshape(s["shape"])
+
+    def host_grad(self, n, g):
+        """A host gradient of parameter `n` as the array its device buffer takes: the buffer's
+        dtype, zero-padded where the state is."""
+        s = self.st[n]
+        g = np.asarray(g)
+        if g.dtype != s["g"].dtype:
+            if s["g"].dtype == np.float32:
+                g = g.astype(np.float32)
+            else:
+                raise TypeError(f"Muon: gradient of '{n}' is {g.dtype}, the optimizer was "
+                                f"built for {s['g'].dtype}")
+        return self._padded(s, g).reshape(s["E"] * s["K"], s["N"])
+
+    def launch(self, grads, stream_int=None, guard=None, defer_join=False, device_steps=False):
         si = stream_int if stream_int is not None else (self.si or 0)
         for n, s in self.st.items():
             g = grads[n]
             if isinstance(g, DevBuf):
+                if g.size != s["E"] * s["K"] * s["N"]:
+                    raise TypeError(f"Muon: the resident gradient of '{n}' has {g.size} elements; its state is "
+                                    f"stored as {(s['E'] * s['K'], s['N'])} (zero-padded to multiples of {NTM}): "
+                                    "pass a host gradient or a DevBuf padded the same way")
                 if self._gptr.get(n) != (g.ptr, g.dtype.str):
                     gv = g.view((s["E"] * s["K"], s["N"]))
                     for r in self._recs_of[n]:
@@ -462,16 +524,9 @@ class Muon:
                     for r in self._recs_of[n]:
                         r["G"] = s["g"].at_pos(r["e"] * s["K"])
                     del self._gptr[n]
-                g = np.asarray(g)
-                if g.dtype != s["g"].dtype:
-                    if s["g"].dtype == np.float32:
-                        g = g.astype(np.float32)
-                    else:
-                        raise TypeError(f"Muon: gradient of '{n}' is {g.dtype}, the optimizer was "
-                                        f"built for {s['g'].dtype}")
-                s["g"].upload(g.reshape(s["E"] * s["K"], s["N"]), si)
+                s["g"].upload(self.host_grad(n, g), si)
         if self.engine is not None:
-            self.engine.step(si, self.lr, self.schedule, guard, defer_join)
+            self.engine.step(si, self.lr, self.schedule, guard, defer_join, device_steps)
         return si
 
     def join(self, si):
@@ -512,17 +567,17 @@ class Muon:
 
     def weights(self):
         """bf16-valued fp32 weights for the forward (ancora/optim/muon.py:311-312)."""
-        return {n: _bf(s["p32"].to_numpy()).reshape(s["shape"]) for n, s in self.st.items()}
+        return {n: _bf(self._unpadded(s, s["p32"].to_numpy())) for n, s in self.st.items()}
 
     def weights16(self):
         """The device-maintained bf16 copy (RNE or SR of the master), as fp32 values."""
-        return {n: bits_f32(s["p16"].to_numpy()).reshape(s["shape"]) for n, s in self.st.items()}
+        return {n: bits_f32(self._unpadded(s, s["p16"].to_numpy())) for n, s in self.st.items()}
 
     def master(self):
-        return {n: s["p32"].to_numpy().reshape(s["shape"]) for n, s in self.st.items()}
+        return {n: self._unpadded(s, s["p32"].to_numpy()) for n, s in self.st.items()}
 
     def momentum_buffers(self):
-        return {n: s["buf"].to_numpy().reshape(s["shape"]) for n, s in self.st.items()}
+        return {n: self._unpadded(s, s["buf"].to_numpy()) for n, s in self.st.items()}
 
     def free(self):
         if self.engine is not None:

@@ -128,30 +128,41 @@ def ns_workspace_bytes(E, M, N, mode="bf16"):
     return int(n)
 
 
-def ns_flops(E, M, N, steps=5, mode="bf16"):
+def _acct_mode(mode, schedule):
+    """Mode of the accounting helpers: `schedule` is the schedule the chain ran under (resolved as
+    the drivers resolve it), so that mode="bf16" counts the plan it really ran; the default sentinel
+    leaves `mode` as given (pass "bf16_late3" etc. yourself)."""
+    return mode if schedule is _ASIS else effective_mode(mode, _resolve(schedule))
+
+
+_ASIS = object()
+
+
+def ns_flops(E, M, N, steps=5, mode="bf16", schedule=_ASIS):
     """(executed, dense) matrix-core FLOPs of one chain call over E (M,N) matrices."""
     _lib.load()
     ex, de = ctypes.c_double(0), ctypes.c_double(0)
-    api.anc_ns_flops(E, M, N, int(steps), MODES[mode], ctypes.byref(ex), ctypes.byref(de))
+    api.anc_ns_flops(E, M, N, int(steps), MODES[_acct_mode(mode, schedule)], ctypes.byref(ex), ctypes.byref(de))
     return ex.value, de.value
 
 
-def ns_hard_info(workspace_ptr, E, M, N, steps=5, mode="bf16", si=0):
+def ns_hard_info(workspace_ptr, E, M, N, steps=5, mode="bf16", si=0, schedule=_ASIS):
     """(n_gated, extra_flops) of the last chain call that used this workspace: how many of its E
     matrices took extra terms through a conditioning gate, and the matrix-core work they add,
-    all together, to `ns_flops`' executed count. Synchronises stream `si`."""
+    all together, to `ns_flops`' executed count. Synchronises stream `si`. `mode` (with `schedule`)
+    must name the mode that call ran in: the workspace layout depends on it."""
     n, ex = ctypes.c_int32(0), ctypes.c_double(0)
-    api.anc_ns_hard_info(int(workspace_ptr), int(E), int(M), int(N), MODES[mode], int(steps),
+    api.anc_ns_hard_info(int(workspace_ptr), int(E), int(M), int(N), MODES[_acct_mode(mode, schedule)], int(steps),
                          ctypes.byref(n), ctypes.byref(ex), int(si))
     return n.value, ex.value
 
 
-def ns_product_flops(E, M, N, k, product, steps=5, mode="bf16"):
+def ns_product_flops(E, M, N, k, product, steps=5, mode="bf16", schedule=_ASIS):
     """Executed matrix-core FLOPs of product 0 (A = X X^T), 1 (B = b A + c A A) or 2
     (X = a X + B X) of iteration k of a chain call."""
     ex = ctypes.c_double(0)
-    api.anc_ns_product_flops(int(E), int(M), int(N), int(steps), MODES[mode], int(k), int(product),
-                             ctypes.byref(ex))
+    api.anc_ns_product_flops(int(E), int(M), int(N), int(steps), MODES[_acct_mode(mode, schedule)], int(k),
+                             int(product), ctypes.byref(ex))
     return ex.value
 
 

@@ -15,14 +15,6 @@ targets, tests/hardware/_ncu_train_target.py:1-3,50-57).
     python3 -m ancora_cutile_amd.prof_target embed [V] [H] [TOKENS] [steps]  sorted-scatter embedding
                                       gradient + row-sparse AdamW step beside the dense AdamW sweep
                                       of the same table (prints us per call from HIP events)
-    python3 -m ancora_cutile_amd.prof_target copy [GiB] [reps]          streaming-kernel shapes
-                                      (anc_copy_shape): TB/s of each, the reference points for
-                                      the elementwise optimizer kernels
-
-    python3 -m ancora_cutile_amd.prof_target mfma [launches]            matrix-pipe reference (anc_mfma_rate):
-                                      TFLOP/s of the register-only matrix-instruction loop on zero,
-                                      constant and random operands, with the shader clock and package
-                                      power sysfs reports while each runs
 
 Each target allocates its operands, runs the kernel(s) `calls` times on the null stream and
 synchronises; nothing is checked here (parity lives in tests/).
@@ -56,45 +48,6 @@ def main(argv):
             pr = _lib.profile_read()
             _lib.profile_enable(False)
             print("  ".join(f"{k}={v[0]:.3f}ms/{v[1]}" for k, v in pr.items() if v[1]))
-    elif what == "mfma":
-        import threading
-        import time
-        launches = int(argv[1]) if len(argv) > 1 else 12
-        sink = DevBuf.empty((1024,), np.float32)
-
-        from .sysfs import sclk_mhz as sclk, power_w
-
-        for name, values in (("zeros", 0), ("constant", 1), ("random", 2), ("zeros", 0), ("random", 2)):
-            samples, watts, stop = [], [], threading.Event()
-
-            def poll():
-                time.sleep(0.5)
-                while not stop.is_set():
-                    v, w = sclk(), power_w()
-                    if v:
-                        samples.append(v)
-                    if w:
-                        watts.append(w)
-                    time.sleep(0.02)
-
-            th = threading.Thread(target=poll, daemon=True)
-            th.start()
-            fl = ctypes.c_double()
-            rates = []
-            for _ in range(launches):
-                e0, e1 = _lib.Event(), _lib.Event()
-                e0.record(0)
-                _lib.api.anc_mfma_rate(values, 400000, sink.ptr, ctypes.byref(fl), 0)
-                e1.record(0)
-                e1.sync()
-                rates.append(fl.value / (e0.elapsed_ms(e1) * 1e-3) / 1e12)
-            stop.set()
-            th.join(timeout=15)
-            busy = sorted(v for v in samples if v > 300)
-            med = lambda xs: xs[len(xs) // 2] if xs else None
-            print(f"{name:9s} first launch {rates[0]:7.1f}  last {rates[-1]:7.1f} TFLOP/s over {launches} launches; "
-                  f"sclk while running: median {med(busy)} MHz (min {busy[0] if busy else None}, max {busy[-1] if busy else None}, "
-                  f"{len(busy)} samples); package power median {med(sorted(watts))} W", flush=True)
     elif what == "adamw":
         n = int(argv[1]) // 64 * 64
         calls = int(argv[2]) if len(argv) > 2 else 3
@@ -225,28 +178,6 @@ def main(argv):
         print(f"  sorted-scatter gradient rows              {t_sc / steps * 1e3:8.1f} us")
         print(f"  row-sparse AdamW step                     {t_sp / steps * 1e3:8.1f} us (includes the 16-byte step-table upload)")
         print(f"  dense AdamW sweep of the same table       {t_de / steps * 1e3:8.1f} us ({28.0 * V * H / (t_de / steps) / 1e9:.2f} TB/s)")
-    elif what == "copy":
-        gib = float(argv[1]) if len(argv) > 1 else 1.0
-        reps = int(argv[2]) if len(argv) > 2 else 5
-        nb = int(gib * (1 << 30)) // (1 << 20) * (1 << 20)
-        a, b = DevBuf.empty((nb // 4,), np.float32), DevBuf.empty((nb // 4,), np.float32)
-        a.fill_zero(0)
-        b.fill_zero(0)
-        names = ("copy 4x16B nt", "copy 4x16B plain", "copy 8x16B nt", "copy persistent 2048 wg", "copy 1024-lane wg",
-                 "read only", "write only", "AdamW mix 4R+4W (14+14 B/elem)", "momentum mix 2R+3W (6+8 B/elem)")
-        e0, e1 = _lib.Event(), _lib.Event()
-        moved = ctypes.c_int64(0)
-        print(f"two buffers of {nb / 2 ** 30:.2f} GiB, {reps} launches each, HIP events around the launches")
-        for shape, name in enumerate(names):
-            _lib.api.anc_copy_shape(b.ptr, a.ptr, nb, shape, ctypes.byref(moved), 0)
-            e0.record(0)
-            for _ in range(reps):
-                _lib.api.anc_copy_shape(b.ptr, a.ptr, nb, shape, ctypes.byref(moved), 0)
-            e1.record(0)
-            e1.sync()
-            ms = e0.elapsed_ms(e1) / reps
-            print(f"  shape {shape}  {name:34s} {moved.value / 1e9:7.3f} GB in {ms * 1e3:8.1f} us = "
-                  f"{moved.value / ms / 1e9:6.3f} TB/s = {moved.value / ms / 1e9 / 8 * 100:5.1f} % of 8 TB/s")
     else:
         raise SystemExit(__doc__)
     _lib.api.anc_device_sync()

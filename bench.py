@@ -16,7 +16,10 @@ Prints ONE JSON line. `value` is milliseconds per step (lower is better). `roofl
 dominant kernel, the bf16 matrix-core GEMM of the Newton-Schulz chain: executed FLOPs over
 the summed duration of its launches, measured with HIP events on the launch stream, against
 the 2.5 PFLOP/s dense bf16 peak. `cpu_baseline` times the numpy restatement of the
-reference's host path on a bounded sample and scales it to the full step.
+reference's host path on a bounded sample and scales it to the full step. `configs` holds the
+other BASELINE configurations measured in the same run (the Newton-Schulz chain alone, the MoE
+family, the flat AdamW buffer) and config 2 under Keller's coefficients and on gradients that
+send every matrix through the chain's wide gate; `--no-configs` skips them.
 """
 import argparse
 import json
@@ -97,102 +100,6 @@ def sustained_sclk(run_steps, seconds=1.5):
             round(watts[len(watts) // 2], 1) if watts else None)
 
 
-def _median_power(fn, seconds, settle=0.5):
-    """(median package power in W, ms per call) while `fn()` is called back to back for `seconds`."""
-    import threading
-    from ancora_cutile_amd import _lib
-    from ancora_cutile_amd.sysfs import power_w
-    watts, stop = [], threading.Event()
-
-    def poll():
-        time.sleep(settle)
-        while not stop.is_set():
-            w = power_w()
-            if w:
-                watts.append(w)
-            time.sleep(0.01)
-
-    th = threading.Thread(target=poll, daemon=True)
-    th.start()
-    e0, e1 = _lib.Event(), _lib.Event()
-    n, t0 = 0, time.perf_counter()
-    e0.record(0)
-    while time.perf_counter() - t0 < seconds:
-        fn()
-        n += 1
-        if n % 4 == 0:
-            _lib.stream_sync(0)
-    e1.record(0)
-    e1.sync()
-    stop.set()
-    th.join(timeout=5)
-    watts.sort()
-    return (watts[len(watts) // 2] if watts else None), e0.elapsed_ms(e1) / max(1, n)
-
-
-def power_reference(_lib, DevBuf):
-    """Energy prices of the board's two resources, from package power (sysfs) while one of them runs
-    alone: pJ per HBM byte from the 1 GiB copy kernel on random data, pJ per matrix-core FLOP from
-    the register-only loop on random operands, each above the idle power. None without sysfs."""
-    import ctypes
-    _lib.stream_sync(0)
-    idle, _ = _median_power(lambda: time.sleep(0.02), 0.8, settle=0.3)
-    if idle is None:
-        return None
-    n = 1 << 28
-    src, dst = DevBuf.empty((n,), np.float32), DevBuf.empty((n,), np.float32)
-    seed = DevBuf(np.random.default_rng(11).standard_normal(1 << 24).astype(np.float32))
-    for i in range(n >> 24):
-        _lib.api.anc_copy_kernel(src.ptr + (i << 26), seed.ptr, 1 << 26, 0)
-    copy_w, copy_ms = _median_power(lambda: _lib.api.anc_copy_kernel(dst.ptr, src.ptr, 1 << 30, 0), 1.5)
-    for b in (src, dst, seed):
-        b.free()
-    sink, fl = DevBuf.empty((1024,), np.float32), ctypes.c_double()
-    mfma_w, mfma_ms = _median_power(lambda: _lib.api.anc_mfma_rate(2, 100000, sink.ptr, ctypes.byref(fl), 0), 1.5)
-    sink.free()
-    copy_bps, mfma_fps = 2.0 * (1 << 30) / (copy_ms * 1e-3), fl.value / (mfma_ms * 1e-3)
-    return {"idle_w": idle, "copy_w": copy_w, "copy_tbps": round(copy_bps / 1e12, 2),
-            "pj_per_hbm_byte": round((copy_w - idle) / copy_bps * 1e12, 1),
-            "mfma_random_w": mfma_w, "mfma_random_tflops": round(mfma_fps / 1e12, 1),
-            "pj_per_flop": round((mfma_w - idle) / mfma_fps * 1e12, 3)}
-
-
-def power_model(ref, step_w, traffic, launches, executed, gemm_ms):
-    """The GEMM launches of a step priced in energy: HBM bytes at the copy kernel's pJ per byte plus
-    executed FLOPs at the register loop's pJ per FLOP, and the time that energy takes at the power
-    the step draws above idle. `frac` = that time / the measured time: how much of the launches'
-    time the two resources' energy alone accounts for under the package limit."""
-    if not ref or not step_w or not traffic or not gemm_ms:
-        return None
-    joule = traffic * launches * ref["pj_per_hbm_byte"] * 1e-12 + executed * ref["pj_per_flop"] * 1e-12
-    ms_min = joule / (step_w - ref["idle_w"]) * 1e3
-    return {**ref, "step_w": step_w, "gemm_joule_per_step": round(joule, 2),
-            "gemm_ms_at_step_power": round(ms_min, 3), "gemm_ms_measured": round(gemm_ms, 3),
-            "frac": round(ms_min / gemm_ms, 4),
-            "note": "energy balance, context only: roofline.traffic x launches at the copy kernel's energy per byte "
-                    "+ executed FLOPs at the register loop's energy per FLOP (random operands), divided by the "
-                    "power the step draws above idle (idle_w is read right after load, clocks still up)"}
-
-
-def mfma_reference(_lib, DevBuf):
-    """TFLOP/s of the register-only matrix-instruction loop (anc_mfma_rate) on zero and on random
-    operands: what the matrix pipe sustains on this board without any memory traffic."""
-    import ctypes
-    sink = DevBuf.empty((1024,), np.float32)
-    out = {}
-    for name, values in (("zeros", 0), ("random", 2)):
-        fl = ctypes.c_double()
-        _lib.api.anc_mfma_rate(values, 20000, sink.ptr, ctypes.byref(fl), 0)      # clocks settle
-        e0, e1 = _lib.Event(), _lib.Event()
-        e0.record(0)
-        _lib.api.anc_mfma_rate(values, 400000, sink.ptr, ctypes.byref(fl), 0)
-        e1.record(0)
-        e1.sync()
-        out[name] = round(fl.value / (e0.elapsed_ms(e1) * 1e-3) / 1e12, 1)
-    sink.free()
-    return out
-
-
 def gemm_bytes_from_counter_db(path, ctr):
     """(bytes per k_ns_gemm_big launch, launches, KiB per count) from a rocprofv3 results database
     that holds counter `ctr` for the GEMM launches and for the 1 GiB copy kernel of the same run
@@ -226,7 +133,7 @@ def measure_gemm_traffic(workload):
     for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
         cmd = ["rocprofv3", "--pmc", ctr, "-d", os.path.join(top, ctr), "-o", ctr, "--",
                "python3", os.path.abspath(__file__), "--workload", workload, "--serial", "--steps", "3",
-               "--warmup", "1", "--no-cpu", "--no-clock"]
+               "--warmup", "1", "--no-cpu", "--no-clock", "--no-configs"]
         log(" ".join(cmd))
         pr = subprocess.Popen(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, start_new_session=True,
                               stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
@@ -310,6 +217,222 @@ def cpu_baseline(shapes, lr_adam=3e-4):
                       f"{len(os.sched_getaffinity(0))} usable, BLAS threads {threads}"}
 
 
+def ns_config(steps):
+    """BASELINE config 3: the 196 Newton-Schulz matrices of the Qwen3-0.6B set through the fp32-input
+    chain entry, group by group, in the bf16 matrix-core mode and in the fp32 validation mode."""
+    from ancora_cutile_amd import DevBuf, PE_SCHEDULE, _lib
+    from ancora_cutile_amd.muon_ns import ns_batched, ns_flops
+    e0, e1 = _lib.Event(), _lib.Event()
+    groups = ((1024, 1024, 56), (1024, 2048, 56), (1024, 3072, 84))
+    res = {}
+    for mode in ("bf16", "fp32"):
+        k = steps if mode == "bf16" else 1
+        total_ms, ex_t, de_t = 0.0, 0.0, 0.0
+        for (M, N, E) in groups:
+            one = np.random.default_rng(M + N).standard_normal((M, N)).astype(np.float32)
+            X = DevBuf.empty((E * M, N), np.float32)
+            for e in range(E):
+                X.at_pos(e * M).upload(one)
+            ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
+            e0.record(0)
+            for _ in range(k):
+                ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
+            e1.record(0)
+            e1.sync()
+            total_ms += e0.elapsed_ms(e1) / k
+            ex, de = ns_flops(E, M, N, 5, mode)
+            ex_t += ex
+            de_t += de
+            X.free()
+        res[mode] = {"ms": round(total_ms, 3), "executed_tflop": round(ex_t / 1e12, 3),
+                     "dense_tflop": round(de_t / 1e12, 3),
+                     "executed_tflops_per_s": round(ex_t / total_ms / 1e9, 1)}
+    return res, groups
+
+
+def adamw_flat_config(steps, warmup):
+    """BASELINE config 5, clean-gradient variant: grad-norm + clip + AdamW + stochastic bf16 downcast
+    over one flat 1.2e9-element buffer, step counter at 1000."""
+    import ctypes
+    from ancora_cutile_amd import DevBuf, StepGuard, _lib
+    from ancora_cutile_amd.adamw import hyper_div
+    from ancora_cutile_amd.bf16 import bf16_bits
+    e0, e1 = _lib.Event(), _lib.Event()
+    n = 1_200_000_000
+    rng = np.random.default_rng(0)
+    chunk = bf16_bits(1e-3 * rng.standard_normal(1 << 24, dtype=np.float32))
+    g = DevBuf.empty((n,), np.uint16)
+    for off in range(0, n, 1 << 24):
+        k = min(1 << 24, n - off)
+        DevBuf(shape=(k,), dtype=np.uint16, ptr=g.ptr + 2 * off).upload(chunk[:k])
+    m, v, p = (DevBuf.zeros((n,), np.float32) for _ in range(3))
+    p16 = DevBuf.zeros((n,), np.uint16)
+    guard = StepGuard(1.0)
+
+    def step(t):
+        guard.compute([g], 0)
+        h = hyper_div(3e-4, 0.9, 0.95, 1e-8, 1000 + t, sr=True, seed_base=t)
+        _lib.api.anc_adamw(g.ptr, m.ptr, v.ptr, p.ptr, p16.ptr, n, _lib.BF16, ctypes.byref(h), 0.1, 0,
+                           guard.ptr, 0)
+    for t in range(warmup):
+        step(t)
+    e0.record(0)
+    for t in range(steps):
+        step(t)
+    e1.record(0)
+    e1.sync()
+    ms = e0.elapsed_ms(e1) / steps
+    _lib.profile_enable(True)
+    step(0)
+    pr = _lib.profile_read()
+    _lib.profile_enable(False)
+    a_ms, g_ms = pr["adamw"][0], pr["gradnorm_partials"][0]
+    out = {"elements": n, "ms": ms, "gbps": round(30.0 * n / (ms * 1e-3) / 1e9, 1),
+           "frac": round(30.0 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+           "adamw_kernel": {"ms": round(a_ms, 3), "gbps": round(28.0 * n / (a_ms * 1e-3) / 1e9, 1)},
+           "gradnorm_kernel": {"ms": round(g_ms, 3), "gbps": round(2.0 * n / (g_ms * 1e-3) / 1e9, 1)},
+           "clip_scale": guard.read(0)["clip_scale"]}
+    for b in (g, m, v, p, p16):
+        b.free()
+    guard.free()
+    return out
+
+
+GEMM_KINDS = ("ns_gemm_gram", "ns_gemm_bmat", "ns_gemm_bx", "ns_gemm_bx_update")
+
+
+def chain_work(opt, schedule):
+    """(executed FLOPs, dense FLOPs, matrices that took a conditioning gate) of the optimizer's last
+    step, from the plan of the mode it ran in and the gate decisions left in the workspaces."""
+    from ancora_cutile_amd.muon_ns import ns_flops, ns_hard_info
+    executed = dense = 0.0
+    hard = 0
+    for b in opt.muon.engine.batches:
+        ex, de = ns_flops(b.E, b.M, b.Nn, 5, "bf16", schedule=schedule)
+        nh, extra = ns_hard_info(b.ws.buf.ptr, b.E, b.M, b.Nn, 5, "bf16", schedule=schedule)
+        executed += ex + extra
+        dense += de
+        hard += nh
+    return executed, dense, hard
+
+
+def hybrid_config(opt, gdev, schedule, steps=5, warmup=2):
+    """A compact measurement of the hybrid step as `opt` stands: ms per step over `steps` steps
+    (HIP events, steps queued without host synchronisation), and the matrix-core GEMM launches'
+    summed duration and executed work from one step under the per-launch event timer."""
+    from ancora_cutile_amd import _lib
+    for _ in range(warmup):
+        opt.step(gdev, 0)
+    _lib.api.anc_device_sync()
+    t_before = opt.step_count()
+    e0, e1 = _lib.Event(), _lib.Event()
+    e0.record(0)
+    for _ in range(steps):
+        opt.step(gdev, 0, sync=False)
+    e1.record(0)
+    e1.sync()
+    ms = e0.elapsed_ms(e1) / steps
+    if opt.step_count() != t_before + steps:
+        raise RuntimeError("the guard skipped a timed step (non-finite gradient norm)")
+    opt.muon.engine.serial = True
+    opt.step(gdev, 0)
+    _lib.profile_enable(True)
+    opt.step(gdev, 0)
+    prof = _lib.profile_read()
+    _lib.profile_enable(False)
+    opt.muon.engine.serial = False
+    gemm_ms = sum(prof[k][0] for k in GEMM_KINDS)
+    executed, dense, hard = chain_work(opt, schedule)
+    tf = executed / (gemm_ms * 1e-3) / 1e12
+    return {"ms": round(ms, 3), "ns_gemm_ms": round(gemm_ms, 3), "executed_tflop": round(executed / 1e12, 3),
+            "dense_tflop": round(dense / 1e12, 3), "ns_gemm_tflops_per_s": round(tf, 1),
+            "ns_gemm_frac": round(tf / PEAK_BF16_TFLOPS, 4),
+            "muon_matrices": sum(b.E for b in opt.muon.engine.batches), "gated_hard_matrices": hard}
+
+
+def wide_spectrum_grad(K, N, rng, decades=3.0):
+    """(K, N) bf16 gradient whose singular values are log-uniform over `decades` decades: the kind of
+    input the chain's wide gate exists for (every residual term from iteration 1 on)."""
+    from ancora_cutile_amd.bf16 import bf16_bits
+    M, L = min(K, N), max(K, N)
+    U, _ = np.linalg.qr(rng.standard_normal((M, M)).astype(np.float32))
+    V, _ = np.linalg.qr(rng.standard_normal((L, M)).astype(np.float32))
+    sv = np.logspace(0.0, -decades, M).astype(np.float32)
+    G = (U * sv) @ V.T                                    # (M, L)
+    G = (1e-3 * np.sqrt(M * L) / np.linalg.norm(G)) * G    # entries of the size of the other gradients
+    return bf16_bits(np.ascontiguousarray(G.T if K > N else G).astype(np.float32)).reshape(K, N)
+
+
+def other_configs(opt, gdev, args):
+    """The non-headline numbers, measured in the same run: config 2 under the reference's default
+    schedule (Keller) and on gradients that send every matrix through the wide gate, then configs
+    4, 3 and 5. `opt` (the headline optimizer) is freed on the way."""
+    from ancora_cutile_amd import HybridOptimizer, PE_SCHEDULE, _lib
+    from ancora_cutile_amd.hybrid import resident_is_muon
+    from ancora_cutile_amd.shapes import moe_shapes
+    cfg = {}
+    # config 2 under Keller's coefficients: the host layer runs the chain in its late-3 plan
+    opt.muon.schedule = None
+    r = hybrid_config(opt, gdev, None)
+    r["note"] = ("config 2, the reference's default schedule (Keller, ancora/kernels/muon_ns.py:21,51-65): "
+                 "the chain runs its bf16_late3 plan")
+    cfg["c2_keller"] = r
+    opt.muon.schedule = PE_SCHEDULE
+    log(f"configs: c2_keller {r['ms']} ms")
+    # config 2 with a three-decade spectrum in every Muon gradient: every matrix takes the wide gate
+    rng = np.random.default_rng(5)
+    by_shape = {}
+    for n in opt.muon_names:
+        s = opt.muon.st[n]
+        K, N = s["K"], s["N"]
+        if (K, N) not in by_shape:
+            by_shape[(K, N)] = wide_spectrum_grad(K, N, rng)
+        s["g"].upload(by_shape[(K, N)])
+        s["buf"].fill_zero(0)
+    r = hybrid_config(opt, gdev, PE_SCHEDULE)
+    r["note"] = ("config 2 with singular values log-uniform over three decades in every Muon gradient "
+                 "(momentum buffers zeroed first): the worst-case Polar-Express step")
+    cfg["c2_all_wide_gate"] = r
+    log(f"configs: c2_all_wide_gate {r['ms']} ms, {r['gated_hard_matrices']} of {r['muon_matrices']} gated")
+    opt.free()
+    # config 4: the 16-layer MoE family
+    shapes = moe_shapes(layers=16)
+    params, grads = synth(shapes)
+    n_params = sum(p.size for p in params.values())
+    mo = HybridOptimizer(params, is_muon=resident_is_muon,
+                         muon_kw=dict(lr=0.02, momentum=0.95, ns_steps=5, schedule=PE_SCHEDULE, sr=True, seed=1),
+                         adamw_kw=dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.1, sr=True, seed=2),
+                         max_grad_norm=1.0, grad_dtype=np.uint16)
+    del params
+    gd = {}
+    for part, names in ((mo.muon, mo.muon_names), (mo.adamw, mo.adamw_names)):
+        for n in names:
+            st = part.st[n]
+            st["g"].upload(grads[n].reshape(st["g"].shape))
+            gd[n] = st["g"]
+    del grads
+    r = hybrid_config(mo, gd, PE_SCHEDULE)
+    r["params"] = n_params
+    r["note"] = "config 4: 16 layers alternating dense / MoE (E = 16), grad-norm + clip + Muon + AdamW"
+    cfg["c4_moe_16l"] = r
+    log(f"configs: c4_moe_16l {r['ms']} ms")
+    mo.free()
+    # config 3: the Newton-Schulz chain alone, both modes
+    res, _ = ns_config(3)
+    cfg["c3_ns_196"] = {"bf16_ms": res["bf16"]["ms"], "fp32_ms": res["fp32"]["ms"],
+                        "bf16_executed_tflops_per_s": res["bf16"]["executed_tflops_per_s"],
+                        "fp32_tflops_per_s": res["fp32"]["executed_tflops_per_s"],
+                        "note": "config 3: 196 matrices through the fp32-input chain entry, 5 Polar-Express steps"}
+    log(f"configs: c3_ns_196 {res['bf16']['ms']} / {res['fp32']['ms']} ms")
+    # config 5: the flat AdamW buffer
+    r = adamw_flat_config(5, 2)
+    cfg["c5_adamw_flat"] = {"ms": round(r["ms"], 3), "gbps": r["gbps"], "frac_of_8tbps": r["frac"],
+                            "adamw_kernel": r["adamw_kernel"], "gradnorm_kernel": r["gradnorm_kernel"],
+                            "note": "config 5, clean gradients: 1.2e9 elements, 30 B per element"}
+    log(f"configs: c5_adamw_flat {r['ms']:.3f} ms")
+    return cfg
+
+
 def side_workload(args):
     """Configs 3 and 5 as stand-alone timings (same JSON shape, their own metric names)."""
     from ancora_cutile_amd import DevBuf, StepGuard, PE_SCHEDULE, _lib
@@ -318,30 +441,7 @@ def side_workload(args):
     info = _lib.device_info()
     e0, e1 = _lib.Event(), _lib.Event()
     if args.workload == "ns":
-        groups = ((1024, 1024, 56), (1024, 2048, 56), (1024, 3072, 84))
-        res = {}
-        for mode in ("bf16", "fp32"):
-            steps = args.steps if mode == "bf16" else 1
-            total_ms, ex_t, de_t = 0.0, 0.0, 0.0
-            for (M, N, E) in groups:
-                one = np.random.default_rng(M + N).standard_normal((M, N)).astype(np.float32)
-                X = DevBuf.empty((E * M, N), np.float32)
-                for e in range(E):
-                    X.at_pos(e * M).upload(one)
-                ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
-                e0.record(0)
-                for _ in range(steps):
-                    ns_batched(X, E, M, N, 0, schedule=PE_SCHEDULE, mode=mode)
-                e1.record(0)
-                e1.sync()
-                total_ms += e0.elapsed_ms(e1) / steps
-                ex, de = ns_flops(E, M, N, 5, mode)
-                ex_t += ex
-                de_t += de
-                X.free()
-            res[mode] = {"ms": round(total_ms, 3), "executed_tflop": round(ex_t / 1e12, 3),
-                         "dense_tflop": round(de_t / 1e12, 3),
-                         "executed_tflops_per_s": round(ex_t / total_ms / 1e9, 1)}
+        res, groups = ns_config(args.steps)
         out = {"metric": "196-matrix Newton-Schulz chain ms (5 x Polar-Express)", "value": res["bf16"]["ms"],
                "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": 1, "ms_per_step": res["bf16"]["ms"],
                "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
@@ -455,49 +555,16 @@ def side_workload(args):
                                          "gbps": round(tr_bytes / (tr_ms * 1e-3) / 1e9, 1),
                                          "note": "what a caller of the x^T form pays on top: x (T,K) -> x^T (K,T) once per group of weights sharing x; never in value"}}
     else:
-        n = 1_200_000_000
-        rng = np.random.default_rng(0)
-        from ancora_cutile_amd.bf16 import bf16_bits
-        chunk = bf16_bits(1e-3 * rng.standard_normal(1 << 24, dtype=np.float32))
-        g = DevBuf.empty((n,), np.uint16)
-        for off in range(0, n, 1 << 24):
-            k = min(1 << 24, n - off)
-            DevBuf(shape=(k,), dtype=np.uint16, ptr=g.ptr + 2 * off).upload(chunk[:k])
-        m, v, p = (DevBuf.zeros((n,), np.float32) for _ in range(3))
-        p16 = DevBuf.zeros((n,), np.uint16)
-        guard = StepGuard(1.0)
-        import ctypes
-        from ancora_cutile_amd.adamw import hyper_div
-
-        def step(t):
-            guard.compute([g], 0)
-            h = hyper_div(3e-4, 0.9, 0.95, 1e-8, 1000 + t, sr=True, seed_base=t)
-            _lib.api.anc_adamw(g.ptr, m.ptr, v.ptr, p.ptr, p16.ptr, n, _lib.BF16, ctypes.byref(h), 0.1, 0,
-                               guard.ptr, 0)
-        for t in range(args.warmup):
-            step(t)
-        e0.record(0)
-        for t in range(args.steps):
-            step(t)
-        e1.record(0)
-        e1.sync()
-        ms = e0.elapsed_ms(e1) / args.steps
-        _lib.profile_enable(True)
-        step(0)
-        pr = _lib.profile_read()
-        _lib.profile_enable(False)
-        a_ms, g_ms = pr["adamw"][0], pr["gradnorm_partials"][0]
+        r = adamw_flat_config(args.steps, args.warmup)
+        n, ms = r["elements"], r["ms"]
         out = {"metric": "flat 1.2e9-element grad-norm + clip + AdamW + SR downcast ms", "value": round(ms, 3),
                "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
                "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
                "data": "synthetic", "config": {"workload": "adamw-flat-1.2e9", "step": 1000},
-               "roofline": {"bound": "hbm", "achieved": round(30.0 * n / (ms * 1e-3) / 1e9, 1),
-                            "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                            "frac": round(30.0 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "traffic": None,
-                            "bytes_per_elem": 30},
-               "adamw_kernel": {"ms": round(a_ms, 3), "gbps": round(28.0 * n / (a_ms * 1e-3) / 1e9, 1)},
-               "gradnorm_kernel": {"ms": round(g_ms, 3), "gbps": round(2.0 * n / (g_ms * 1e-3) / 1e9, 1)},
-               "clip_scale": guard.read(0)["clip_scale"]}
+               "roofline": {"bound": "hbm", "achieved": r["gbps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                            "frac": r["frac"], "traffic": None, "bytes_per_elem": 30},
+               "adamw_kernel": r["adamw_kernel"], "gradnorm_kernel": r["gradnorm_kernel"],
+               "clip_scale": r["clip_scale"]}
     out["device"] = {"name": info["name"] or info["arch"].split(":")[0], "arch": info["arch"], "cus": info["cu_count"]}
     print(json.dumps(out), flush=True)
 
@@ -509,8 +576,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=28, help=argparse.SUPPRESS)   # smaller sets for debugging
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the `configs` block (configs 3, 4, 5 and the two other config-2 steps)")
     ap.add_argument("--no-clock", action="store_true",
-                    help="skip the sustained-clock sampling and the matrix-pipe reference launches")
+                    help="skip the sustained-clock sampling")
     ap.add_argument("--traffic", action="store_true",
                     help="measure roofline.traffic now: two extra runs of this script under rocprofv3 --pmc "
                          "(about a minute); without it the figure recorded under profiles/ is reported while "
@@ -597,18 +666,20 @@ def main():
         opt.step(gdev, 0)
     _lib.api.anc_device_sync()
     e0, e1 = _lib.Event(), _lib.Event()
+    t_before = opt.step_count()
     t0 = time.perf_counter()
     e0.record(0)
-    skipped = 0
     for _ in range(args.steps):
-        opt.step(gdev, 0)
-        skipped += int(opt.last_skipped)
+        # queued without a host synchronisation: the steps are counted on the device, the guard's
+        # block is read once, after the timed region
+        opt.step(gdev, 0, sync=False)
     e1.record(0)
     e1.sync()
     _lib.api.anc_device_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    skipped = t_before + args.steps - opt.step_count()
     if skipped:       # a skipped step returns early from every kernel and would time as falsely fast
         sys.exit(f"bench.py: the guard skipped {skipped} of {args.steps} timed steps (non-finite gradient norm)")
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ev_ms = e0.elapsed_ms(e1) / args.steps
     ms_per_step = max(wall_ms, ev_ms)
     ctl = opt.last_ctl
@@ -648,8 +719,6 @@ def main():
         _lib.stream_sync(0)
 
     sclk, watts = (None, None) if args.no_clock else sustained_sclk(run_steps)
-    mfma_ref = {} if args.no_clock else mfma_reference(_lib, DevBuf)
-    power_ref = None if args.no_clock else power_reference(_lib, DevBuf)
 
     # every launch of k_ns_gemm_big; with the fused update one of them (kind ns_gemm_bx_update, the
     # last X = a X + B X) also reads and writes the weights
@@ -723,12 +792,9 @@ def main():
                                                      "avg_launch_ms": round(pure_ms / max(1, pure_launches), 4)},
                      "avg_launch_ms": round(gemm_ms / max(1, gemm_launches), 4),
                      # context, not the fraction asked for: the board holds `sustained_sclk_mhz`, not
-                     # its nominal clock, under the step's load, and its matrix pipe alone (registers
-                     # only) sustains `mfma_register_loop_tflops.random` on operands that vary
+                     # its nominal clock, under the step's load
                      "frac_of_peak_at_sustained_clock": (round(achieved / (PEAK_BF16_TFLOPS * sclk * 1e3 / info["clock_khz"]), 4)
                                                          if sclk and info["clock_khz"] else None),
-                     "frac_of_register_loop_on_random_operands": (round(achieved / mfma_ref["random"], 4)
-                                                                  if mfma_ref.get("random") else None),
                      "executed_tflop_per_step": round(executed / 1e12, 3),
                      "executed_counts": "what the kernels multiply: residual and gated terms, and of the symmetric "
                                         "products the 256x256 tiles on or below the diagonal, each in full "
@@ -753,16 +819,18 @@ def main():
         "kernel_ms_per_step": {k: round(v, 4) for k, v in kind_ms.items()},
         "event_ms_per_step": round(ev_ms, 3), "wall_ms_per_step": round(wall_ms, 3),
         "streams": "serial" if args.serial else "one: the Newton-Schulz chains of all shape groups advance together (grouped launches)",
+        "host_sync": "none inside the timed region: the steps are counted on the device and queued back to back",
         "copy_kernel_gbps": round(copy_gbps, 1),
         "sustained_sclk_mhz": sclk,
         "sustained_power_w": watts,
-        "mfma_register_loop_tflops": mfma_ref,
-        "power_model": power_model(power_ref, watts, traffic, gemm_launches, executed, gemm_ms),
         "grad_norm": ctl["norm"], "clip_scale": ctl["clip_scale"],
         "device": {"name": info["name"] or info["arch"].split(":")[0], "arch": info["arch"], "cus": info["cu_count"],
                    "clock_khz": info["clock_khz"]},
     }
-    opt.free()
+    if args.workload == "qwen3" and args.layers == 28 and not args.no_configs:
+        out["configs"] = other_configs(opt, gdev, args)        # frees opt on the way
+    else:
+        opt.free()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(shapes)
     print(json.dumps(out), flush=True)

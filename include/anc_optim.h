@@ -89,25 +89,6 @@ int anc_event_elapsed_ms(uint64_t start, uint64_t stop, float *ms);
 /* Plain streaming copy kernel of n_bytes (multiple of 16): the calibration
  * reference for HBM traffic counters and the measured copy ceiling. */
 int anc_copy_kernel(uint64_t dst, uint64_t src, int64_t n_bytes, uint64_t stream);
-/* The same streaming traffic in other kernel shapes, to establish what an elementwise kernel can
- * reach on this memory system (no reference counterpart; the reference's own method is a timed
- * copy beside its AdamW kernel, tests/hardware/_probe_adamw_bw.py:24-25,58-91). shape: 0 as
- * anc_copy_kernel; 1 ordinary instead of non-temporal accesses; 2 eight 16-byte accesses in
- * flight per lane; 3 2048 persistent workgroups, grid-stride; 4 1024 lanes per workgroup; 5 read
- * only; 6 write only; 7 AdamW's access mix without its arithmetic (four read streams of 2+4+4+4
- * and four write streams of 4+4+4+2 bytes per element, same block and lane layout); 8 the Muon
- * momentum kernel's mix (read 2+4, write 4+2+2). n_bytes (a multiple of 1 MiB) is the size of
- * each of the two buffers; *bytes_moved receives the bytes read plus written. */
-int anc_copy_shape(uint64_t dst, uint64_t src, int64_t n_bytes, int shape, int64_t *bytes_moved,
-                   uint64_t stream);
-/* The matrix pipe's counterpart of anc_copy_shape (no reference counterpart): `iters` rounds of 16
- * v_mfma_f32_32x32x16_bf16 on register operands per wavefront, eight wavefronts on every CU, no
- * memory traffic. values: 0 zeros, 1 one constant pair, 2 pseudo-random bf16 values. The board
- * runs under a power limit and the rate it sustains depends on the operand values, so this is
- * the ceiling a GEMM K loop has on this board with such operands, next to the nominal
- * 2.5 PFLOP/s. sink: device buffer of at least 2 KiB (never written); *flops receives the
- * floating-point operations of the launch; time it with events around the call. */
-int anc_mfma_rate(int values, int64_t iters, uint64_t sink, double *flops, uint64_t stream);
 
 /* ------------------------------------------------------------- profiling ----
  * Per-kernel timing with HIP events on the launch stream, for the benchmarks (the
@@ -145,14 +126,29 @@ int anc_profile_read(float *ms /* [ANC_PROF_KINDS] */, int64_t *launches /* [ANC
  * No reference counterpart: the reference has no grad-norm, clip or non-finite
  * guard (its closest pattern is the single-block fixed-order reduction of
  * ancora/kernels/muon_ns.py:156-165). Passing ctl = 0 to an update kernel means
- * "clip_scale = 1, never skip". */
+ * "clip_scale = 1, never skip".
+ * `t` counts the steps that passed the guard: anc_gradnorm_finalize with count_step != 0
+ * advances it when the step is not skipped, so a skipped step needs no undo on the host and the
+ * whole guarded step can be issued without a host synchronisation (the reference's resident
+ * step never synchronises, ancora/model/resident_train.py:338-339). The update kernels take the
+ * step's bias corrections and rounding seed from it on request (anc_adamw_hyper_t.step_table,
+ * ANC_SR_STEP_SEED). The caller zeroes the block once (or sets t when resuming). */
 typedef struct {
   double   sumsq;        /* sum of g*g over every gradient element, fp64          */
   float    norm;         /* (float)sqrt(sumsq)                                    */
   float    clip_scale;   /* min(1, max_norm / (norm + eps)); 1 if max_norm <= 0   */
   uint32_t skip;         /* 1 if sumsq is not finite: update kernels write nothing */
-  uint32_t reserved[3];
+  uint32_t t;            /* steps counted so far, this one included if not skipped */
+  uint32_t reserved[2];
 } anc_step_ctl_t;
+/* Stochastic-rounding switch of the update kernels (`sr` arguments and anc_adamw_hyper_t.sr):
+ * 0 = round to nearest even; ANC_SR_ON = stochastic rounding with the seed base given;
+ * ANC_SR_ON | ANC_SR_STEP_SEED = the seed base of the call is seed_base +
+ * ANC_SR_SEED_STRIDE * ctl->t (uint32 wrap-around), i.e. the per-step seed is formed on the device
+ * from the step count of the control block (ctl must not be 0). */
+#define ANC_SR_ON           1
+#define ANC_SR_STEP_SEED    2
+#define ANC_SR_SEED_STRIDE  1000003u
 
 /* ------------------------------------------------------------ grad-norm ----
  * Deterministic global gradient norm, no atomics. Stage 1 writes one fp64
@@ -178,14 +174,16 @@ typedef struct {
 int anc_gradnorm_partials_multi(uint64_t desc_table, int32_t n_tensors,
                                 int64_t total_chunks, uint64_t partials,
                                 uint64_t stream);
+/* count_step != 0: ctl->t is advanced by one unless the step is skipped; 0: ctl->t is left as it is. */
 int anc_gradnorm_finalize(uint64_t partials, int64_t n_partials,
-                          float max_norm, float eps,
+                          float max_norm, float eps, int32_t count_step,
                           uint64_t ctl /* anc_step_ctl_t* */, uint64_t stream);
 
 /* The same norm for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference. One
  * tensor of n elements; result in ctl bit-identical to anc_gradnorm_partials(g, n, g_dtype, buf, 0)
- * followed by anc_gradnorm_finalize(buf, anc_gradnorm_num_partials(n), ...). The stage-1 partial
+ * followed by anc_gradnorm_finalize(buf, anc_gradnorm_num_partials(n), ..., count_step = 0, ...).
+ * The stage-1 partial
  * sums live in a 2 MiB array built into the library (one copy per GPU, held until the process
  * ends), so n is limited to anc_gradnorm_static_max_elements() = 2^31; larger n returns
  * ANC_ERR_ARG. The call allocates nothing (no hipMalloc/hipFree, no events, and it is not seen
@@ -227,10 +225,18 @@ typedef struct {
   float   eps, lr;
   float   bc1, bc2;      /* FORM_DIV: fp32(1-beta^t); FORM_IBC: fp32(1/(1-beta^t)) */
   int32_t form;
-  int32_t sr;            /* 0 = RNE downcast, 1 = stochastic rounding              */
+  int32_t sr;            /* 0 = RNE downcast, ANC_SR_ON (| ANC_SR_STEP_SEED)        */
   uint32_t seed_base;    /* per-step SR seed; a tensor's seed is seed_base + its own */
-  uint32_t reserved;
+  int32_t step_cap;      /* entries 1 .. step_cap of step_table are valid           */
+  uint64_t step_table;   /* 0, or a device array of anc_adamw_step_t: bc1 and bc2 are then taken
+                            from entry min(ctl->t, step_cap) instead of from this block (steps
+                            counted on the device; ctl must not be 0). The host fills the table
+                            ahead with the same fp32 values it would pass per step; once both
+                            corrections have reached 1.0f the last entry serves every later step */
 } anc_adamw_hyper_t;
+/* One entry per counted step (entry 0 unused): the scalars of that step. The dense kernels read
+ * bc1 and bc2; anc_adamw_rows reads all four. */
+typedef struct { float bc1, bc2, lr; uint32_t seed_base; } anc_adamw_step_t;
 
 int anc_adamw(uint64_t g, uint64_t m, uint64_t v, uint64_t p32, uint64_t p16,
               int64_t n /* multiple of 64, as ancora/optim/adamw.py:20,79 */,
@@ -258,7 +264,7 @@ int anc_adamw_multi(uint64_t desc_table, int32_t n_tensors, int64_t total_blocks
  * dense step moves rows with zero gradient too (moment decay, bias-corrected momentum, weight
  * decay), so each row carries the last counted step it is current for (last_step, int32[V], zero
  * at the start) and the steps it missed are replayed on it, with g = 0 and that step's own
- * scalars from step_table (device array of {float bc1, bc2, lr; uint32 seed_base} per counted
+ * scalars from step_table (device array of anc_adamw_step_t {bc1, bc2, lr, seed_base} per counted
  * step, entries 1 .. t_now, bc as in anc_adamw_hyper_t for the chosen form), before anything else
  * is done to it. m, v, p32 and p16 of a current row are bit-identical to anc_adamw's.
  *   grads != 0: rows[i]'s gradient is row i of grads, (n_rows, H) fp32: replay through t_now - 1,
@@ -306,7 +312,7 @@ int anc_muon_momentum(uint64_t buf, uint64_t g, uint64_t u, int64_t K, int64_t N
  * 220-242, 421-427; numpy form ancora/optim/muon.py:308-309):
  *     p32 = p32 - lr_scale*O;   p16 = bf16(p32)   (RNE, or SR keyed as for AdamW)
  * O is (K,N), or (N,K) when transpose_in != 0; o_dtype ANC_BF16 or ANC_F32.
- * p16 = 0 skips the bf16 refresh. */
+ * p16 = 0 skips the bf16 refresh. sr: 0 or ANC_SR_ON. */
 int anc_muon_update(uint64_t p32, uint64_t p16, uint64_t O, int64_t K, int64_t N,
                     float lr_scale, int transpose_in, int o_dtype,
                     int sr, uint32_t seed, uint64_t ctl, uint64_t stream);
@@ -342,7 +348,8 @@ int anc_muon_momentum_multi_pair(uint64_t desc_table, int32_t n_weights, int64_t
                                  uint64_t ctl, uint64_t stream);
 /* lr_scales: host array of ANC_MUON_MAX_SCALES values lr * sqrt(max(1, K/N))
  * (ancora/optim/muon.py:308), one per distinct weight shape class; the table itself
- * holds nothing that changes from step to step. */
+ * holds nothing that changes from step to step. sr: 0, ANC_SR_ON, or
+ * ANC_SR_ON | ANC_SR_STEP_SEED (seed base formed from ctl->t on the device). */
 int anc_muon_update_multi(uint64_t desc_table, int32_t n_weights, int64_t total_tiles,
                           const float *lr_scales, int o_dtype, int sr, uint32_t seed_base,
                           uint64_t ctl, uint64_t stream);
@@ -554,7 +561,8 @@ int anc_ns_batched_pair_multi(const anc_ns_problem_t *probs, int32_t n_probs, in
  * whose orthogonalised update is matrix e of the batch (fields read: p32, p16 (may be 0), K, N,
  * transpose, scale_idx, seed; p16t must be 0). X32_out of the problems is not used. Results in
  * p32 and p16 are bit-identical to the unfused sequence; the fp32 hand-off (8 bytes per parameter
- * of HBM traffic) disappears. ctl: the step's control block or 0 (skip flag honoured). */
+ * of HBM traffic) disappears. ctl: the step's control block or 0 (skip flag honoured). sr as
+ * for anc_muon_update_multi. */
 int anc_muon_ns_update_multi(const anc_ns_problem_t *problems, int32_t n_problems,
                              const uint64_t *desc_tables, int steps, const float *coef, float eps,
                              int mode, const float *lr_scales /* [ANC_MUON_MAX_SCALES] */, int sr,

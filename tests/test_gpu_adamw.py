@@ -172,38 +172,3 @@ def test_special_values(gpu):
     w16 = opt.st["x"]["p16"].to_numpy().ravel()
     assert (w16[3] & 0x7F80) == 0x7F80        # Inf * wd(0) is NaN: still non-finite, not wrapped
     opt.free()
-
-
-def test_copy_shapes_move_what_they_say_and_stay_in_bounds(gpu):
-    """`anc_copy_shape`: the plain-copy shapes reproduce the source, the write-only shape fills,
-    the two optimizer access mixes stay inside their buffers (a canary behind each buffer keeps its
-    bits) and report the bytes of their element counts."""
-    import ctypes
-    from ancora_cutile_amd import DevBuf
-    nb = 8 << 20
-    words = nb // 4
-    rng = np.random.default_rng(3)
-    src_h = rng.integers(0, 2 ** 32, words + 4096, dtype=np.uint32)
-    src, dst = DevBuf(src_h), DevBuf.zeros((words + 4096,), np.uint32)
-    canary = np.full(4096, 0xC0FFEE11, np.uint32)
-    moved = ctypes.c_int64(0)
-    for shape in range(9):
-        dst.fill_zero(0)
-        DevBuf(shape=(4096,), dtype=np.uint32, ptr=dst.ptr + nb).upload(canary)
-        gpu.api.anc_copy_shape(dst.ptr, src.ptr, nb, shape, ctypes.byref(moved), 0)
-        out = dst.to_numpy()
-        assert np.array_equal(out[words:], canary), shape
-        if shape <= 4:
-            assert np.array_equal(out[:words], src_h[:words]) and moved.value == 2 * nb, shape
-        elif shape == 5:
-            assert moved.value == nb and not out[:words].any()          # reads only
-        elif shape == 6:
-            assert moved.value == nb and np.array_equal(out[:8], np.array([1, 2, 3, 4, 1, 2, 3, 4], np.uint32))
-        elif shape == 7:
-            assert moved.value == 28 * (nb // 14 // 4096 * 4096)
-        else:
-            assert moved.value == 14 * (nb // 8 // 4096 * 4096)
-    assert np.array_equal(src.to_numpy(), src_h)
-    with pytest.raises(gpu.AncoraError):
-        gpu.api.anc_copy_shape(dst.ptr, src.ptr, nb, 9, ctypes.byref(moved), 0)
-    src.free(); dst.free()

@@ -79,7 +79,7 @@ def test_config4_moe_family_small(gpu):
             want = muon_update(W[e], ns_any_shape(u, PE_SCHEDULE, 5), 0.02)
             assert rel_fro(W[e] - got[e], W[e] - want) < 2e-3, (n, e)
     for n in r["adamw"]:
-        wd = 0.0 if params[n].ndim == 1 else 0.1
+        wd = 0.0 if params[n].ndim == 1 or "router" in n else 0.1    # the router is not decayed (ancora/kernels/moe.py:603-604)
         want, _, _ = adamw_step_div(params[n], 0 * params[n], 0 * params[n], g[n], 3e-4, 0.9, 0.95, 1e-8,
                                     wd, 1, clip=clip)
         assert max_ulp(am[n], want) == 0, n
@@ -197,7 +197,7 @@ def test_config4_moe_family_real_width(gpu):
             assert err < 2e-3, (n, e, err)
     print(f"\nconfig 4 at width 1024: worst update-direction error {worst:.3e}")
     for n in r["adamw"]:
-        wd = 0.0 if params[n].ndim == 1 else 0.1
+        wd = 0.0 if params[n].ndim == 1 or "router" in n else 0.1    # the router is not decayed (ancora/kernels/moe.py:603-604)
         want, _, _ = adamw_step_div(params[n], 0 * params[n], 0 * params[n], g[n], 3e-4, 0.9, 0.95, 1e-8,
                                     wd, 1, clip=clip)
         assert max_ulp(am[n], want) == 0, n

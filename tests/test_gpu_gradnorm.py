@@ -76,7 +76,7 @@ def test_independent_of_launch_grouping_and_repeatable(gpu):
     for b, k in zip(bufs, nparts):
         api.anc_gradnorm_partials(b.ptr, b.size, _lib.BF16, parts.ptr, off, 0)
         off += k
-    api.anc_gradnorm_finalize(parts.ptr, sum(nparts), 1.0, 1e-6, ctl.ptr, 0)
+    api.anc_gradnorm_finalize(parts.ptr, sum(nparts), 1.0, 1e-6, 0, ctl.ptr, 0)
     raw = ctl.to_numpy()
     assert raw.view(np.float64)[0] == a
     for b in bufs + [parts, ctl]:

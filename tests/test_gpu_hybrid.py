@@ -5,6 +5,7 @@ import pytest
 from oracle.adamw_ref import AdamWRef
 from oracle.muon_ref import MuonRef, PE_SCHEDULE
 from oracle.bf16_ref import bf16_rne_bits, bits_to_f32
+from oracle import gradnorm_ref as gn
 from util import max_ulp, rel_fro, bits_equal, bf16_grad
 
 pytestmark = pytest.mark.gpu
@@ -218,7 +219,10 @@ def test_checkpoint_resume_is_bitwise(gpu, tmp_path):
 def test_default_predicate_with_a_misaligned_router(gpu):
     """`HybridOptimizer(model.params())` on a MoE parameter set with the default predicate
     (tests/training/test_moe_pipeline.py:36): the (H, E) router is 2-D, so the predicate names it
-    for Muon, but it is not 128-aligned; it goes to AdamW instead of raising, and the step runs."""
+    for Muon, but it is not 128-aligned. The reference keeps it on Muon with Newton-Schulz on the
+    host (ancora/optim/muon.py:37-41, 307); here it stays on Muon too, zero-padded through the
+    device chain: its master weights follow the numpy Muon (Keller, the default) over three steps,
+    the padding never leaks into what the accessors return, and it saves and reloads."""
     from ancora_cutile_amd import HybridOptimizer
     rng = np.random.default_rng(8)
     params = {"embed": (0.02 * rng.standard_normal((256, 128))).astype(np.float32),
@@ -226,15 +230,129 @@ def test_default_predicate_with_a_misaligned_router(gpu):
               "layer1.ffn.gate_proj": (0.02 * rng.standard_normal((4, 128, 128))).astype(np.float32),
               "layer1.q_proj": (0.02 * rng.standard_normal((128, 256))).astype(np.float32)}
     opt = HybridOptimizer(params)
-    assert opt.routing() == {"muon": ["layer1.q_proj"],
-                             "adamw": ["embed", "layer1.ffn.router", "layer1.ffn.gate_proj"]}
-    assert opt.misaligned_to_adamw == ["layer1.ffn.router"]
+    assert opt.routing() == {"muon": ["layer1.ffn.router", "layer1.q_proj"],
+                             "adamw": ["embed", "layer1.ffn.gate_proj"]}
+    assert opt.muon_padded == ["layer1.ffn.router"]
+    mr = MuonRef({n: params[n] for n in opt.muon_names})
+    for step in range(3):
+        grads = {n: (1e-2 * rng.standard_normal(p.shape)).astype(np.float32) for n, p in params.items()}
+        opt.step(grads, 0)
+        mr.step(grads)
+    got = opt.muon.master()
+    for n in opt.muon_names:
+        assert got[n].shape == params[n].shape
+        d = np.linalg.norm(got[n].astype(np.float64) - mr.w[n]) / np.linalg.norm(params[n] - mr.w[n])
+        assert d < 2e-3, (n, d)
+    # the shape factor is that of the router's own dims: sqrt(128 / 16), not of the padded ones
+    upd = np.linalg.norm(params["layer1.ffn.router"] - got["layer1.ffn.router"])
+    assert upd > 0.02 * (128 / 16) ** 0.5 * 3 * 0.5
+    # padding rows and columns of the stored state stay exactly zero
+    full = opt.muon.st["layer1.ffn.router"]["p32"].to_numpy().reshape(128, 128)
+    assert not full[:, 16:].any()
+    assert opt.muon.weights()["layer1.ffn.router"].shape == (128, 16)
+    assert opt.muon.momentum_buffers()["layer1.ffn.router"].shape == (128, 16)
+    opt.free()
+
+
+def test_router_left_to_adamw_is_not_decayed(gpu):
+    """Under the resident routing the router is an AdamW tensor, and the resident models run it
+    with wd = 0 (ancora/kernels/moe.py:603-604): the default `no_decay` exempts it like the gains."""
+    from ancora_cutile_amd import HybridOptimizer, resident_is_muon
+    rng = np.random.default_rng(9)
+    params = {"layer1.ffn.router": (0.02 * rng.standard_normal((128, 16))).astype(np.float32),
+              "layer1.post_ln": (1 + 0.05 * rng.standard_normal(128)).astype(np.float32),
+              "layer1.q_proj": (0.02 * rng.standard_normal((128, 256))).astype(np.float32)}
+    opt = HybridOptimizer(params, is_muon=resident_is_muon)
+    assert opt.routing() == {"muon": ["layer1.q_proj"], "adamw": ["layer1.ffn.router", "layer1.post_ln"]}
+    assert opt.adamw.st["layer1.ffn.router"]["wd"] == 0.0 and opt.adamw.st["layer1.post_ln"]["wd"] == 0.0
     grads = {n: (1e-2 * rng.standard_normal(p.shape)).astype(np.float32) for n, p in params.items()}
     opt.step(grads, 0)
-    ar = AdamWRef({n: params[n] for n in opt.adamw_names}, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.01)
+    ar = AdamWRef({n: params[n] for n in opt.adamw_names}, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, wd=0.01,
+                  no_decay=tuple(opt.adamw_names))
     ar.step(grads)
     assert max_ulp(opt.adamw.master()["layer1.ffn.router"], ar.st["layer1.ffn.router"]["p"]) == 0
     opt.free()
+
+
+def test_unsynchronised_guarded_steps_equal_the_synchronous_ones(gpu, monkeypatch):
+    """`step(..., sync=False)`: six guarded steps with resident bf16 gradients, the second and the
+    fifth with a non-finite gradient, issued without a single host synchronisation (every
+    synchronising library call is counted), as the reference's resident step is
+    (ancora/model/resident_train.py:338-339). The steps are counted on the device, so a skipped
+    step needs no undo: every state tensor equals, bit for bit, the state after the same six
+    synchronous steps, the step count is 4, and the AdamW master weights equal the numpy oracle's
+    after its four steps (bias corrections of steps 1..4, rounding seeds of steps 1..4)."""
+    from ancora_cutile_amd import HybridOptimizer, DevBuf, PE_SCHEDULE, resident_is_muon, _lib
+    rng = np.random.default_rng(21)
+    params = {"embed": (0.02 * rng.standard_normal((512, 256))).astype(np.float32),
+              "final_norm": (1 + 0.05 * rng.standard_normal(256)).astype(np.float32),
+              "layer0.q_proj": (0.02 * rng.standard_normal((256, 512))).astype(np.float32),
+              "layer0.o_proj": (0.02 * rng.standard_normal((512, 256))).astype(np.float32)}
+    steps = []
+    for t in range(6):
+        g = {n: bf16_rne_bits((1e-2 * rng.standard_normal(p.shape)).astype(np.float32)).reshape(p.shape)
+             for n, p in params.items()}
+        if t in (1, 4):
+            g["embed"] = g["embed"].copy()
+            g["embed"][3, 5] = 0x7FC0 if t == 1 else 0x7F80          # NaN, +Inf
+        steps.append(g)
+    kw = dict(is_muon=resident_is_muon, muon_kw=dict(schedule=PE_SCHEDULE, sr=True, seed=5),
+              adamw_kw=dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, wd=0.1, sr=True, seed=7),
+              max_grad_norm=1.0, grad_dtype=np.uint16)
+
+    def run(sync):
+        opt = HybridOptimizer(params, **kw)
+        bufs = [{n: DevBuf(g[n]) for n in params} for g in steps]       # resident before the steps
+        _lib.stream_sync(0)
+        calls = {"n": 0}
+        names = ("anc_stream_sync", "anc_device_sync", "anc_memcpy_d2h", "anc_memcpy_h2d", "anc_event_sync")
+        if not sync:
+            for name in names:
+                real = getattr(_lib.api, name)
+                monkeypatch.setattr(_lib.api, name, (lambda real: lambda *a: (calls.__setitem__("n", calls["n"] + 1), real(*a))[1])(real))
+        # one set of gradient buffers for every step, as in a training loop (the descriptor tables
+        # are built for them once, at the first step); each step's gradient arrives by an
+        # asynchronous device copy on the step's stream
+        cur = {n: DevBuf(steps[0][n]) for n in params}
+        opt.step(cur, 0)                   # first step: descriptor and step tables are uploaded here
+        calls["n"] = 0
+        skipped = []
+        for b in bufs[1:]:
+            for n in params:
+                _lib.api.anc_memcpy_d2d(cur[n].ptr, b[n].ptr, cur[n].nbytes, 0)
+            opt.step(cur, 0, sync=sync)
+            if sync:
+                skipped.append(opt.last_skipped)
+        n_sync = calls["n"]
+        monkeypatch.undo()
+        state = opt.state_dict()
+        out = dict(state=state, t=opt.step_count(), skipped=skipped, n_sync=n_sync, last=dict(opt.last_ctl),
+                   adamw=opt.adamw.master(), at=opt.adamw.t, mt=opt.muon.engine.t)
+        opt.free()
+        for b in bufs + [cur]:
+            for d in b.values():
+                d.free()
+        return out
+
+    a, b = run(True), run(False)
+    assert a["skipped"] == [True, False, False, True, False]
+    assert b["n_sync"] == 0, "an unsynchronised step called a synchronising entry point"
+    assert a["t"] == b["t"] == 4 and a["at"] == b["at"] == 4 and a["mt"] == b["mt"] == 4
+    assert a["state"].keys() == b["state"].keys()
+    for k in a["state"]:
+        assert np.atleast_1d(a["state"][k]).tobytes() == np.atleast_1d(b["state"][k]).tobytes(), k
+    assert a["last"] == b["last"] and not b["last"]["skip"]
+    # the oracle takes the four finite steps
+    ar = AdamWRef({n: params[n] for n in ("embed", "final_norm")}, lr=3e-3, betas=(0.9, 0.95), eps=1e-8,
+                  wd=0.1, no_decay=("final_norm",))
+    order = ["layer0.q_proj", "layer0.o_proj", "embed", "final_norm"]
+    for t, g in enumerate(steps):
+        if t in (1, 4):
+            continue
+        gf = {n: bits_to_f32(g[n]).reshape(g[n].shape) for n in g}
+        ar.step(gf, clip=gn.control(gn.gradnorm_fixed([g[n] for n in order]), 1.0, 1e-6)["clip_scale"])
+    for n in ("embed", "final_norm"):
+        assert max_ulp(b["adamw"][n], ar.st[n]["p"]) == 0, n
 
 
 @pytest.mark.parametrize("sr", [False, True])

@@ -26,13 +26,13 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} declared in include/anc_optim.h but not exported"
     assert sorted(_lib.EXPORTS) == names, "ctypes prototypes and header disagree"
     _lib.load()
-    assert _lib.api.anc_abi_version() == 2
+    assert _lib.api.anc_abi_version() == _lib.ABI_VERSION == 3
 
 
 def test_struct_sizes_match_header():
     from ancora_cutile_amd import _lib
     assert ctypes.sizeof(_lib.StepCtl) == 32
-    assert ctypes.sizeof(_lib.AdamWHyper) == 48
+    assert ctypes.sizeof(_lib.AdamWHyper) == 56
     assert ctypes.sizeof(_lib.AdamWDesc) == 72
     assert ctypes.sizeof(_lib.GnDesc) == 40
     assert ctypes.sizeof(_lib.MuonDesc) == 80
@@ -49,6 +49,7 @@ def test_header_is_plain_c_and_layouts_match_ctypes(tmp_path):
     if gcc is None:
         pytest.skip("no gcc")
     pairs = [("anc_step_ctl_t", _lib.StepCtl), ("anc_adamw_hyper_t", _lib.AdamWHyper),
+             ("anc_adamw_step_t", _lib.AdamWStepEntry),
              ("anc_adamw_desc_t", _lib.AdamWDesc), ("anc_gn_desc_t", _lib.GnDesc),
              ("anc_muon_desc_t", _lib.MuonDesc), ("anc_ns_problem_t", _lib.NsProblem),
              ("anc_dw_problem_t", _lib.DwProblem),

@@ -13,7 +13,7 @@ def _reference_ctl(api, DevBuf, g, n, code, max_norm, eps):
     parts = DevBuf.empty((api.anc_gradnorm_num_partials(n),), np.float64)
     ctl = DevBuf.zeros((8,), np.uint32)
     api.anc_gradnorm_partials(g.ptr, n, code, parts.ptr, 0, 0)
-    api.anc_gradnorm_finalize(parts.ptr, parts.size, max_norm, eps, ctl.ptr, 0)
+    api.anc_gradnorm_finalize(parts.ptr, parts.size, max_norm, eps, 0, ctl.ptr, 0)
     out = _ctl_bytes(ctl)
     parts.free(); ctl.free()
     return out
