@@ -28,13 +28,14 @@ k_embed_dw_scatter(const int32_t *__restrict__ cnt, const int32_t *__restrict__ 
   const int c0 = (int)blockIdx.y * kChunk + (int)threadIdx.x * 4;
   if (c0 >= H) return;
   float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  bool bad = false;                                     // an index outside dy: the group writes nothing
   for (int r0 = 0; r0 < n; r0 += 8) {
     anc_u32x2 v[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if (r0 + j < n) {
         int64_t sr = srt[st + r0 + j];
-        if (sr < 0 || sr >= M) sr = 0;                 // malformed index: stay inside dy
+        if (sr < 0 || sr >= M) { sr = 0; bad = true; }  // malformed index: stay inside dy
         v[j] = *(const anc_u32x2 *)(dy + sr * H + c0);
       }
     }
@@ -48,6 +49,7 @@ k_embed_dw_scatter(const int32_t *__restrict__ cnt, const int32_t *__restrict__ 
       }
     }
   }
+  if (bad) return;
   if (compact != nullptr) {
     const anc_f32x4 o = {acc[0], acc[1], acc[2], acc[3]};
     *(anc_f32x4 *)(compact + (int64_t)g * H + c0) = o;

@@ -701,11 +701,10 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
         sp.gate_bx = (1u << 2) | (1u << 3);
         sp.x_from = 4;
       }
-    } else if (N > 2 * M || M > 1024) {
-      // iteration 2 alone. Not at 1024x2048 itself: there the outlier-column case meets the bar
-      // without (1.57e-3 .. 1.61e-3 over seeds) and the term would cost its matrices 6 %; the rest
-      // of 2M <= N < 3M does not (1024x2560 1.8e-3, 1536x3072 2.1e-3, 2048x4096 2.2e-3, 4096x8192
-      // 2.3e-3 without).
+    } else {
+      // N >= 2M: iteration 2 alone (1 % of the columns x100 without it: 1024x2048 1.6e-3 .. 1.7e-3,
+      // 1024x2560 1.8e-3, 1536x3072 2.1e-3, 1024x3072 2.2e-3, 2048x4096 2.2e-3, 4096x8192 2.3e-3;
+      // with it 1.0e-3 .. 1.2e-3). One rule for every such shape.
       sp.gate_tau[2] = kTauHard;
       // a chain shorter than the 5 steps this was measured on ends before iteration 2's term has
       // paid off (3 steps at 1024x3072: 2.3e-3, 2 steps 2.7e-3): iteration 1 as well

@@ -90,23 +90,36 @@ class RowSparseAdamW:
         self.table = DevBuf.zeros((self._cap + 1, 4), np.uint32)
         self._rows_buf = None
         self.last_skipped = False
+        self._filled_to = 0          # table entries 1 .. _filled_to hold the scalars of their steps
+        self._filled_lr = None       # ... computed with this learning rate
 
     def _hyper(self):
         return AdamWHyper(beta1=self.b1, beta2=self.b2, omb1=1 - self.b1, omb2=1 - self.b2, eps=self.eps,
                           lr=0.0, bc1=1.0, bc2=1.0, form=FORM_DIV if self.form == "div" else FORM_IBC,
                           sr=int(self.sr), seed_base=0)
 
-    def _append_step(self, si):
-        t = self.t
-        if t > self._cap:
-            raise RuntimeError(f"RowSparseAdamW: step table holds {self._cap} steps; raise max_steps")
+    FILL_AHEAD = 256
+
+    def _step_record(self, t, lr):
         bc1, bc2 = 1 - self.b1 ** t, 1 - self.b2 ** t
         if self.form != "div":
             bc1, bc2 = 1.0 / bc1, 1.0 / bc2
         rec = np.zeros(4, np.uint32)
-        rec[:3] = np.array([bc1, bc2, self.lr], np.float32).view(np.uint32)
+        rec[:3] = np.array([bc1, bc2, lr], np.float32).view(np.uint32)
         rec[3] = sr_seed_base(self.seed, t) if self.sr else 0
-        DevBuf(shape=(4,), dtype=np.uint32, ptr=self.table.ptr + 16 * t).upload(rec, si)
+        return rec
+
+    def _ensure_step(self, t, si):
+        """Table entry t holds step t's scalars at the current learning rate. Entries are written
+        FILL_AHEAD steps at a time, so a run at a constant learning rate uploads (and synchronises)
+        once per FILL_AHEAD steps instead of at every step; a changed learning rate rewrites from t
+        on (earlier entries keep the rate their steps ran with: the replay needs it)."""
+        if t <= self._filled_to and self._filled_lr == self.lr:
+            return
+        hi = min(self._cap, t + self.FILL_AHEAD - 1)
+        block = np.stack([self._step_record(s, self.lr) for s in range(t, hi + 1)])
+        DevBuf(shape=block.shape, dtype=np.uint32, ptr=self.table.ptr + 16 * t).upload(block, si)
+        self._filled_to, self._filled_lr = hi, self.lr
 
     def _rows(self, rows, si):
         rows = np.ascontiguousarray(rows, dtype=np.int32).reshape(-1)
@@ -134,8 +147,10 @@ class RowSparseAdamW:
     def step(self, gid, n_groups, grads, si, guard=None):
         """gid: device int32 array of distinct row ids (e.g. `IdGroups.gid`), the first n_groups
         valid; grads: (>= n_groups, H) fp32 DevBuf, row i the gradient of gid[i]."""
+        if self.t + 1 > self._cap:             # before the counter moves: t always matches the table
+            raise RuntimeError(f"RowSparseAdamW: step table holds {self._cap} steps; raise max_steps")
+        self._ensure_step(self.t + 1, si)
         self.t += 1
-        self._append_step(si)
         if n_groups > 0:
             self._launch(gid.ptr, int(n_groups), grads.ptr, self.t, 0 if guard is None else guard.ptr, si)
         self.last_skipped = False

@@ -41,11 +41,14 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def synth(shapes, seed=0):
-    """Synthetic weights (fp32) and gradients (bf16 bits) of the workload."""
+def synth(shapes, seed=0, idle_experts=4):
+    """Synthetic weights (fp32) and gradients (bf16 bits) of the workload: weights 0.02 N(0,1), gains
+    1 + 0.05 N(0,1), gradients N(0, 1e-3) with 1 % of the rows of every matrix x100. A stacked
+    [E, K, N] expert tensor is E matrices; per MoE layer `idle_experts` of its experts (the same ones
+    in the layer's three tensors, drawn from the seeded generator) have an all-zero gradient."""
     from ancora_cutile_amd.bf16 import bf16_bits
     rng = np.random.default_rng(seed)
-    params, grads = {}, {}
+    params, grads, idle = {}, {}, {}
     for name, shape in shapes.items():
         n = int(np.prod(shape))
         if len(shape) == 1:
@@ -54,9 +57,15 @@ def synth(shapes, seed=0):
             p = (0.02 * rng.standard_normal(n, dtype=np.float32)).reshape(shape)
         g = (1e-3 * rng.standard_normal(n, dtype=np.float32)).reshape(shape)
         if len(shape) >= 2:                      # 1% of rows carry a x100 outlier scale
-            rows = shape[0]
+            g2 = g.reshape(-1, shape[-1])
+            rows = g2.shape[0]
             k = max(1, rows // 100)
-            g[rng.choice(rows, k, replace=False)] *= 100.0
+            g2[rng.choice(rows, k, replace=False)] *= 100.0
+        if len(shape) == 3 and idle_experts:
+            layer = name.split(".")[0]
+            if layer not in idle:
+                idle[layer] = np.sort(rng.choice(shape[0], min(idle_experts, shape[0]), replace=False))
+            g[idle[layer]] = 0.0
         params[name] = p
         grads[name] = bf16_bits(g).reshape(shape)
     return params, grads

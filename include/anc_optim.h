@@ -188,7 +188,9 @@ int anc_gradnorm_finalize(uint64_t partials, int64_t n_partials,
  * ends), so n is limited to anc_gradnorm_static_max_elements() = 2^31; larger n returns
  * ANC_ERR_ARG. The call allocates nothing (no hipMalloc/hipFree, no events, and it is not seen
  * by anc_profile_*). All calls on one GPU share that array: calls that overlap in time on one
- * GPU (different streams without ordering) race and must be serialised by the caller. */
+ * GPU (different streams without ordering) race and must be serialised by the caller. A call on
+ * another stream than the previous call's while that stream still has work queued is refused
+ * (ANC_ERR_UNSUPPORTED): the one overlap the library can see without allocating anything. */
 int64_t anc_gradnorm_static_max_elements(void);
 int anc_gradnorm_static(uint64_t g, int64_t n, int g_dtype, float max_norm, float eps,
                         uint64_t ctl /* anc_step_ctl_t* */, uint64_t stream);
@@ -285,7 +287,8 @@ int anc_adamw_rows(uint64_t rows, int64_t n_rows, uint64_t grads, uint64_t m, ui
  *   out != 0:     out[gid[g]] += sum_r f32(dy[srt[start[g] + r]]), out (V, H) fp32 (the reference)
  *   compact != 0: compact[g]   = that sum, (M, H) fp32: the gradient rows anc_adamw_rows takes
  * Rows of a group are added in sorted order starting from zero, one writer per element, no
- * atomics: bit-identical to the sequential fp32 sum, and from run to run. H % 64 == 0. */
+ * atomics: bit-identical to the sequential fp32 sum, and from run to run. H % 64 == 0. A group
+ * whose start / count / id / sorted indices point outside the arrays writes nothing. */
 int anc_embed_dw_scatter(uint64_t cnt, uint64_t start, uint64_t gid, uint64_t srt, uint64_t dy,
                          uint64_t out, uint64_t compact, int64_t M, int64_t V, int64_t H,
                          uint64_t stream);
@@ -453,15 +456,14 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  * r directions spread over all rows (about 100 with 1 % of the columns x100). Later products of a
  * matrix add the residual of X (three accumulation terms in A = X X^T, two in X = a X + B X)
  * according to it:
- *   N >= 3M:  above 2.5, A = X X^T of iteration 2 (1 % of the columns x100 at 1024x3072: 1.15e-3
+ *   N >= 2M:  above 2.5, A = X X^T of iteration 2 (1 % of the columns x100 at 1024x3072: 1.15e-3
  *             instead of 2.2e-3), and of iteration 1 in chains shorter than 5 steps;
  *   N < 2M:   above 2.5, A = X X^T of iterations 1 and 2 (1024x1024: 8e-4 instead of 3.8e-3); above
  *             1.3, both X-products of iterations 2 and 3 (5-step chains; every matrix has them in
  *             iteration 4): a matrix with independent entries or outlier rows does without
  *             (1.67e-3 / 5e-4 at 1024x1024), column-scaled ones need them (columns scaled over
  *             0.1..3: 1.45e-3; 2.1e-3 with iteration 4 alone, 1.9e-3 with iterations 3 and 4);
- *   2M <= N < 3M: as N >= 3M (1536x3072, 2048x4096: 1.0e-3 instead of 2.1e-3 .. 2.3e-3), except
- *             1024x2048 itself: none (1.6e-3 on the outlier-column case as it is);
+ *   2M <= N < 3M: as N >= 3M (1536x3072, 2048x4096: 1.0e-3 instead of 2.1e-3 .. 2.3e-3);
  *   M < 1024: no gates. Small matrices average fewer rounding errors per element and cost next to
  *             nothing: every product carries the residuals of X, F and Boff from iteration 1 on
  *             (from iteration 0 below M = 256), for every matrix, in ANC_NS_BF16 and

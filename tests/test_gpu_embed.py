@@ -132,3 +132,65 @@ def test_row_sparse_adamw_skip_and_clip(gpu):
     for b in (gid, grads):
         b.free()
     guard.free(); opt.free()
+
+
+def test_row_sparse_adamw_step_table_capacity_and_constant_rate_uploads(gpu, monkeypatch):
+    """The step table is written ahead in blocks (one upload per block of steps at a constant
+    learning rate, a rewrite when the rate changes), and a step beyond its capacity raises before
+    the counter moves, so `t` never runs ahead of the table."""
+    from ancora_cutile_amd import DevBuf, _lib
+    from ancora_cutile_amd.embed import RowSparseAdamW
+    V, H = 256, 64
+    rng = np.random.default_rng(1)
+    opt = RowSparseAdamW((0.02 * rng.standard_normal((V, H))).astype(np.float32), max_steps=3)
+    gid = DevBuf(np.arange(4, dtype=np.int32))
+    g = DevBuf((1e-2 * rng.standard_normal((4, H))).astype(np.float32))
+    uploads = {"n": 0}
+    real = _lib.api.anc_memcpy_h2d
+    monkeypatch.setattr(_lib.api, "anc_memcpy_h2d", lambda *a: (uploads.__setitem__("n", uploads["n"] + 1), real(*a))[1])
+    opt.step(gid, 4, g, 0)
+    opt.step(gid, 4, g, 0)
+    assert uploads["n"] == 1                     # both steps' scalars went up with the first
+    opt.lr = 1e-4
+    opt.step(gid, 4, g, 0)
+    assert uploads["n"] == 2 and opt.t == 3
+    with pytest.raises(RuntimeError):
+        opt.step(gid, 4, g, 0)
+    assert opt.t == 3
+    monkeypatch.undo()
+    tab = opt.table.to_numpy().reshape(-1, 4)
+    lrs = tab[1:4, 2].copy().view(np.float32)
+    assert lrs[0] == lrs[1] == np.float32(3e-4) and lrs[2] == np.float32(1e-4)
+    for b in (gid, g):
+        b.free()
+    opt.free()
+
+
+def test_embed_dw_scatter_leaves_out_a_group_with_an_index_outside_the_batch(gpu):
+    """A sorted index outside [0, M) cannot name a row of dy: its group writes nothing (it used to
+    be served row 0), every other group is the sequential sum as before."""
+    from ancora_cutile_amd import DevBuf
+    from ancora_cutile_amd.embed import IdGroups, embed_dw_scatter
+    M, V, H = 64, 32, 64
+    rng = np.random.default_rng(2)
+    ids = rng.integers(0, V, M).astype(np.int32)
+    dyb = bf16_rne_bits(rng.standard_normal((M, H)).astype(np.float32)).reshape(M, H)
+    base = (0.1 * rng.standard_normal((V, H))).astype(np.float32)
+    grp = IdGroups(ids)
+    want = scatter_ref(ids, dyb, base)
+    srt = grp.srt.to_numpy().copy()
+    start, gids = grp.host[1].reshape(-1), grp.host[3].reshape(-1)
+    victim = 1                                       # break the first sorted index of group 1
+    srt[start[victim]] = M + 7
+    grp.srt.upload(srt)
+    gdy, out = DevBuf(dyb), DevBuf(base)
+    embed_dw_scatter(grp, gdy, 0, out=out)
+    got = out.to_numpy()
+    row = int(gids[victim])
+    assert bits_equal(got[row], base[row])
+    keep = np.ones(V, bool)
+    keep[row] = False
+    assert bits_equal(got[keep], want[keep])
+    for b in (gdy, out):
+        b.free()
+    grp.free()

@@ -6,7 +6,7 @@ from oracle.adamw_ref import AdamWRef
 from oracle.muon_ref import MuonRef, PE_SCHEDULE
 from oracle.bf16_ref import bf16_rne_bits, bits_to_f32
 from oracle import gradnorm_ref as gn
-from util import max_ulp, rel_fro, bits_equal, bf16_grad
+from util import max_ulp, rel_fro, bits_equal, bf16_grad, StubMoELayer as _StubMoELayer
 
 pytestmark = pytest.mark.gpu
 
@@ -416,28 +416,6 @@ def test_fused_update_equals_separate_update_kernel(gpu, sr):
         for k in ("buf", "p32", "p16", "G"):
             if w[k] is not None:
                 w[k].free()
-
-
-class _StubMoELayer:
-    """What `GroupedMoEFFN` carries when its optimizer methods run: masters in `w`, packed bf16
-    forward weights and their transposes, fp32 gradient buffers, router buffers."""
-
-    def __init__(self, E, H, rng, optimizer, device_route):
-        from ancora_cutile_amd import DevBuf
-        from ancora_cutile_amd.bf16 import bf16_bits
-        self.E, self.H, self.Ie, self.optimizer, self.device_route = E, H, H, optimizer, device_route
-        self.w = {k: (0.02 * rng.standard_normal((E, H, H))).astype(np.float32)
-                  for k in ("gate_proj", "up_proj", "down_proj")}
-        self.w["router"] = (0.02 * rng.standard_normal((H, E))).astype(np.float32)
-        for attr, key in (("Wg", "gate_proj"), ("Wu", "up_proj"), ("Wd", "down_proj")):
-            setattr(self, attr, DevBuf(bf16_bits(self.w[key]).reshape(E * H, H)))
-            setattr(self, attr + "T", DevBuf.zeros((E * H, H), np.uint16))
-            setattr(self, "d" + attr, DevBuf.zeros((E * H, H), np.float32))
-        self.Wr_dev = DevBuf(self.w["router"].reshape(-1))
-        self.G_router_dev = DevBuf.zeros((H * E,), np.float32)
-        self.Gr_acc = DevBuf.zeros((H * E,), np.float32)
-        self.G_router = np.zeros((H, E), np.float32)
-        self._muon_lr = 0.02
 
 
 @pytest.mark.parametrize("optimizer", ["muon", "adamw"])

@@ -354,8 +354,8 @@ def test_outlier_columns_take_the_gate_and_meet_the_bar(gpu, M, N):
     X = np.stack([gauss, cols, rows])
     got = run_ns(X)
     n_hard, extra = _hard_count(3, M, N)
-    # 1024x2048 meets the bar without the extra terms; M < 1024 has them for every matrix
-    gated = M >= 1024 and (M, N) != (1024, 2048)
+    # M < 1024 has the extra terms for every matrix
+    gated = M >= 1024
     assert (n_hard == 1 and extra > 0) if gated else (n_hard == 0 and extra == 0)
     errs = [rel_fro(got[e], host_ns(X[e], PE_SCHEDULE, 5)) for e in range(3)]
     print(f"({M},{N}) gaussian {errs[0]:.3e}  outlier columns {errs[1]:.3e}  outlier rows {errs[2]:.3e}")
@@ -452,7 +452,7 @@ def test_low_rank_signal_over_weak_noise_is_told_from_outlier_columns(gpu, M, N)
     print(f"({M},{N}) rank 32 + 10 % noise {errs[0]:.3e}  outlier columns {errs[1]:.3e}  "
           f"rank 32 + 1 % noise {errs[2]:.3e}  gaussian {errs[3]:.3e}")
     assert errs[0] < 4e-4 and errs[2] < 6e-4 and errs[1] < TOL_BF16 and errs[3] < TOL_BF16
-    assert n_gated == (2 if (M, N) == (1024, 2048) else 3)      # 1024x2048 has no outlier-column gate
+    assert n_gated == 3
     per = []
     for e in range(4):
         alone = run_ns(X[e:e + 1])

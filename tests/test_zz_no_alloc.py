@@ -53,3 +53,63 @@ def test_static_gradnorm_nonfinite_and_limits(gpu):
     with pytest.raises(_lib.AncoraError):
         api.anc_gradnorm_static(g.ptr, 2 ** 31 + 1, _lib.F32, 1.0, 1e-6, ctl.ptr, 0)
     g.free(); ctl.free()
+
+
+def test_static_gradnorm_allocates_nothing_and_refuses_a_visible_overlap(gpu):
+    """Free device memory is the same before and after a call; a call on a second stream while the
+    first call's stream is still busy is refused, and accepted once that stream has drained."""
+    from ancora_cutile_amd import DevBuf, _lib
+    api = _lib.api
+    n = 1 << 28
+    g = DevBuf.zeros((n,), np.uint16)
+    ctl, ctl2 = DevBuf.zeros((8,), np.uint32), DevBuf.zeros((8,), np.uint32)
+    api.anc_gradnorm_static(g.ptr, n, _lib.BF16, 1.0, 1e-6, ctl.ptr, 0)        # symbol looked up by now
+    _lib.stream_sync(0)
+    import ctypes
+    free0, free1, total = ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int64(0)
+    api.anc_mem_info(ctypes.byref(free0), ctypes.byref(total))
+    for _ in range(3):
+        api.anc_gradnorm_static(g.ptr, n, _lib.BF16, 1.0, 1e-6, ctl.ptr, 0)
+    _lib.stream_sync(0)
+    api.anc_mem_info(ctypes.byref(free1), ctypes.byref(total))
+    assert free1.value == free0.value
+    s1, s2 = _lib.stream_create(), _lib.stream_create()
+    for _ in range(8):                                  # about half a millisecond of queued work each
+        api.anc_gradnorm_static(g.ptr, n, _lib.BF16, 1.0, 1e-6, ctl.ptr, s1)
+    with pytest.raises(_lib.AncoraError):
+        api.anc_gradnorm_static(g.ptr, n, _lib.BF16, 1.0, 1e-6, ctl2.ptr, s2)
+    _lib.stream_sync(s1)
+    api.anc_gradnorm_static(g.ptr, n, _lib.BF16, 1.0, 1e-6, ctl2.ptr, s2)
+    _lib.stream_sync(s2)
+    assert _ctl_bytes(ctl) == _ctl_bytes(ctl2)
+    api.anc_stream_destroy(s1); api.anc_stream_destroy(s2)
+    api.anc_gradnorm_static(g.ptr, n, _lib.BF16, 1.0, 1e-6, ctl.ptr, 0)        # the remembered stream is gone: still fine
+    _lib.stream_sync(0)
+    g.free(); ctl.free(); ctl2.free()
+
+
+def test_static_gradnorm_first_call_without_init(gpu, tmp_path):
+    """A process that never calls anc_init: the first anc_gradnorm_static looks the scratch array's
+    address up itself and gives the sum of squares of the fixed-order oracle."""
+    import subprocess
+    import sys
+    from ancora_cutile_amd import _lib
+    from oracle import gradnorm_ref as gn
+    x = (1e-3 * np.random.default_rng(3).standard_normal(8192 * 5 + 24)).astype(np.float32)
+    np.save(tmp_path / "x.npy", x)
+    code = f"""
+import ctypes as C, numpy as np
+lib = C.CDLL({_lib.LIB_PATH!r})
+x = np.load({str(tmp_path / 'x.npy')!r})
+u64 = C.c_uint64
+g, ctl = u64(0), u64(0)
+assert lib.anc_malloc(C.byref(g), C.c_int64(x.nbytes)) == 0 and lib.anc_malloc(C.byref(ctl), C.c_int64(32)) == 0
+assert lib.anc_memcpy_h2d(g, x.ctypes.data_as(C.c_void_p), C.c_int64(x.nbytes), u64(0)) == 0
+assert lib.anc_gradnorm_static(g, C.c_int64(x.size), C.c_int(0), C.c_float(1.0), C.c_float(1e-6), ctl, u64(0)) == 0
+out = np.zeros(4, np.float64)
+assert lib.anc_memcpy_d2h(out.ctypes.data_as(C.c_void_p), ctl, C.c_int64(32), u64(0)) == 0
+print(repr(float(out[0])))
+"""
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr
+    assert float(r.stdout.strip().splitlines()[-1]) == gn.gradnorm_fixed([x])

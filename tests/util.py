@@ -34,3 +34,25 @@ def bf16_grad(rng, shape, std=1e-3):
     g = (rng.standard_normal(shape) * std).astype(np.float32)
     bits = bf16_rne_bits(g)
     return bits, bits_to_f32(bits).reshape(shape)
+
+
+class StubMoELayer:
+    """What `GroupedMoEFFN` carries when its optimizer methods run: masters in `w`, packed bf16
+    forward weights and their transposes, fp32 gradient buffers, router buffers."""
+
+    def __init__(self, E, H, rng, optimizer, device_route):
+        from ancora_cutile_amd import DevBuf
+        from ancora_cutile_amd.bf16 import bf16_bits
+        self.E, self.H, self.Ie, self.optimizer, self.device_route = E, H, H, optimizer, device_route
+        self.w = {k: (0.02 * rng.standard_normal((E, H, H))).astype(np.float32)
+                  for k in ("gate_proj", "up_proj", "down_proj")}
+        self.w["router"] = (0.02 * rng.standard_normal((H, E))).astype(np.float32)
+        for attr, key in (("Wg", "gate_proj"), ("Wu", "up_proj"), ("Wd", "down_proj")):
+            setattr(self, attr, DevBuf(bf16_bits(self.w[key]).reshape(E * H, H)))
+            setattr(self, attr + "T", DevBuf.zeros((E * H, H), np.uint16))
+            setattr(self, "d" + attr, DevBuf.zeros((E * H, H), np.float32))
+        self.Wr_dev = DevBuf(self.w["router"].reshape(-1))
+        self.G_router_dev = DevBuf.zeros((H * E,), np.float32)
+        self.Gr_acc = DevBuf.zeros((H * E,), np.float32)
+        self.G_router = np.zeros((H, E), np.float32)
+        self._muon_lr = 0.02
