@@ -143,9 +143,6 @@ static __device__ __align__(256) double scratch[ANC_GN_STATIC_MAX_PARTIALS];
 namespace {
 constexpr int kMaxDevices = 64;
 std::atomic<double *> g_scratch_ptr[kMaxDevices];
-// the stream of the last call per device (plus one, so that 0 means "none yet"): a call that
-// arrives on another stream while that one still has work queued would share the array with it
-std::atomic<uint64_t> g_last_stream[kMaxDevices];
 }  // namespace
 
 // Look up the device address of `scratch` on the current device (once per device).
@@ -179,16 +176,6 @@ extern "C" int anc_gradnorm_static(uint64_t g, int64_t n, int g_dtype, float max
   int dev = 0;
   ANC_HIP(hipGetDevice(&dev));
   double *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
-  // Calls on one stream are ordered; a call on another stream is refused while the previous call's
-  // stream still has work queued (it may be that call's kernels). hipStreamQuery allocates nothing.
-  const uint64_t prev = g_last_stream[dev].exchange(stream + 1, std::memory_order_acq_rel);
-  if (prev != 0 && prev != stream + 1 && hipStreamQuery(anc_stream(prev - 1)) == hipErrorNotReady) {
-    g_last_stream[dev].store(prev, std::memory_order_release);
-    anc_set_error("anc_gradnorm_static: the previous call on this GPU, on another stream, may still be running; "
-                  "calls share one scratch array and must not overlap");
-    return ANC_ERR_UNSUPPORTED;
-  }
-  (void)hipGetLastError();      // a stale handle in the query above is not this call's error
   // Stage 1 overwrites partials [0, chunks) and stage 2 reads exactly those: nothing of an
   // earlier call is read, so nothing needs clearing.
   hipStream_t s = anc_stream(stream);

@@ -188,9 +188,9 @@ int anc_gradnorm_finalize(uint64_t partials, int64_t n_partials,
  * ends), so n is limited to anc_gradnorm_static_max_elements() = 2^31; larger n returns
  * ANC_ERR_ARG. The call allocates nothing (no hipMalloc/hipFree, no events, and it is not seen
  * by anc_profile_*). All calls on one GPU share that array: calls that overlap in time on one
- * GPU (different streams without ordering) race and must be serialised by the caller. A call on
- * another stream than the previous call's while that stream still has work queued is refused
- * (ANC_ERR_UNSUPPORTED): the one overlap the library can see without allocating anything. */
+ * GPU (different streams without ordering) race and must be serialised by the caller: issue them
+ * on one stream, or order the streams with events. (The library cannot check this for the caller
+ * without allocating: it holds no event, and a remembered stream handle may be stale.) */
 int64_t anc_gradnorm_static_max_elements(void);
 int anc_gradnorm_static(uint64_t g, int64_t n, int g_dtype, float max_norm, float eps,
                         uint64_t ctl /* anc_step_ctl_t* */, uint64_t stream);
@@ -427,77 +427,55 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *     X = X / (||X||_F + eps)
  *     for k < steps: (a,b,c) = coef[3k..3k+2];  A = X X^T;  B = b A + c A A;  X = a X + B X
  *
- *   ANC_NS_BF16       GEMM operands are bf16 at the matrix-core input, fp32 accumulate
- *                     (MFMA); between steps the iterate is carried as a bf16 pair
- *                     hi + lo (16 significant bits), the diagonals of A and B in fp32,
- *                     and where the shape needs it late iterations add the bf16
- *                     residuals of X, A, B as extra accumulation terms.
- *   ANC_NS_BF16_FAST  as ANC_NS_BF16 without the residual terms (15 GEMM passes);
- *                     no accuracy bar of its own (about 2.2e-3 on 1024x1024).
- *   ANC_NS_BF16_X3    every product also multiplies the bf16 residuals of both operands (three
- *                     accumulation terms per product in every iteration): about 1e-5 from the
- *                     fp32 chain on every input tried, ill-conditioned ones included, for three
- *                     times the matrix-core work of ANC_NS_BF16_FAST.
- *   ANC_NS_BF16_LATE3 ANC_NS_BF16 with the residual of X in its two products from iteration 2 on and
- *                     the residuals of F and Boff from iteration 3 on (chains of 5 steps and
- *                     more; all of them in the last three iterations of a shorter one) for every
- *                     matrix, and every residual from iteration 1 on for the matrices the wide
- *                     gate flags (below); none of the other gates. For M >= 1024
- *                     (M < 1024 runs a heavier plan in either mode, see below): about 2.05 times the
- *                     matrix-core work of ANC_NS_BF16_FAST. For coefficients that do not drive the
- *                     singular values to 1: Keller's quintic (ancora/kernels/muon_ns.py:21) leaves
- *                     them in 0.7 .. 1.2, offdiag(A) never becomes small and ANC_NS_BF16 reaches
- *                     2.8e-3 .. 5e-3 only; this mode 2e-5 .. 9e-4.
- *   ANC_NS_FP32       every product in fp32 (validation mode).
+ * Modes
+ *   ANC_NS_BF16       GEMM operands are bf16 at the matrix-core input, fp32 accumulate (MFMA).
+ *                     Between steps the iterate is a bf16 pair hi + lo (16 significant bits), the
+ *                     diagonals of A and B stay fp32, and selected products add the bf16 residuals
+ *                     of X, A, B as further accumulation terms: by shape (the plan) and, per
+ *                     matrix, by the gates below.
+ *   ANC_NS_BF16_FAST  the same without any residual term (15 GEMM passes); no accuracy bar of its
+ *                     own (about 2.2e-3 on 1024x1024).
+ *   ANC_NS_BF16_X3    the residuals of both operands in every product of every iteration: about
+ *                     1e-5 from the fp32 chain whatever the input, three times the matrix-core work.
+ *   ANC_NS_BF16_LATE3 for coefficients that do not drive the singular values to 1 (Keller's quintic,
+ *                     ancora/kernels/muon_ns.py:21, leaves them in 0.7 .. 1.2, so operand rounding
+ *                     stays a first-order error to the end: ANC_NS_BF16 reaches 2.8e-3 .. 5e-3 there).
+ *                     Every matrix: residual of X from iteration 2 on, of A and B from iteration 3
+ *                     on (the last three iterations of a chain shorter than 5 steps); the wide gate
+ *                     below; 2.05 times the work of ANC_NS_BF16_FAST; 2e-5 .. 9e-4.
+ *   ANC_NS_FP32       every product in fp32 (validation mode, 1e-5).
  *
- * Conditioning gates (ANC_NS_BF16 only). After the first A = X X^T the chain measures
- * N * ||offdiag(A)||_F^2 per matrix: 1.0 for independent entries whatever the row scaling (1.2 with
- * 1 % of the rows x100), 1.7 for columns scaled over 0.1..3, N/r - N/M when the Frobenius mass sits in
- * r directions spread over all rows (about 100 with 1 % of the columns x100). Later products of a
- * matrix add the residual of X (three accumulation terms in A = X X^T, two in X = a X + B X)
- * according to it:
- *   N >= 2M:  above 2.5, A = X X^T of iteration 2 (1 % of the columns x100 at 1024x3072: 1.15e-3
- *             instead of 2.2e-3), and of iteration 1 in chains shorter than 5 steps;
- *   N < 2M:   above 2.5, A = X X^T of iterations 1 and 2 (1024x1024: 8e-4 instead of 3.8e-3); above
- *             1.3, both X-products of iterations 2 and 3 (5-step chains; every matrix has them in
- *             iteration 4): a matrix with independent entries or outlier rows does without
- *             (1.67e-3 / 5e-4 at 1024x1024), column-scaled ones need them (columns scaled over
- *             0.1..3: 1.45e-3; 2.1e-3 with iteration 4 alone, 1.9e-3 with iterations 3 and 4);
- *   2M <= N < 3M: as N >= 3M (1536x3072, 2048x4096: 1.0e-3 instead of 2.1e-3 .. 2.3e-3);
- *   M < 1024: no gates. Small matrices average fewer rounding errors per element and cost next to
- *             nothing: every product carries the residuals of X, F and Boff from iteration 1 on
- *             (from iteration 0 below M = 256), for every matrix, in ANC_NS_BF16 and
- *             ANC_NS_BF16_LATE3 alike (at most 1e-3 on the input classes below, both schedules);
- *   M >= 1024, every N, chains of any length: the wide gate. A matrix takes it if its proxy lies strictly
- *             between 2.5 and 40 (a spectrum spread over two or three decades reads 3.6 .. 19, 10 %
- *             of the columns x10 reads 8.4, a rank-128 signal over weak noise 17), or if it lies
- *             outside and the matrix's column norms say what the proxy cannot: with
- *             colc = N * sum_j c_j^4 / (sum_j c_j^2)^2 over the column norms c_j of the input
- *             (every fourth row of it),
- *             proxy >= 40 and colc < proxy / 4 (a low-rank signal over weak noise, a steep
- *             spectrum: colc about 1, where outlier columns read colc = proxy and keep the cheap
- *             gates above), or proxy >= 40 and less than 3e-3 of the mass outside the outlier
- *             columns (estimated from the lightest block of 64 columns: 1 % of the columns x100
- *             leaves 1e-2 there and keeps the cheap gates, x300 and beyond 1e-3 and less), or N < 2M, 1.9 < proxy <= 2.5 and colc < 1.3 (a gap in the spectrum,
- *             e.g. near-duplicate rows; scaled columns read colc = proxy and keep the low gate).
- *             Such a matrix adds the residuals of X, F and Boff to all three products from iteration
- *             1 on (about 2.6 times the matrix-core work, for that matrix alone): condition number
- *             1e2 .. 1e4 2e-5 .. 8e-5 instead of 2.5e-3 .. 4.2e-3, rank 32 over 10 % / 1 % noise
- *             2.2e-4 / 3.9e-4 instead of 2.9e-3 / 5.0e-3, near-duplicate rows 6e-5 instead of
- *             2.4e-3, 1 % of the columns x1000 1e-4 .. 2e-4 instead of 3.6e-3 .. 4.0e-3. It takes
- *             precedence over the gates above.
- * The decision depends on the matrix alone (fixed-order sums), never on the batch. Accuracy bar of
- * ANC_NS_BF16 with the Polar-Express schedule: 2e-3 relative Frobenius on inputs with independent
- * entries, with row or column outliers up to x100 on 1 % of the rows or columns, with 10 % of the
- * columns x10, with columns scaled over a factor 30, with log-uniform spectra up to condition
- * number 1e4, with power-law spectra, with low-rank signals over noise down to 1 %, with
- * near-duplicate rows, with sparse (90 % zeros) and heavy-tailed (Student t, 1.5 degrees of freedom
- * and up) entries, with 1 % of the rows or columns x30 .. x3000, on shapes up to 4096x8192 (the
- * worst of them: 1.7e-3, independent entries at N = M). Keller coefficients amplify operand rounding about twice as much (4.5e-3 at
- * 1024x1024): with them the bar is that of ANC_NS_BF16_LATE3, which the host layer selects for
- * that schedule; it holds on the same classes except a single element of 1000 standard deviations
- * (3e-5 .. 3e-3 depending on the shape: an isolated singular value that hangs on one rounded
- * operand element and that Keller's polynomial, unlike the Polar-Express one, does not contract).
+ * Plan of ANC_NS_BF16 by shape
+ *   M < 1024          residuals of X, A, B from iteration 1 on (iteration 0 below M = 256); no gates.
+ *   M >= 1024, N < 2M residual of X in A = X X^T and X = a X + B X of the last iteration.
+ *   M >= 1024, N >= 2M  no residual term; B = b A + c A A takes the off-diagonal entries of A from the
+ *                     bf16 copy it multiplies anyway (no fp32 copy of A: 3 .. 8 % of accuracy).
+ * Gates (M >= 1024), per matrix, from statistics of the matrix alone, so that a result never
+ * depends on the batch: after the first A = X X^T, proxy = N * ||offdiag(A)||_F^2 (1.0 for independent
+ * entries whatever the row scaling, 1.7 for columns scaled over 0.1 .. 3, about N/r when the mass sits
+ * in r directions); for some ranges of it the column concentration colc = N * sum_j c_j^4 /
+ * (sum_j c_j^2)^2 over the column norms c_j of the input (every fourth row), which equals the proxy
+ * exactly when column norms explain it, and the share of the mass in the lightest 64-column block.
+ *   proxy > 1.3, N < 2M     residual of X in both X-products of iterations 2 and 3 (5-step chains);
+ *   proxy > 2.5             residual of X in A = X X^T of iteration 2 (N >= 2M; also iteration 1 in
+ *                           chains shorter than 5 steps) or of iterations 1 and 2 (N < 2M);
+ *   the wide gate           every residual in all three products from iteration 1 on (2.6 times the
+ *                           work, for that matrix alone; it keeps the fp32 copy of A) if
+ *                           2.5 < proxy < 40 (spectra spread over decades, many moderately large
+ *                           columns), or proxy >= 40 and (colc < 0.85 proxy: a low-rank signal, a
+ *                           steep spectrum, alone or mixed with outlier columns; or less than 3e-3 of
+ *                           the mass outside the outlier columns), or N < 2M, 1.5 < proxy <= 2.5 and
+ *                           colc < 0.85 proxy (a gap in the spectrum, e.g. near-duplicate rows).
+ * Accuracy bar of ANC_NS_BF16 under the Polar-Express schedule (ANC_NS_BF16_LATE3 under Keller's):
+ * 2e-3 relative Frobenius against the fp32 chain, held on independent, sparse and heavy-tailed
+ * entries, row or column outliers (1 % x30 .. x3000, 10 % x10), scaled columns, log-uniform spectra
+ * up to condition number 1e4, power-law spectra, low-rank signals over noise down to 1 %,
+ * near-duplicate rows, shapes up to 4096x8192, chains of 3 .. 8 steps. Known limits: a low-rank
+ * bulk hidden behind independent outlier columns (the column norms explain the proxy, the bulk's own
+ * spectrum is not seen: 2.5e-3 at 1024x3072); for N >= 2M a gap in the spectrum with flat column
+ * norms and a proxy between 1.2 and 2.5 (a quarter of the rows near-copies of other rows: 2.2e-3 ..
+ * 4.6e-3; N < 2M and proxies above 2.5 are covered); under Keller a single element of 1000 standard
+ * deviations (up to 3e-3). ANC_NS_BF16_X3 has none of them.
  *
  * M and N must be multiples of 128 (the reference's tile alignment,
  * ancora/optim/muon.py:98). workspace must hold anc_ns_workspace_bytes(E,M,N,mode)

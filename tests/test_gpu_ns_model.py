@@ -1,0 +1,54 @@
+"""Pins the numpy model of the bf16 chain (oracle/ns_chain_model.py) to the GPU: on every input
+class of the sweep and the threshold families, at the three BASELINE shapes, the model's error
+against `host_ns` agrees with the GPU's to the two digits it is trusted for, and the model takes
+the GPU's gate decisions. The CPU tests that walk the thresholds (tests/test_oracle_ns_model.py)
+rest on this."""
+import numpy as np
+import pytest
+
+from oracle import ns_inputs as I
+from oracle.muon_ref import host_ns, PE_SCHEDULE
+from oracle.ns_chain_model import chain
+from util import rel_fro
+from test_gpu_ns import run_ns, _hard_count
+from test_gpu_ns_classes import classes
+
+pytestmark = pytest.mark.gpu
+
+
+def _families(M, N):
+    yield "scaled columns 1.35", I.scaled_columns(M, N, I.solve_knob(lambda v: I.scaled_columns(M, N, v), 1.35, 0.0, 1.0))
+    yield "duplicated rows 1.45", I.duplicated_rows(M, N, I.solve_knob(lambda v: I.duplicated_rows(M, N, v), 1.45, 0.0, 1.0))
+    yield "duplicated rows 1.6", I.duplicated_rows(M, N, I.solve_knob(lambda v: I.duplicated_rows(M, N, v), 1.6, 0.0, 1.0))
+    yield "log spectrum 2.4", I.log_spectrum(M, N, I.solve_knob(lambda v: I.log_spectrum(M, N, v), 2.4, 0.0, 3.0))
+    yield "outlier columns 42", I.outlier_columns(M, N, N // 50, I.solve_knob(lambda v: I.outlier_columns(M, N, N // 50, v), 42.0, 1.0, 100.0))
+    yield "low rank + columns", I.low_rank_plus_columns(M, N, 32, 0.1, N // 100, 12.0)
+    yield "outlier columns x159", I.outlier_columns(M, N, N // 100, 159.0)
+
+
+@pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 2048), (1024, 3072)])
+def test_model_reproduces_the_gpu_chain(gpu, M, N):
+    rng = np.random.default_rng(M * 7 + N)
+    items = list(classes(M, N, rng)) + list(_families(M, N))
+    names, mats = zip(*items)
+    got = run_ns(np.stack(mats))
+    rows = []
+    for e, (name, X) in enumerate(items):
+        ref = host_ns(X, PE_SCHEDULE, 5)
+        info = {}
+        model = chain(X, PE_SCHEDULE, 5, "bf16", info=info)
+        alone = run_ns(X[None])                        # this matrix's own gate decision
+        n_gated, _ = _hard_count(1, M, N)
+        p = info["plan"]
+        model_gated = info["wide"] or any(info["proxy"] > tau for tau in p.gate_tau.values())
+        rows.append((name, rel_fro(got[e], ref), rel_fro(model, ref), bool(n_gated), model_gated,
+                     rel_fro(alone[0], got[e])))
+    print(f"\n({M},{N})  class: GPU error / model error (gated)")
+    for name, eg, em, gg, mg, _ in rows:
+        print(f"  {name:24s} {eg:.3e} / {em:.3e}  {'gated' if gg else ''}")
+    for name, eg, em, gg, mg, batch in rows:
+        assert batch == 0.0, name                      # the batch does not enter a matrix's bits
+        assert gg == mg, (name, "gate decision")
+        # two digits: within 12 % of each other, or both below 1e-4 (there the accumulation order
+        # of the products, which the model does not share, is the error)
+        assert abs(eg - em) <= 0.12 * max(eg, em) or max(eg, em) < 1e-4, (name, eg, em)
