@@ -458,6 +458,8 @@ __global__ void __launch_bounds__(kThreads) k_ns_cond(NsCondArgs a) {
 // the partial sums in order and writes the flag every later product reads.
 struct WideRule {
   double near_lo, lo, hi;    // in units of the proxy N * ||offdiag(A0)||^2; near_lo == lo: no near range
+  double near_diff;          // > 0: in the near range the gate takes a matrix whose proxy exceeds its column
+                             // concentration by more than this; 0: the kColcFrac rule there as above the band
 };
 // kBulkShare: outlier columns keep the cheap gates while the other columns still hold a few
 // thousandths of the mass (1 % of the columns x100: 1e-2 of it, 8e-4 .. 1.6e-3 with those gates);
@@ -561,7 +563,8 @@ __global__ void __launch_bounds__(kThreads) k_ns_classify(NsColArgs a) {
     const double colc = s2 > 0.0 ? (double)N * s4 / (s2 * s2) : 1.0;
     // outlier columns: the share of the mass outside them, from the lightest block of columns
     const double bulk = s2 > 0.0 ? (double)a.parts[q] * lightest / s2 : 1.0;
-    wide = colc < kColcFrac * p || (p >= r.hi && bulk < kBulkShare);
+    if (p < r.hi && r.near_diff > 0.0) wide = p - colc > r.near_diff;
+    else wide = colc < kColcFrac * p || (p >= r.hi && bulk < kBulkShare);
   }
   a.flag[q][e] = wide ? 1 : 0;
 }
@@ -599,6 +602,7 @@ struct SplitPlan {
   // wide_gram_from on and the residuals of X, F and Boff to all three products from iteration
   // wide_all_from on. wide_hi == 0: no such gate.
   float wide_lo, wide_hi, wide_near;   // wide_near: start of the near range below the band (== wide_lo: none)
+  float wide_near_diff;                // see WideRule::near_diff
   int wide_gram_from, wide_all_from;
   // No fp32 copy of A except for the matrices the wide gate flags: B = b A + c A A takes the
   // off-diagonal entries of A from the bf16 Fh it multiplies anyway. Costs 3 .. 8 % of accuracy where
@@ -654,11 +658,19 @@ struct SplitPlan {
 //     1.5e-3 .. 2.7e-3.
 //   N >= 2M carries no residual term in its plan and has no low gate: an input whose spectrum has
 //     a gap with flat column norms (a fraction of near-duplicate rows, proxy 1 + twice that fraction
-//     times N/M) leaves the bar between proxy 1.2 and the band of the wide gate: 1024x2048 reads
-//     1.80e-3 at proxy 1.15, 2.15e-3 at 1.3, 2.8e-3 at 1.6, 4.6e-3 at 2.3 (1024x3072: 1.57e-3,
-//     1.91e-3, 2.5e-3, 3.7e-3). The residual of X in both X-products of iterations 2 .. 4 would hold
-//     them at 6e-4 .. 1.4e-3 (numpy model of this chain); a gate for it was built and taken out again
-//     (a GPU fault in the test run that carried it, cause not found): a known limit of ANC_NS_BF16.
+//     times N/M) would leave the bar between proxy 1.2 and the band: 1024x2048 reads 1.80e-3 at
+//     proxy 1.15, 2.15e-3 at 1.3, 2.8e-3 at 1.6, 4.6e-3 at 2.3 (1024x3072: 1.57e-3, 1.91e-3, 2.5e-3,
+//     3.7e-3) with the plan alone. What decides is the part of the proxy the column norms do not
+//     explain: with the columns of such a matrix scaled by exp(sigma z), sigma 0 .. 0.4 (proxy up to
+//     2.5), the error stays a function of proxy - colc alone (0.10: 1.67e-3 .. 1.76e-3, 0.19: 1.90e-3
+//     .. 1.94e-3, 0.29: 2.12e-3 .. 2.15e-3, 0.5: 2.5e-3 .. 2.6e-3 at 1024x2048), where the ratio
+//     colc / proxy moves from 0.78 to 0.87. So the near range of these shapes starts at
+//     kTauWideNear2M and takes a matrix with proxy - colc > kNearDiff2M (the wide gate's terms: 1e-5
+//     .. 5e-5). Independent entries, outlier rows, scaled or outlier columns and heavy tails read
+//     proxy - colc < 0.01. (A cheaper gate for the range -- the residual of X in both X-products of
+//     iterations 2 .. 4, 6e-4 .. 1.4e-3 in the numpy model of this chain -- was built and taken out
+//     again: a GPU fault in the test run that carried it, cause not found.)
+constexpr float kTauWideNear2M = 1.15f, kNearDiff2M = 0.15f;
 constexpr float kTauHard = 2.5f, kTauPlain = 1.3f, kTauWideLo = 2.5f, kTauWideHi = 40.0f, kTauWideNear = 1.5f;
 SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
   SplitPlan sp{};
@@ -705,6 +717,7 @@ SplitPlan split_plan(int64_t M, int64_t N, int mode, int steps) {
                                               // (cond 1e3 without: 6 steps 4.4e-3 .. 7e-3, 8 steps 6e-3 .. 1.8e-2)
       sp.wide_lo = kTauWideLo; sp.wide_hi = kTauWideHi;
       sp.wide_near = N < 2 * M ? kTauWideNear : kTauWideLo;
+      if (mode == ANC_NS_BF16 && N >= 2 * M) { sp.wide_near = kTauWideNear2M; sp.wide_near_diff = kNearDiff2M; }
       sp.wide_gram_from = 1; sp.wide_all_from = 1;
     }
     if (N < 2 * M) {
@@ -963,7 +976,8 @@ int run_bf16_chain(ChainProb *cp, int n, int steps, const float *coef, bool forc
         const int i = cs.n;
         cs.Xh[i] = cp[q].inH; cs.cond[i] = pl.cond; cs.part[i] = pl.colpart; cs.flag[i] = pl.wide_flag;
         cs.M[i] = (int)cp[q].M; cs.N[i] = (int)cp[q].N; cs.parts[i] = pl.col_parts;
-        cs.rule[i] = WideRule{(double)pl.sp.wide_near, (double)pl.sp.wide_lo, (double)pl.sp.wide_hi};
+        cs.rule[i] = WideRule{(double)pl.sp.wide_near, (double)pl.sp.wide_lo, (double)pl.sp.wide_hi,
+                              (double)pl.sp.wide_near_diff};
         cs.blocks[i] = (int)(cp[q].E * pl.col_parts);
         cs_blocks += cs.blocks[i];
         ++cs.n;

@@ -63,7 +63,7 @@ struct NsGemm {
   int lower;                 // symmetric output: tiles with tn <= tm only, mirrored
   int plain_sum;             // plain product: 1 = write X32 = (A32, if not null, else 0) + A B and, if Yh is
                              // not null, its bf16 copy (RNE) to Yh; 0 = write X32 = A B
-  int blk_r, blk_c;          // plain product: the tile sequence of a matrix runs block by block, blocks of
+  int blk_r, blk_c;          // plain product and X = a X + B X: the tile sequence of a matrix runs block by block, blocks of
                              // blk_r x blk_c tiles (rows x columns): (tiles_m, 1) = column panel by column
                              // panel, (1, tiles_n) or 0 = row by row
   int M, N;                  // matrix dims of the chain (A, B are MxM; X is MxN)

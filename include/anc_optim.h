@@ -464,18 +464,18 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *                           2.5 < proxy < 40 (spectra spread over decades, many moderately large
  *                           columns), or proxy >= 40 and (colc < 0.85 proxy: a low-rank signal, a
  *                           steep spectrum, alone or mixed with outlier columns; or less than 3e-3 of
- *                           the mass outside the outlier columns), or N < 2M, 1.5 < proxy <= 2.5 and
- *                           colc < 0.85 proxy (a gap in the spectrum, e.g. near-duplicate rows).
+ *                           the mass outside the outlier columns), or just below the band, where the
+ *                           column norms leave part of the proxy unexplained (a gap in the spectrum,
+ *                           e.g. near-duplicate rows): N < 2M, 1.5 < proxy <= 2.5 and colc < 0.85
+ *                           proxy; N >= 2M, 1.15 < proxy <= 2.5 and proxy - colc > 0.15.
  * Accuracy bar of ANC_NS_BF16 under the Polar-Express schedule (ANC_NS_BF16_LATE3 under Keller's):
  * 2e-3 relative Frobenius against the fp32 chain, held on independent, sparse and heavy-tailed
  * entries, row or column outliers (1 % x30 .. x3000, 10 % x10), scaled columns, log-uniform spectra
  * up to condition number 1e4, power-law spectra, low-rank signals over noise down to 1 %,
  * near-duplicate rows, shapes up to 4096x8192, chains of 3 .. 8 steps. Known limits: a low-rank
  * bulk hidden behind independent outlier columns (the column norms explain the proxy, the bulk's own
- * spectrum is not seen: 2.5e-3 at 1024x3072); for N >= 2M a gap in the spectrum with flat column
- * norms and a proxy between 1.2 and 2.5 (a quarter of the rows near-copies of other rows: 2.2e-3 ..
- * 4.6e-3; N < 2M and proxies above 2.5 are covered); under Keller a single element of 1000 standard
- * deviations (up to 3e-3). ANC_NS_BF16_X3 has none of them.
+ * spectrum is not seen: 2.5e-3 at 1024x3072); under Keller a single element of 1000 standard
+ * deviations (up to 3e-3). ANC_NS_BF16_X3 has neither.
  *
  * M and N must be multiples of 128 (the reference's tile alignment,
  * ancora/optim/muon.py:98). workspace must hold anc_ns_workspace_bytes(E,M,N,mode)

@@ -29,6 +29,7 @@ f32 = np.float32
 TAU_HARD, TAU_PLAIN = 2.5, 1.3
 TAU_WIDE_LO, TAU_WIDE_HI, TAU_WIDE_NEAR = 2.5, 40.0, 1.5
 COLC_FRAC, BULK_SHARE = 0.85, 3e-3
+TAU_WIDE_NEAR_2M, NEAR_DIFF_2M = 1.15, 0.15
 COL_BLOCK, COL_ROW_STEP = 64, 4
 
 
@@ -43,6 +44,7 @@ class Plan:
         self.gate_bx_hi = None       # upper bound of the X = a X + B X gates
         self.wide = False
         self.wide_near = TAU_WIDE_LO
+        self.wide_near_diff = 0.0    # > 0: the near range flags on proxy - colc > this instead of the ratio rule
         self.wide_from = 1
         self.drop_a32 = False
         if mode == "bf16_x3":
@@ -61,6 +63,8 @@ class Plan:
             self.drop_a32 = mode == "bf16" and N >= 2 * M
             if steps >= 2:
                 self.wide, self.wide_near = True, (TAU_WIDE_NEAR if N < 2 * M else TAU_WIDE_LO)
+                if mode == "bf16" and N >= 2 * M:
+                    self.wide_near, self.wide_near_diff = TAU_WIDE_NEAR_2M, NEAR_DIFF_2M
             if N < 2 * M:
                 self.x_from = min(steps - 2, 3)
                 self.gate_tau = {1: TAU_HARD, 2: TAU_HARD}
@@ -105,6 +109,8 @@ def wide_flag(plan, proxy, colc, bulk):
     if proxy >= TAU_WIDE_HI:
         return colc < COLC_FRAC * proxy or bulk < BULK_SHARE
     if plan.wide_near < proxy <= TAU_WIDE_LO:
+        if plan.wide_near_diff > 0:
+            return proxy - colc > plan.wide_near_diff
         return colc < COLC_FRAC * proxy
     return False
 

@@ -33,6 +33,21 @@ def duplicated_rows(M, N, frac, seed=0):
     return g
 
 
+def gap_scaled_columns(M, N, frac, sigma, seed=0):
+    """`duplicated_rows` with its columns scaled by exp(sigma z): the gap raises the proxy and leaves
+    the column concentration alone, the scaling raises both by the same amount."""
+    scale = np.exp(sigma * np.random.default_rng(seed + 1).standard_normal(N)).astype(f32)
+    return duplicated_rows(M, N, frac, seed) * scale[None, :]
+
+
+def unexplained_proxy(X):
+    """proxy - colc in fp64 over all rows: the part of the proxy the column norms do not explain
+    (the chain samples every fourth row for colc: flat columns then read 0.006 more)."""
+    X = np.asarray(X, dtype=np.float64)
+    c2 = np.sum(X * X, axis=0)
+    return proxy_of(X) - X.shape[1] * float(np.sum(c2 * c2)) / float(np.sum(c2)) ** 2
+
+
 def log_spectrum(M, N, decades, seed=0):
     """Singular values log-uniform over `decades` decades, random singular vectors."""
     rng = np.random.default_rng(seed)

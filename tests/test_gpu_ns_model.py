@@ -1,5 +1,5 @@
 """Pins the numpy model of the bf16 chain (oracle/ns_chain_model.py) to the GPU: on every input
-class of the sweep and the threshold families, at the three BASELINE shapes, the model's error
+class of the sweep and nine threshold families, at the three BASELINE shapes, the model's error
 against `host_ns` agrees with the GPU's to the two digits it is trusted for, and the model takes
 the GPU's gate decisions. The CPU tests that walk the thresholds (tests/test_oracle_ns_model.py)
 rest on this."""
@@ -20,6 +20,9 @@ def _families(M, N):
     yield "scaled columns 1.35", I.scaled_columns(M, N, I.solve_knob(lambda v: I.scaled_columns(M, N, v), 1.35, 0.0, 1.0))
     yield "duplicated rows 1.45", I.duplicated_rows(M, N, I.solve_knob(lambda v: I.duplicated_rows(M, N, v), 1.45, 0.0, 1.0))
     yield "duplicated rows 1.6", I.duplicated_rows(M, N, I.solve_knob(lambda v: I.duplicated_rows(M, N, v), 1.6, 0.0, 1.0))
+    for d in (0.11, 0.19):             # either side of the N >= 2M near range's rule, columns scaled on top
+        f = I.solve_knob(lambda v: I.gap_scaled_columns(M, N, v, 0.4), d, 0.0, 0.5, stat=I.unexplained_proxy)
+        yield f"gap + scaled columns {d}", I.gap_scaled_columns(M, N, f, 0.4)
     yield "log spectrum 2.4", I.log_spectrum(M, N, I.solve_knob(lambda v: I.log_spectrum(M, N, v), 2.4, 0.0, 3.0))
     yield "outlier columns 42", I.outlier_columns(M, N, N // 50, I.solve_knob(lambda v: I.outlier_columns(M, N, N // 50, v), 42.0, 1.0, 100.0))
     yield "low rank + columns", I.low_rank_plus_columns(M, N, 32, 0.1, N // 100, 12.0)
@@ -52,3 +55,5 @@ def test_model_reproduces_the_gpu_chain(gpu, M, N):
         # two digits: within 12 % of each other, or both below 1e-4 (there the accumulation order
         # of the products, which the model does not share, is the error)
         assert abs(eg - em) <= 0.12 * max(eg, em) or max(eg, em) < 1e-4, (name, eg, em)
+        if name.startswith(("duplicated rows", "gap +")):
+            assert eg < 2e-3, (name, eg)                # the near ranges hold the bar on either side

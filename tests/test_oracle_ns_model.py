@@ -11,7 +11,8 @@ import pytest
 from oracle import ns_inputs as I
 from oracle.bf16_ref import bf16_round
 from oracle.muon_ref import PE_SCHEDULE, host_ns
-from oracle.ns_chain_model import Plan, chain, statistics, TAU_PLAIN, TAU_HARD, TAU_WIDE_NEAR, TAU_WIDE_HI, COLC_FRAC, BULK_SHARE
+from oracle.ns_chain_model import (Plan, chain, statistics, TAU_PLAIN, TAU_HARD, TAU_WIDE_NEAR, TAU_WIDE_HI, COLC_FRAC,
+                                   BULK_SHARE, NEAR_DIFF_2M)
 
 BAR = 2e-3
 
@@ -83,23 +84,28 @@ def test_near_range_from_both_sides(M, N):
 
 
 @pytest.mark.parametrize("M,N", [(1024, 2048), (1024, 3072)])
-def test_known_limit_gap_spectrum_on_wide_shapes(M, N):
-    """N >= 2M has no residual term in its plan and no low gate. A gap in the spectrum with flat
-    column norms (a fraction of near-duplicate rows) between proxy 1.3 and the wide gate's band is
-    therefore outside the bar (stated in the header as a known limit); the residual of X in both
-    X-products of iterations 2 .. 4 would hold it. This test keeps both numbers honest."""
-    f = I.solve_knob(lambda v: I.duplicated_rows(M, N, v), 1.6, 0.0, 1.0)
+def test_near_range_of_wide_shapes_from_both_sides(M, N):
+    """N >= 2M has no residual term in its plan and no low gate: a gap in the spectrum with flat
+    column norms (a fraction of near-duplicate rows) would leave the bar from proxy 1.25 on. Its near
+    range takes a matrix whose proxy exceeds its column concentration by more than NEAR_DIFF_2M:
+    either side of that, the same with the columns scaled on top (the part of the proxy the columns
+    explain does not count: a ratio rule would miss the scaled case), and the top of the range."""
+    for sigma in (0.0, 0.4):
+        for target, wide in ((NEAR_DIFF_2M - 0.03, False), (NEAR_DIFF_2M + 0.03, True), (0.3, True)):
+            f = I.solve_knob(lambda v: I.gap_scaled_columns(M, N, v, sigma), target, 0.0, 0.5, stat=I.unexplained_proxy)
+            err, info = run(I.gap_scaled_columns(M, N, f, sigma))
+            assert info["wide"] == wide, (sigma, target, info["proxy"], info["colc"])
+            assert err < (BAR if not wide else 1e-4), (sigma, target, err)
+    f = I.solve_knob(lambda v: I.duplicated_rows(M, N, v), 2.3, 0.0, 1.0)
+    err, info = run(I.duplicated_rows(M, N, f))
+    assert info["wide"] and err < 1e-4
+    # what the plan alone would leave there (the price list of the gate)
     X = I.duplicated_rows(M, N, f)
-    ref = host_ns(X, PE_SCHEDULE, 5)
-    info = {}
-    plain = rel(chain(X, PE_SCHEDULE, 5, "bf16", info=info), ref)
-    assert not info["wide"] and 2e-3 < plain < 3.2e-3
-    fixed = rel(chain(X, PE_SCHEDULE, 5, "bf16", overrides={"gram3": (2, 3, 4), "bx_l": (2, 3, 4)}), ref)
-    assert fixed < 1.3e-3
-    # below proxy 1.15 the plan holds the bar by itself
-    f = I.solve_knob(lambda v: I.duplicated_rows(M, N, v), 1.12, 0.0, 1.0)
-    err, _ = run(I.duplicated_rows(M, N, f))
-    assert err < BAR
+    assert rel(chain(X, PE_SCHEDULE, 5, "bf16", overrides={"wide": False}), host_ns(X, PE_SCHEDULE, 5)) > 3e-3
+    # scaled columns with a proxy inside the range: the columns explain it, no gate, inside the bar
+    s = I.solve_knob(lambda v: I.scaled_columns(M, N, v), 2.0, 0.0, 1.0)
+    err, info = run(I.scaled_columns(M, N, s))
+    assert not info["wide"] and abs(info["proxy"] - info["colc"]) < 0.05 and err < BAR
 
 
 @pytest.mark.parametrize("M,N", [(1024, 1024), (1024, 3072)])
@@ -110,7 +116,8 @@ def test_band_edges_from_both_sides(M, N):
     for target in (TAU_HARD - 0.1, TAU_HARD + 0.1):
         d = I.solve_knob(lambda v: I.log_spectrum(M, N, v), target, 0.0, 3.0)
         err, info = run(I.log_spectrum(M, N, d))
-        assert info["wide"] == (target > TAU_HARD or (N < 2 * M and info["colc"] < COLC_FRAC * info["proxy"]))
+        near = info["colc"] < COLC_FRAC * info["proxy"] if N < 2 * M else info["proxy"] - info["colc"] > NEAR_DIFF_2M
+        assert info["wide"] == (target > TAU_HARD or near)
         assert err < BAR, ("log spectrum", target, err)
     r = N // 50
     for target, wide in ((TAU_WIDE_HI - 2, True), (TAU_WIDE_HI + 2, False)):
