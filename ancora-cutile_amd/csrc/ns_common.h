@@ -109,6 +109,15 @@ struct NsGemm {
   int f_panel;               // Fh, Fl, Bh, Bl are in panel layout (GRAM, BMAT write them so; BMAT, BX read them so)
   int x_panel;               // the input iterate (operands X of GRAM and BX, Xh/Xl of the BX epilogue)
   int y_panel;               // the output iterate Yh/Yl of BX
+  // 8-bit low halves (256-tile X = a X + B X, panel layout only). Where the low half of a matrix's
+  // iterate is never a matrix-core operand it is kept as one byte per element (anc_low8_encode), in the first M*N bytes of the matrix's Xl (Yl) region, panels of
+  // (M, 32) bytes: the epilogue then reads and writes 3 instead of 4 bytes per element. A matrix
+  // takes the format on the input side if l8_in > 0, it is not flagged in l8_wide and its proxy
+  // sum (l8_cond, the units of cond_thresh) does not exceed l8_in; l8_out likewise for the output.
+  // The launches that read an iterate must be given the threshold it was written with.
+  const double *l8_cond;     // (E, kCondParts) or null (no matrix takes the format)
+  const int32_t *l8_wide;    // (E) or null
+  double l8_in, l8_out;
 };
 
 
@@ -130,6 +139,30 @@ __device__ __forceinline__ bool anc_ns_wide(const NsGemm &p, int e) {
 __device__ __forceinline__ bool anc_ns_has_a32(const NsGemm &p, int e) {
   if (p.A32 == nullptr) return false;
   return p.a32_gated == 0 || (p.a32_flag != nullptr && p.a32_flag[e] != 0);
+}
+// Is the low half of matrix e's iterate one byte per element (thresh = p.l8_in or p.l8_out)?
+__device__ __forceinline__ bool anc_ns_low8(const NsGemm &p, int e, double thresh) {
+  if (!(thresh > 0.0) || p.l8_cond == nullptr) return false;
+  if (p.l8_wide != nullptr && p.l8_wide[e] != 0) return false;
+  const double *c = p.l8_cond + (int64_t)e * kCondParts;
+  double s = c[0];
+#pragma unroll
+  for (int i = 1; i < kCondParts; ++i) s = s + c[i];
+  return !(s > thresh);
+}
+// The 8-bit low half of y next to its high half h = bf16(y), in the integer space of the fp32 bit
+// patterns, where rounding to bf16 is rounding to a multiple of 0x10000: d = bits(y) - (h << 16) lies
+// in -0x8000 .. 0x8000, and q = (d + 0x80) >> 8 (capped at 127) is d rounded to 8 bits. The pair reads
+// back as the float whose bits are (h << 16) + (q << 8): y to 24 bits, exponent carries and borrows
+// included, no special cases. `htop` is h in the upper half of a dword (lower half zero).
+__device__ __forceinline__ uint32_t anc_low8_encode(float y, uint32_t htop) {
+  int d = (int)(__float_as_uint(y) - htop) + 0x80;
+  d = d < 0x7FFF ? d : 0x7FFF;
+  return ((uint32_t)d >> 8) & 0xFFu;
+}
+// x = Xh + Xl from htop and the byte q, sign-extended
+__device__ __forceinline__ float anc_low8_decode(uint32_t htop, int q) {
+  return __uint_as_float(htop + ((uint32_t)q << 8));
 }
 __device__ __forceinline__ int anc_ns_terms(const NsGemm &p, int e) {
   if (p.nterms_wide > 0 && anc_ns_wide(p, e)) return p.nterms_wide;

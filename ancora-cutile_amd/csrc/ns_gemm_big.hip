@@ -500,6 +500,12 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const uint32_t vo_in1 = x_pan ? (uint32_t)((lane >> 3) * 64 + (int64_t)(ci1 >> 2) * panel + (ci1 & 3) * 16)
                                 : (uint32_t)((lane >> 3) * N * 2 + ci1 * 16);
   const int64_t in_row = x_pan ? 64 : (int64_t)N * 2;       // bytes between consecutive rows of the slab
+  // 8-bit low halves (NsGemm::l8_in, l8_out; uniform over the workgroup: a function of the
+  // matrix): a 32x64 slab of bytes is 32 rows of two (M, 32)-byte panels, 1 KiB contiguous each: 2
+  // DMA instructions instead of 4, in the buffer [panel][row][32 bytes].
+  // (readfirstlane: the flags live in scalar registers, so the branches on them are scalar branches)
+  const bool in8 = EPI == EPI_BX && !PLAINV && __builtin_amdgcn_readfirstlane((int)anc_ns_low8(p, e, p.l8_in)) != 0;
+  const bool out8 = EPI == EPI_BX && !PLAINV && __builtin_amdgcn_readfirstlane((int)anc_ns_low8(p, e, p.l8_out)) != 0;
   auto fetch_in = [&](int bi) {
     const int64_t ub = x_pan ? mn * 2 + (int64_t)(gj0w / 32) * panel + (int64_t)(gi0w + bi * 32) * 64
                              : (mn + (int64_t)(gi0w + bi * 32) * N + gj0w) * 2;
@@ -509,7 +515,13 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       const int64_t ro = (int64_t)(8 * j) * in_row;
       const uint32_t vo = (j & 1) ? vo_in1 : vo_in0;
       dma16_epi((const char *)p.Xh + ub + ro + vo, lds_addr(b + j * 1024));
-      dma16_epi((const char *)p.Xl + ub + ro + vo, lds_addr(b + 4096 + j * 1024));
+      if (!in8) dma16_epi((const char *)p.Xl + ub + ro + vo, lds_addr(b + 4096 + j * 1024));
+    }
+    if (in8) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        dma16_epi((const char *)p.Xl + mn * 2 + ((int64_t)(gj0w / 32 + j) * M + gi0w + bi * 32) * 32 + lane * 16,
+                  lds_addr(b + 4096 + j * 1024));
     }
   };
   // B = b A + c A A reads A32 at the output position the same way: a 32x64 fp32 slab is 32 rows
@@ -618,14 +630,28 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       // the fetch of slab bi this wavefront issued the 8 row stores of slab bi-1 and the fetch
       // of slab bi+1 (8 DMA); in the fused update the stores of a slab are 8 (master) + 8 (bf16
       // copy, if there is one) and the 8 master loads of slab bi are younger too.
+      // A slab's fetch is 8 DMA instructions, 6 with an 8-bit low half; its pair stores 8 or 6.
       if (plain) {
         // no inputs: nothing to wait for
       } else if (!fused) {
-        if (bi == 0 || bi == 3) wait_vm<8>(); else wait_vm<16>();
-      } else if (W16 != nullptr) {
-        if (bi == 0) wait_vm<16>(); else if (bi == 3) wait_vm<24>(); else wait_vm<32>();
+        if (bi == 0) { if (in8) wait_vm<6>(); else wait_vm<8>(); }
+        else if (bi == 3) { if (out8) wait_vm<6>(); else wait_vm<8>(); }
+        else if (in8 && out8) wait_vm<12>();
+        else if (in8 || out8) wait_vm<14>();
+        else wait_vm<16>();
       } else {
-        if (bi == 0) wait_vm<16>(); else if (bi == 3) wait_vm<16>(); else wait_vm<24>();
+        // (the fused launch writes no iterate: out8 does not occur)
+        if (W16 != nullptr) {
+          if (bi == 0) { if (in8) wait_vm<14>(); else wait_vm<16>(); }
+          else if (bi == 3) wait_vm<24>();
+          else if (in8) wait_vm<30>();
+          else wait_vm<32>();
+        } else {
+          if (bi == 0) { if (in8) wait_vm<14>(); else wait_vm<16>(); }
+          else if (bi == 3) wait_vm<16>();
+          else if (in8) wait_vm<22>();
+          else wait_vm<24>();
+        }
       }
       unsigned char *b = inbuf(bi);
       float y[2][16];
@@ -636,26 +662,49 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           for (int r = 0; r < 16; ++r) y[bj][r] = acc[bi][bj][r];
       } else {
         const float dr = *(const float *)(dvec_lds + (bi * 32 + rr) * 4);
-        anc_u32x2 xh[2][4], xl[2][4];
-#pragma unroll
-        for (int bj = 0; bj < 2; ++bj)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int off = rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8;
-            xh[bj][q] = *(const anc_u32x2 *)(b + off);
-            xl[bj][q] = *(const anc_u32x2 *)(b + 4096 + off);
-          }
         const float cf = p.ca + dr;
+        if (!in8) {
+          anc_u32x2 xh[2][4], xl[2][4];
 #pragma unroll
-        for (int bj = 0; bj < 2; ++bj)
+          for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const uint32_t wh = (r & 2) ? xh[bj][r >> 2].y : xh[bj][r >> 2].x;
-            const uint32_t wl = (r & 2) ? xl[bj][r >> 2].y : xl[bj][r >> 2].x;
-            const float x = ((r & 1) ? __uint_as_float(wh & 0xFFFF0000u) : __uint_as_float(wh << 16)) +
-                            ((r & 1) ? __uint_as_float(wl & 0xFFFF0000u) : __uint_as_float(wl << 16));
-            y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
-          }
+            for (int q = 0; q < 4; ++q) {
+              const int off = rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8;
+              xh[bj][q] = *(const anc_u32x2 *)(b + off);
+              xl[bj][q] = *(const anc_u32x2 *)(b + 4096 + off);
+            }
+#pragma unroll
+          for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const uint32_t wh = (r & 2) ? xh[bj][r >> 2].y : xh[bj][r >> 2].x;
+              const uint32_t wl = (r & 2) ? xl[bj][r >> 2].y : xl[bj][r >> 2].x;
+              const float x = ((r & 1) ? __uint_as_float(wh & 0xFFFF0000u) : __uint_as_float(wh << 16)) +
+                              ((r & 1) ? __uint_as_float(wl & 0xFFFF0000u) : __uint_as_float(wl << 16));
+              y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
+            }
+        } else {
+          // 8-bit low halves: w8[bj][q] holds the 4 bytes of columns bj*32 + 8q + 4hh .. +3 of row
+          // rr, which with the high half give x directly
+          anc_u32x2 xh[2][4];
+          uint32_t w8[2][4];
+#pragma unroll
+          for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              xh[bj][q] = *(const anc_u32x2 *)(b + rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8);
+              w8[bj][q] = *(const uint32_t *)(b + 4096 + bj * 1024 + rr * 32 + q * 8 + hh * 4);
+            }
+#pragma unroll
+          for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const uint32_t wh = (r & 2) ? xh[bj][r >> 2].y : xh[bj][r >> 2].x;
+              const uint32_t htop = (r & 1) ? (wh & 0xFFFF0000u) : (wh << 16);
+              const float x = anc_low8_decode(htop, (int)(w8[bj][r >> 2] << (24 - 8 * (r & 3))) >> 24);
+              y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
+            }
+        }
       }
       if (fp32_out || fused || plain) {
         // fp32 result: [32 rows][16 chunks of 16 B], chunk XOR (row & 15)
@@ -728,18 +777,35 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           }
         }
       } else {
+        if (!out8) {
 #pragma unroll
-        for (int bj = 0; bj < 2; ++bj)
+          for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            uint32_t h0, l0, h1, l1;
-            anc_pk_pair(y[bj][4 * q], y[bj][4 * q + 1], h0, l0);
-            anc_pk_pair(y[bj][4 * q + 2], y[bj][4 * q + 3], h1, l1);
-            const anc_u32x2 wh = {h0, h1}, wl = {l0, l1};
-            const int off = rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8;
-            *(anc_u32x2 *)(b + off) = wh;
-            *(anc_u32x2 *)(b + 4096 + off) = wl;
-          }
+            for (int q = 0; q < 4; ++q) {
+              uint32_t h0, l0, h1, l1;
+              anc_pk_pair(y[bj][4 * q], y[bj][4 * q + 1], h0, l0);
+              anc_pk_pair(y[bj][4 * q + 2], y[bj][4 * q + 3], h1, l1);
+              const anc_u32x2 wh = {h0, h1}, wl = {l0, l1};
+              const int off = rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8;
+              *(anc_u32x2 *)(b + off) = wh;
+              *(anc_u32x2 *)(b + 4096 + off) = wl;
+            }
+        } else {
+#pragma unroll
+          for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const uint32_t h0 = anc_pk_bf16(y[bj][4 * q], y[bj][4 * q + 1]);
+              const uint32_t h1 = anc_pk_bf16(y[bj][4 * q + 2], y[bj][4 * q + 3]);
+              const anc_u32x2 wh = {h0, h1};
+              *(anc_u32x2 *)(b + rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8) = wh;
+              const uint32_t q0 = anc_low8_encode(y[bj][4 * q], h0 << 16);
+              const uint32_t q1 = anc_low8_encode(y[bj][4 * q + 1], h0 & 0xFFFF0000u);
+              const uint32_t q2 = anc_low8_encode(y[bj][4 * q + 2], h1 << 16);
+              const uint32_t q3 = anc_low8_encode(y[bj][4 * q + 3], h1 & 0xFFFF0000u);
+              *(uint32_t *)(b + 4096 + bj * 1024 + rr * 32 + q * 8 + hh * 4) = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
+            }
+        }
         __builtin_amdgcn_s_waitcnt(0xC07F);
         __builtin_amdgcn_wave_barrier();
         // element offset of chunk c (8 columns) of slab row `row` in the output iterate
@@ -755,12 +821,21 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
           const anc_u32x4 qh = *(const anc_u32x4 *)(b + off);
           epi_st((anc_u32x4 *)(p.Yh + y_off(row, c)), qh);
         }
+        if (!out8) {
 #pragma unroll
-        for (int pz = 0; pz < 4; ++pz) {
-          const int idx = pz * 64 + lane, row = idx >> 3, c = idx & 7;
-          const int off = row * 128 + ((c ^ ((row & 7) ^ ((row >> 3) & 1))) * 16);
-          const anc_u32x4 ql = *(const anc_u32x4 *)(b + 4096 + off);
-          epi_st((anc_u32x4 *)(p.Yl + y_off(row, c)), ql);
+          for (int pz = 0; pz < 4; ++pz) {
+            const int idx = pz * 64 + lane, row = idx >> 3, c = idx & 7;
+            const int off = row * 128 + ((c ^ ((row & 7) ^ ((row >> 3) & 1))) * 16);
+            const anc_u32x4 ql = *(const anc_u32x4 *)(b + 4096 + off);
+            epi_st((anc_u32x4 *)(p.Yl + y_off(row, c)), ql);
+          }
+        } else {
+          // one byte per element: the slab's 32 rows of a panel are 1 KiB contiguous
+#pragma unroll
+          for (int pz = 0; pz < 2; ++pz) {
+            const anc_u32x4 ql = *(const anc_u32x4 *)(b + 4096 + pz * 1024 + lane * 16);
+            epi_st((anc_u32x4 *)((char *)p.Yl + mn * 2 + ((int64_t)(gj0w / 32 + pz) * M + gi0) * 32 + lane * 16), ql);
+          }
         }
       }
       // the buffer is free again once the staged rows have been read back
@@ -907,6 +982,10 @@ int launch_bx(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s, const N
     pm.g[k].tiles_m = ps[k].M / 128;
     pm.g[k].tiles_n = ps[k].N / 256;
     pm.g[k].lower = 0;
+    ANC_REQUIRE(!(ps[k].l8_in > 0.0) || (ps[k].x_panel && ps[k].Xl != nullptr),
+                "anc_ns_gemm_big: 8-bit low halves of the input need the panel layout");
+    ANC_REQUIRE(!(ps[k].l8_out > 0.0) || (ps[k].y_panel && ps[k].Yl != nullptr),
+                "anc_ns_gemm_big: 8-bit low halves of the output need the panel layout");
     // A matrix's tiles are walked in blocks of 4 x 2 tiles (512 rows of B, 512 columns of X) instead
     // of row by row: the 64 workgroups an XCD runs together then share 4 row blocks of B and a few
     // column blocks of X per matrix instead of all of X, and its L2 fetches X from HBM about once

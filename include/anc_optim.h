@@ -449,7 +449,9 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
  *   M < 1024          residuals of X, A, B from iteration 1 on (iteration 0 below M = 256); no gates.
  *   M >= 1024, N < 2M residual of X in A = X X^T and X = a X + B X of the last iteration.
  *   M >= 1024, N >= 2M  no residual term; B = b A + c A A takes the off-diagonal entries of A from the
- *                     bf16 copy it multiplies anyway (no fp32 copy of A: 3 .. 8 % of accuracy).
+ *                     bf16 copy it multiplies anyway (no fp32 copy of A: 3 .. 8 % of accuracy); with
+ *                     the 256-tile kernels the low half of the iterate is kept as 8 instead of 16
+ *                     bits wherever no product multiplies it (the iterate to 24 bits).
  * Gates (M >= 1024), per matrix, from statistics of the matrix alone, so that a result never
  * depends on the batch: after the first A = X X^T, proxy = N * ||offdiag(A)||_F^2 (1.0 for independent
  * entries whatever the row scaling, 1.7 for columns scaled over 0.1 .. 3, about N/r when the mass sits
@@ -486,12 +488,14 @@ int anc_quant_mxfp8_w(uint64_t w_bf16, uint64_t fp8_out, uint64_t scale_out, int
 #define ANC_NS_BF16_X3 3
 #define ANC_NS_BF16_LATE3 4
 /* Flag OR-ed into a bf16 mode: use the 128x128-tile GEMM kernel even where the 256x256-tile
- * kernel applies. The two produce the same bits wherever no product has residual terms
- * (ANC_NS_BF16_FAST; ANC_NS_BF16 on wide matrices that take no gate). Residual terms are added
- * in an order that depends on which elements of a symmetric product are computed and which are
- * mirrored, hence on the tile size: the results then differ in the last fp32 bits of A and B
- * (1e-6 .. 4e-4 of the result, largest on gated outlier-column inputs, inside the accuracy bar
- * either way). The flag exists so that tests can show both. */
+ * kernel applies. The two produce the same bits in ANC_NS_BF16_FAST (no residual terms). Residual
+ * terms are added in an order that depends on which elements of a symmetric product are computed
+ * and which are mirrored, hence on the tile size: the results then differ in the last fp32 bits
+ * of A and B (1e-6 .. 4e-4 of the result, largest on gated outlier-column inputs). ANC_NS_BF16 on
+ * N >= 2M keeps 8-bit low halves of the iterate with the 256-tile kernels only: the 24-bit iterate
+ * differs from the 32-bit pair by 2^-16 per element, which the chain turns into another
+ * realisation of its rounding error (the results are then 1.2e-3 apart, each inside the accuracy
+ * bar). The flag exists so that tests can show both. */
 #define ANC_NS_TILE128 0x100
 int64_t anc_ns_workspace_bytes(int64_t E, int64_t M, int64_t N, int mode);
 int anc_ns_batched(uint64_t X, int64_t E, int64_t M, int64_t N,

@@ -18,7 +18,9 @@ Rounding points modelled (same as the kernels):
   B = b A + c A A with A A = dA^2 + dA F + F dA + F F: only F F from bf16 operands (Fh Fh, plus
     Fh Fl + Fl Fh where needed); the entries of A in the fp32 terms are the fp32 F where the chain
     keeps the fp32 copy of A and Fh where it does not; diag(B) in fp32 (dB), Boff -> Bh (, Bl);
-  X' = (a + dB) (.) x + Boff X from bf16 operands: Bh Xh (+ Bh Xl) (+ Bl Xh).
+  X' = (a + dB) (.) x + Boff X from bf16 operands: Bh Xh (+ Bh Xl) (+ Bl Xh);
+  where the plan says so (N >= 2M) and no product of the next iteration multiplies it, the low half
+    Xl is kept as 8 bits relative to the ulp of Xh instead of a bf16.
 """
 import numpy as np
 
@@ -47,6 +49,7 @@ class Plan:
         self.wide_near_diff = 0.0    # > 0: the near range flags on proxy - colc > this instead of the ratio rule
         self.wide_from = 1
         self.drop_a32 = False
+        self.low8 = False            # low halves of the iterate as 8 bits where no product multiplies them
         if mode == "bf16_x3":
             self.x_from = self.fb_from = 0
             return
@@ -61,6 +64,7 @@ class Plan:
             return
         if M >= 1024:
             self.drop_a32 = mode == "bf16" and N >= 2 * M
+            self.low8 = self.drop_a32
             if steps >= 2:
                 self.wide, self.wide_near = True, (TAU_WIDE_NEAR if N < 2 * M else TAU_WIDE_LO)
                 if mode == "bf16" and N >= 2 * M:
@@ -113,6 +117,18 @@ def wide_flag(plan, proxy, colc, bulk):
             return proxy - colc > plan.wide_near_diff
         return colc < COLC_FRAC * proxy
     return False
+
+
+def low8(y, Xh):
+    """anc_low8_encode / _decode (csrc/ns_common.h): the low half of y next to Xh = bf16(y) as 8 bits
+    in the integer space of the fp32 bit patterns: d = bits(y) - bits(Xh) in -0x8000 .. 0x8000,
+    q = min(d + 0x80, 0x7FFF) >> 8, read back as the float with bits(Xh) + (q << 8) (y to 24 bits).
+    Returns that float minus Xh (exact in fp32)."""
+    yb, hb = np.ascontiguousarray(y, dtype=f32).view(np.uint32), np.ascontiguousarray(Xh, dtype=f32).view(np.uint32)
+    d = (yb - hb).astype(np.int32) + np.int32(0x80)
+    q = np.minimum(d, np.int32(0x7FFF)) >> 8
+    x = (hb + (q.astype(np.uint32) << np.uint32(8))).view(f32)
+    return (x - Xh).astype(f32)
 
 
 def chain(X, sched, steps=5, mode="bf16", eps=1e-7, info=None, overrides=None):
@@ -177,7 +193,14 @@ def chain(X, sched, steps=5, mode="bf16", eps=1e-7, info=None, overrides=None):
             Y = Y + bf16_round(Boff - Bh) @ Xh
         y = (a + dB)[:, None] * (Xh + Xl) + Y
         Xh = bf16_round(y)
-        Xl = bf16_round(y - Xh)
+        # 8-bit low half where no product of the next iteration multiplies it
+        nk = k + 1
+        if (plan.low8 and nk < steps and plan.gate_tau and not flagged and nk < plan.x_from
+                and not (nk in plan.gate_tau and proxy > plan.gate_tau[nk])
+                and not any(nk in ov.get(key, ()) for key in ("gram3", "bx_l"))):
+            Xl = low8(y, Xh)
+        else:
+            Xl = bf16_round(y - Xh)
     if info is not None:
         info.update(proxy=proxy, colc=colc, bulk=bulk, wide=flagged, plan=plan)
     return y

@@ -143,11 +143,21 @@ def test_batching_is_bitwise_neutral_and_repeatable(gpu):
 def test_tile_size_does_not_change_bits(gpu, M, N):
     """The 256x256-tile kernel and the 128x128-tile kernel accumulate every output element in the
     same order: identical bits without residual terms. With residual terms only the elements a
-    diagonal tile computes directly instead of mirroring can differ, in the last bits."""
+    diagonal tile computes directly instead of mirroring can differ, in the last bits. Where
+    N >= 2M the 256-tile chain keeps the iterate's low halves as 8 bits: a perturbation of 2^-17
+    per element, which the chain turns into another realisation of its own rounding error (the
+    numpy model of the chain: 7e-6 after iteration 1, 4e-4 after 2, 1.2e-3 at the end, the same
+    with an exact low half), so there both results are held to the bar instead of to each other."""
     rng = np.random.default_rng(M + 7 * N)
     X = rng.standard_normal((3, M, N)).astype(np.float32)
     assert bits_equal(run_ns(X, mode="bf16_fast"), run_ns(X, mode="bf16_fast_tile128"))
-    assert rel_fro(run_ns(X, mode="bf16"), run_ns(X, mode="bf16_tile128")) < 2e-4
+    big, small = run_ns(X, mode="bf16"), run_ns(X, mode="bf16_tile128")
+    if N < 2 * M or M < 1024:
+        assert rel_fro(big, small) < 2e-4
+    else:
+        for e in range(3):
+            want = host_ns(X[e], PE_SCHEDULE, 5)
+            assert rel_fro(big[e], want) < TOL_BF16 and rel_fro(small[e], want) < TOL_BF16
 
 
 @pytest.mark.parametrize("M,N", [(768, 1280), (1280, 2560), (1536, 1536), (2048, 2048), (2048, 4096), (4096, 4096)])
@@ -461,7 +471,11 @@ def test_low_rank_signal_over_weak_noise_is_told_from_outlier_columns(gpu, M, N)
     assert per[0] == per[2] > 2 * per[1] and per[3] == 0 and abs(sum(per) - extra) <= 1e-6 * extra
     if M == 1024:      # the 128x128-tile kernel reads the same flags
         small = run_ns(X[:2], mode="bf16_tile128")
-        assert rel_fro(small[0], got[0]) < 1e-4 and rel_fro(small[1], got[1]) < 5e-4
+        assert rel_fro(small[0], got[0]) < 1e-4
+        if N < 2 * M:
+            assert rel_fro(small[1], got[1]) < 5e-4
+        else:          # 8-bit low halves in the 256-tile chain: another realisation of the rounding error
+            assert rel_fro(small[1], host_ns(X[1], PE_SCHEDULE, 5)) < TOL_BF16
         assert _hard_count(2, M, N, "bf16_tile128")[0] == n_gated - 1
 
 

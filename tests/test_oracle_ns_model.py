@@ -57,6 +57,38 @@ def test_plan_mirrors_the_library():
                 assert ex.value == want, (M, N, mode, steps, p.x_from, p.fb_from)
 
 
+def test_low_half_as_eight_bits():
+    """The 8-bit low half of the iterate (csrc/ns_common.h anc_low8_encode / _decode, restated in
+    the model): high half + low half reproduce the value to 24 bits (2^-16 relative, 2^-15 where the
+    cap at 127 bites), without bias, exactly where the value has 16 significant bits, across binade
+    borders in both directions and for zeros; what comes back is exactly representable next to the
+    high half (the chain adds the two in fp32)."""
+    from oracle.ns_chain_model import low8
+    rng = np.random.default_rng(1)
+    y = (rng.standard_normal(1 << 20) * np.exp(rng.uniform(-30, 10, 1 << 20))).astype(np.float32)
+    special = np.array([0.0, -0.0, 1.0, -1.0, 2.0 - 2.0 ** -17, -(2.0 - 2.0 ** -17), 1.0 + 2.0 ** -9, 1.0 + 2.0 ** -8 + 2.0 ** -16,
+                        3.0 * 2.0 ** -100, 1.0078125 - 2.0 ** -23], np.float32)
+    y[:special.size] = special
+    h = bf16_round(y)
+    lo = low8(y, h)
+    x = (h + lo).astype(np.float32)
+    assert np.array_equal((x - h).astype(np.float32), lo)                   # exact next to the high half
+    err = (x.astype(np.float64) - y) / np.where(y == 0, 1.0, y)
+    assert np.abs(err).max() <= 2.0 ** -15 and np.percentile(np.abs(err), 99) <= 2.0 ** -16
+    assert abs(err.mean()) < 1e-7                                           # rounded, not truncated
+    nz = y != 0                                                             # (h + lo loses the sign of -0)
+    q = (x.view(np.uint32).astype(np.int64) - h.view(np.uint32).astype(np.int64))[nz] / 256
+    assert np.array_equal(q, np.rint(q)) and q.min() >= -128 and q.max() <= 127   # a whole byte
+    # values that sit k / 256 of a bf16 step next to a bf16 number, |k| <= 127, come back exactly
+    k = rng.integers(-127, 128, y.size).astype(np.int64)
+    hb = h.view(np.uint32).astype(np.int64)
+    ok = (hb & 0x7F800000 > 0x10000000) & (hb & 0x7F800000 < 0x7F000000)
+    exact = ((hb + (k << 8)) & 0xFFFFFFFF).astype(np.uint32).view(np.float32)[ok]
+    he = bf16_round(exact)
+    assert np.array_equal(he, h[ok]) and np.array_equal((he + low8(exact, he)).astype(np.float32), exact)
+    assert x[0] == 0 and x[2] == 1 and x[3] == -1
+
+
 @pytest.mark.parametrize("M,N", [(1024, 1024)])
 def test_low_gate_from_both_sides(M, N):
     """Scaled columns just below and just above the low gate (proxy 1.3, N < 2M)."""
