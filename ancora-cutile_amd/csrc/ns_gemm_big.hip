@@ -681,7 +681,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
               const uint32_t wl = (r & 2) ? xl[bj][r >> 2].y : xl[bj][r >> 2].x;
               const float x = ((r & 1) ? __uint_as_float(wh & 0xFFFF0000u) : __uint_as_float(wh << 16)) +
                               ((r & 1) ? __uint_as_float(wl & 0xFFFF0000u) : __uint_as_float(wl << 16));
-              y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
+              y[bj][r] = x;
             }
         } else {
           // 8-bit low halves: w8[bj][q] holds the 4 bytes of columns bj*32 + 8q + 4hh .. +3 of row
@@ -701,9 +701,22 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
             for (int r = 0; r < 16; ++r) {
               const uint32_t wh = (r & 2) ? xh[bj][r >> 2].y : xh[bj][r >> 2].x;
               const uint32_t htop = (r & 1) ? (wh & 0xFFFF0000u) : (wh << 16);
-              const float x = anc_low8_decode(htop, (int)(w8[bj][r >> 2] << (24 - 8 * (r & 3))) >> 24);
-              y[bj][r] = cf * (x * sc) + acc[bi][bj][r] * acc_scale;
+              y[bj][r] = anc_low8_decode(htop, (int)(w8[bj][r >> 2] << (24 - 8 * (r & 3))) >> 24);
             }
+        }
+        // y = (a + dB) x + B X; only the first iteration carries the input's scale (times 1.0f is the
+        // identity, so leaving the factors out elsewhere changes no bit; the fused instantiation,
+        // which has no register to spare for a second version, keeps them)
+        if (fused || p.scale != nullptr) {
+#pragma unroll
+          for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) y[bj][r] = cf * (y[bj][r] * sc) + acc[bi][bj][r] * acc_scale;
+        } else {
+#pragma unroll
+          for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) y[bj][r] = cf * y[bj][r] + acc[bi][bj][r];
         }
       }
       if (fp32_out || fused || plain) {
