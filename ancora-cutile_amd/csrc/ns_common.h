@@ -121,34 +121,38 @@ struct NsGemm {
 };
 
 
+// Per-matrix statistics and flags were written by earlier kernels and are the same for every lane:
+// read through the constant address space they come in by scalar loads, which neither occupy the
+// vector memory counter nor wait behind the kernel's own vector traffic.
+template <typename T> __device__ __forceinline__ T anc_ld_const(const T *p) {
+  return *(const __attribute__((address_space(4))) T *)(p);
+}
+
 // Number of accumulation terms of matrix e: p.nterms, or p.nterms_hard for a matrix that the
 // conditioning proxy marks as hard. The partial sums are added in a fixed order, so every
 // workgroup of every launch takes the same decision for a matrix.
-__device__ __forceinline__ double anc_ns_proxy(const NsGemm &p, int e) {
-  const double *c = p.cond + (int64_t)e * kCondParts;
-  double s = c[0];
+__device__ __forceinline__ double anc_cond_sum(const double *cond, int e) {
+  const double *c = cond + (int64_t)e * kCondParts;
+  double s = anc_ld_const(c);
 #pragma unroll
-  for (int i = 1; i < kCondParts; ++i) s = s + c[i];
+  for (int i = 1; i < kCondParts; ++i) s = s + anc_ld_const(c + i);
   return s;
 }
+__device__ __forceinline__ double anc_ns_proxy(const NsGemm &p, int e) { return anc_cond_sum(p.cond, e); }
 // Did the classification flag matrix e for the second gate?
 __device__ __forceinline__ bool anc_ns_wide(const NsGemm &p, int e) {
-  return p.wide_flag != nullptr && p.wide_flag[e] != 0;
+  return p.wide_flag != nullptr && anc_ld_const(p.wide_flag + e) != 0;
 }
 // Does matrix e keep the fp32 copy of A (GRAM writes it, BMAT reads it)?
 __device__ __forceinline__ bool anc_ns_has_a32(const NsGemm &p, int e) {
   if (p.A32 == nullptr) return false;
-  return p.a32_gated == 0 || (p.a32_flag != nullptr && p.a32_flag[e] != 0);
+  return p.a32_gated == 0 || (p.a32_flag != nullptr && anc_ld_const(p.a32_flag + e) != 0);
 }
 // Is the low half of matrix e's iterate one byte per element (thresh = p.l8_in or p.l8_out)?
 __device__ __forceinline__ bool anc_ns_low8(const NsGemm &p, int e, double thresh) {
   if (!(thresh > 0.0) || p.l8_cond == nullptr) return false;
-  if (p.l8_wide != nullptr && p.l8_wide[e] != 0) return false;
-  const double *c = p.l8_cond + (int64_t)e * kCondParts;
-  double s = c[0];
-#pragma unroll
-  for (int i = 1; i < kCondParts; ++i) s = s + c[i];
-  return !(s > thresh);
+  if (p.l8_wide != nullptr && anc_ld_const(p.l8_wide + e) != 0) return false;
+  return !(anc_cond_sum(p.l8_cond, e) > thresh);
 }
 // The 8-bit low half of y next to its high half h = bf16(y), in the integer space of the fp32 bit
 // patterns, where rounding to bf16 is rounding to a multiple of 0x10000: d = bits(y) - (h << 16) lies
@@ -180,7 +184,8 @@ constexpr int kMaxGroups = ANC_MAX_GROUPS;
 struct NsGemmMulti {
   int n;
   int seq;                   // plain product: 1 = anc_seq_tile dealing, 0 = anc_group_tile
-  int tiles[kMaxGroups];
+  int tiles[kMaxGroups];     // 0 past n
+  int seg_start[kXcds + 1];  // anc_group_tile: first logical tile of each XCD's segment (anc_fill_segments)
   NsGemm g[kMaxGroups];
   // fused weight update (problems with `upd` set): lr*shape_scale by descriptor scale index,
   // stochastic-rounding switch and seed, the step's control block (skip flag) or null
@@ -189,6 +194,15 @@ struct NsGemmMulti {
   uint32_t seed_base;
   const anc_step_ctl_t *ctl;
 };
+// Segment x holds the x-th eighth of every problem's tiles, problems in the order given.
+inline void anc_fill_segments(NsGemmMulti &pm) {
+  int at = 0;
+  for (int x = 0; x < kXcds; ++x) {
+    pm.seg_start[x] = at;
+    for (int k = 0; k < pm.n; ++k) at += pm.tiles[k] / kXcds + (x < pm.tiles[k] % kXcds ? 1 : 0);
+  }
+  pm.seg_start[kXcds] = at;
+}
 struct NsUpdate {
   float lr[ANC_MUON_MAX_SCALES];
   int sr;
@@ -206,17 +220,30 @@ __device__ __forceinline__ void anc_group_tile(const NsGemmMulti &pm, int bid, i
   g = 0;
   L = pos;
   if (pm.n == 1) return;
-  for (int x = 0; x < kXcds; ++x)
-    for (int k = 0; k < pm.n; ++k) {
-      const int T = pm.tiles[k], base = T / kXcds, rem = T % kXcds;
-      const int c = base + (x < rem ? 1 : 0);
-      if (pos < c) {
-        g = k;
-        L = x * base + (x < rem ? x : rem) + pos;
-        return;
-      }
-      pos -= c;
+  // the segment, from the starts the host summed up (anc_fill_segments); then the problem inside
+  // it: all in scalar registers, no memory access inside the loops
+  int T[kMaxGroups];
+#pragma unroll
+  for (int k = 0; k < kMaxGroups; ++k) T[k] = pm.tiles[k];          // (entries past pm.n are 0)
+  int x = 0, start = 0;
+#pragma unroll
+  for (int xx = 1; xx < kXcds; ++xx) {
+    const int st = pm.seg_start[xx];
+    if (pos >= st) { x = xx; start = st; }
+  }
+  pos -= start;
+  bool found = false;
+#pragma unroll
+  for (int k = 0; k < kMaxGroups; ++k) {
+    const int base = T[k] / kXcds, rem = T[k] % kXcds;
+    const int c = base + (x < rem ? 1 : 0);
+    if (!found && pos < c) {
+      found = true;
+      g = k;
+      L = x * base + (x < rem ? x : rem) + pos;
     }
+    if (!found) pos -= c;
+  }
 }
 
 // The other dealing: the problems' tile sequences one after the other, cut into 8 contiguous runs,

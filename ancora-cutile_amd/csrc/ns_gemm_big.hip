@@ -472,7 +472,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   const int gi0w = tm * TM + wm * 128, gj0w = tn * TN + wn * 64;
   const bool mirror = (EPI != EPI_BX) && (TN * (tn + 1) <= TM * tm);
   float sc = 1.0f;
-  if (EPI != EPI_BMAT && p.scale != nullptr) sc = p.scale[e];
+  if (EPI != EPI_BMAT && p.scale != nullptr) sc = anc_ld_const(p.scale + e);
   const float acc_scale = (EPI == EPI_GRAM) ? sc * sc : sc;
   // residual output (Fl of GRAM, Bl of BMAT): for every matrix, or only for those in the band of
   // the second conditioning gate (uniform over the workgroup: a function of the matrix)
@@ -976,6 +976,7 @@ int launch_sym(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s) {
     grid += t;
   }
   ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
+  anc_fill_segments(pm);
   hipLaunchKernelGGL((k_ns_gemm_big<EPI, 256, 256, 32, 4, 1>), dim3((unsigned)grid), dim3(512), 0, s, pm);
   ANC_LAUNCH_CHECK();
   return ANC_OK;
@@ -1017,6 +1018,7 @@ int launch_bx(const NsGemm *ps, const int64_t *Es, int n, hipStream_t s, const N
     grid += t;
   }
   ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big: grid out of range");
+  anc_fill_segments(pm);
   const bool fused = ps[0].upd != nullptr;
   if (fused) {
     for (int k = 0; k < ANC_MUON_MAX_SCALES; ++k) pm.lr[k] = upd->lr[k];
@@ -1100,6 +1102,7 @@ int anc_ns_gemm_big_plain(const NsGemm *ps, const int64_t *Es, int n, hipStream_
     grid += t;
   }
   ANC_REQUIRE(grid < (1ll << 31), "anc_ns_gemm_big_plain: grid out of range");
+  anc_fill_segments(pm);
   // Every XCD has an L2 of its own, so which tiles it runs decides how often an operand byte is
   // fetched from HBM. A launch that fits the GPU's 512 workgroup slots runs in one round: its
   // problems' tile sequences are dealt one after the other (anc_seq_tile), an XCD works on one or
