@@ -903,37 +903,71 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
       region = const_cast<unsigned char *>(b);
     }
     float ov[2][16];          // the values that leave as bf16 (pairs)
+    // Only a slab whose rows gi0 .. gi0+31 meet its columns gj0w .. gj0w+63 holds diagonal elements
+    // (the same for every lane of the wavefront): every other slab runs without the per-element test.
+    const bool slab_diag = gi0 + 31 >= gj0w && gi0 <= gj0w + 63;
+    if (EPI == EPI_GRAM && has_a32) {
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj) {
+      for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int gi = gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        const int gj = gj0w + bj * 32 + (lane & 31);
-        const float v = (EPI == EPI_BMAT) ? acc[bi][bj][r] : acc[bi][bj][r] * acc_scale;
-        if (EPI == EPI_GRAM) {
-          const bool diag = gi == gj;
-          if (has_a32) p.A32[mm + (int64_t)gi * M + gj] = v;
-          ov[bj][r] = diag ? 0.0f : v;
-          if (diag) p.dA[mv + gi] = v;
-        } else if (EPI == EPI_BMAT) {
-          const float a = in[bj][r];
-          const float di = drow[r], dj = dcol[bj];
-          if (gi != gj) {
-            const float a2 = v + (di * a + a * dj);   // symmetric in (i,j)
-            ov[bj][r] = p.cb * a + p.cc * a2;
+        for (int r = 0; r < 16; ++r) {
+          const int gi = gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          const int gj = gj0w + bj * 32 + (lane & 31);
+          p.A32[mm + (int64_t)gi * M + gj] = acc[bi][bj][r] * acc_scale;
+        }
+    }
+    if (!slab_diag) {
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (EPI == EPI_GRAM) {
+            ov[bj][r] = acc[bi][bj][r] * acc_scale;
           } else {
-            const float a2 = v + di * di;
-            p.dB[mv + gi] = p.cb * di + p.cc * a2;
-            ov[bj][r] = 0.0f;
+            const float v = acc[bi][bj][r], a = in[bj][r];
+            const float a2 = v + (drow[r] * a + a * dcol[bj]);   // symmetric in (i,j)
+            ov[bj][r] = p.cb * a + p.cc * a2;
+          }
+        }
+    } else {
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int gi = gi0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          const int gj = gj0w + bj * 32 + (lane & 31);
+          const float v = (EPI == EPI_BMAT) ? acc[bi][bj][r] : acc[bi][bj][r] * acc_scale;
+          if (EPI == EPI_GRAM) {
+            const bool diag = gi == gj;
+            ov[bj][r] = diag ? 0.0f : v;
+            if (diag) p.dA[mv + gi] = v;
+          } else if (EPI == EPI_BMAT) {
+            const float a = in[bj][r];
+            const float di = drow[r], dj = dcol[bj];
+            if (gi != gj) {
+              const float a2 = v + (di * a + a * dj);   // symmetric in (i,j)
+              ov[bj][r] = p.cb * a + p.cc * a2;
+            } else {
+              const float a2 = v + di * di;
+              p.dB[mv + gi] = p.cb * di + p.cc * a2;
+              ov[bj][r] = 0.0f;
+            }
           }
         }
       }
     }
     uint32_t hv[2][8], lv[2][8];
+    if (write_lo) {
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj)
+      for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) anc_pk_pair(ov[bj][2 * i], ov[bj][2 * i + 1], hv[bj][i], lv[bj][i]);
+        for (int i = 0; i < 8; ++i) anc_pk_pair(ov[bj][2 * i], ov[bj][2 * i + 1], hv[bj][i], lv[bj][i]);
+    } else {
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { hv[bj][i] = anc_pk_bf16(ov[bj][2 * i], ov[bj][2 * i + 1]); lv[bj][i] = 0u; }
+    }
     // Where the slab (rows gi0.., columns gj0w..) and its mirror image (rows gj0w.., columns gi0..:
     // 64 rows of one 32-column panel, a contiguous 4 KiB in panel layout) go in an (M, M) matrix.
     const bool f_pan = p.f_panel != 0;
