@@ -35,6 +35,11 @@ How each function is pinned (see tests/test_oracle_*.py):
   id_groups / embed_dw_rows /       (embed_ref.py) defining properties of the group arrays (permutation,
   embed_dw_scatter                  stability, counts), an exact integer case, the reference-held gate
                                     against an fp64 scatter-add (tests/kernels/test_embed_dw_scatter.py:55-61,91)
+ns_chain_model.py and ns_inputs.py are not restatements of the reference: the first models the
+arithmetic of this library's bf16 chain (rounding points, plan, gate statistics, the 8-bit low
+half), the second holds input families for walking its thresholds. The model is pinned to the GPU
+by tests/test_gpu_ns_model.py (errors against host_ns to three digits, gate decisions, two-step
+results to 2e-6); the parity target of every Newton-Schulz test stays host_ns.
 No function of the optimizer step is "parity unpinned". quant_mxfp8_w has three edge behaviours
 that no reference-held vector fixes (blocks with amax < 2**-120, bf16 subnormal inputs,
 non-finite inputs): they are parity unpinned and listed in the header of quant_ref.py.
