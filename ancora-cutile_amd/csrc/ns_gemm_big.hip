@@ -506,6 +506,10 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
   // (readfirstlane: the flags live in scalar registers, so the branches on them are scalar branches)
   const bool in8 = EPI == EPI_BX && !PLAINV && __builtin_amdgcn_readfirstlane((int)anc_ns_low8(p, e, p.l8_in)) != 0;
   const bool out8 = EPI == EPI_BX && !PLAINV && __builtin_amdgcn_readfirstlane((int)anc_ns_low8(p, e, p.l8_out)) != 0;
+  // In the buffer the two 16-byte halves of a row's 32 bytes are swapped for rows with bit 3 set:
+  // LDS chunk l holds row l/2, half (l%2) ^ ((l/16)%2), which halves the bank conflicts of the
+  // 4-byte accesses below (rows 8 apart would otherwise meet in one bank four at a time).
+  const int l8_src = (lane >> 1) * 32 + (((lane & 1) ^ ((lane >> 4) & 1)) * 16);
   auto fetch_in = [&](int bi) {
     const int64_t ub = x_pan ? mn * 2 + (int64_t)(gj0w / 32) * panel + (int64_t)(gi0w + bi * 32) * 64
                              : (mn + (int64_t)(gi0w + bi * 32) * N + gj0w) * 2;
@@ -520,7 +524,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
     if (in8) {
 #pragma unroll
       for (int j = 0; j < 2; ++j)
-        dma16_epi((const char *)p.Xl + mn * 2 + ((int64_t)(gj0w / 32 + j) * M + gi0w + bi * 32) * 32 + lane * 16,
+        dma16_epi((const char *)p.Xl + mn * 2 + ((int64_t)(gj0w / 32 + j) * M + gi0w + bi * 32) * 32 + l8_src,
                   lds_addr(b + 4096 + j * 1024));
     }
   };
@@ -693,7 +697,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               xh[bj][q] = *(const anc_u32x2 *)(b + rr * 128 + (((bj * 4 + q) ^ key) * 16) + hh * 8);
-              w8[bj][q] = *(const uint32_t *)(b + 4096 + bj * 1024 + rr * 32 + q * 8 + hh * 4);
+              w8[bj][q] = *(const uint32_t *)(b + 4096 + bj * 1024 + rr * 32 + (((q >> 1) ^ ((rr >> 3) & 1)) * 16) + (q & 1) * 8 + hh * 4);
             }
 #pragma unroll
           for (int bj = 0; bj < 2; ++bj)
@@ -816,7 +820,8 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
               const uint32_t q1 = anc_low8_encode(y[bj][4 * q + 1], h0 & 0xFFFF0000u);
               const uint32_t q2 = anc_low8_encode(y[bj][4 * q + 2], h1 << 16);
               const uint32_t q3 = anc_low8_encode(y[bj][4 * q + 3], h1 & 0xFFFF0000u);
-              *(uint32_t *)(b + 4096 + bj * 1024 + rr * 32 + q * 8 + hh * 4) = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
+              *(uint32_t *)(b + 4096 + bj * 1024 + rr * 32 + (((q >> 1) ^ ((rr >> 3) & 1)) * 16) + (q & 1) * 8 + hh * 4) =
+                  q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
             }
         }
         __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -847,7 +852,7 @@ __global__ void __launch_bounds__((TM / 128) * (TN / 64) * 64, MINBLOCKS) k_ns_g
 #pragma unroll
           for (int pz = 0; pz < 2; ++pz) {
             const anc_u32x4 ql = *(const anc_u32x4 *)(b + 4096 + pz * 1024 + lane * 16);
-            epi_st((anc_u32x4 *)((char *)p.Yl + mn * 2 + ((int64_t)(gj0w / 32 + pz) * M + gi0) * 32 + lane * 16), ql);
+            epi_st((anc_u32x4 *)((char *)p.Yl + mn * 2 + ((int64_t)(gj0w / 32 + pz) * M + gi0) * 32 + l8_src), ql);
           }
         }
       }
